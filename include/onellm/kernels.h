@@ -1,0 +1,54 @@
+// The six launcher functions of the decode hot path, with the signatures the oneLLM layers and
+// unit tests call.  Each is a thin shim over the C ABI in onellm_hip.h: it unpacks shapes the
+// way the reference launcher does and throws std::runtime_error on a non-zero return code.
+#pragma once
+#include "onellm/tensor.h"
+#include "onellm/base_weights.h"
+#include "onellm/norm_weights.h"
+#include "onellm/llama_params.h"
+
+// src/kernels/decoder_masked_attn.h:7-14
+void launchDecoderMaskedMHA(Tensor* qkv_buf,
+                            BaseWeight& qkv,
+                            Tensor* k_cache,
+                            Tensor* v_cache,
+                            Tensor* finished,
+                            Tensor* step,
+                            Tensor* mha_output,
+                            LLaMAAttentionStaticParams& static_params);
+
+// src/kernels/rmsnorm_kernel.h:6-9
+void launchRMSNorm(Tensor* decoder_out, LayerNormWeight& attn_norm_weight, float eps);
+
+// src/kernels/fused_addresidual_norm.h:4-12 (float as in the reference, half added)
+template<typename T>
+void launchFusedAddBiasResidualRMSNorm(T* residual,
+                                       T* decoder_out,
+                                       const T* bias,
+                                       const T* scale,
+                                       float eps,
+                                       int num_tokens,
+                                       int hidden_units);
+
+// src/kernels/append_to_kvcache.h:20-26
+void launchAppendKVCache(Tensor* k_src,
+                         Tensor* v_src,
+                         Tensor* layer_id,
+                         Tensor* cur_query_length,
+                         Tensor* history_length,
+                         Tensor* k_dst,
+                         Tensor* v_dst);
+
+// src/kernels/transpose_kernel.h:5-11
+void launchTransposeKVCache(Tensor* k_cache_src,
+                            Tensor* v_cache_src,
+                            Tensor* context_length,
+                            Tensor* layer_id,
+                            Tensor* k_cache_dst,
+                            Tensor* v_cache_dst);
+
+// src/kernels/beamsearch_topK.h:35-38
+void launchTopKforBeamSearch(const float* probs,
+                             const int batch_size,
+                             const int vocab_size,
+                             float* topk_workspace);

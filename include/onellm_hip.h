@@ -1,0 +1,154 @@
+/*
+ * onellm_hip.h — C ABI of the MI355X (gfx950) backend for oneLLM's per-token
+ * decode hot path.
+ *
+ * Every entry point takes raw device pointers, plain ints/floats and a stream
+ * handle, and returns an int: 0 on success, a positive hipError_t value when
+ * the HIP runtime reported an error, or a negative ONELLM_E* code when an
+ * argument is rejected before anything is launched.  Nothing here allocates
+ * or frees device memory and nothing synchronises the device; the caller owns
+ * all buffers.  `stream` is a hipStream_t passed as void* (NULL = the null
+ * stream) so that a binder needs no HIP header.
+ *
+ * Each function names the reference interface it stands in for (paths are
+ * relative to the oneLLM tree).
+ */
+#ifndef ONELLM_HIP_H
+#define ONELLM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of activations / KV cache; values equal the reference's
+ * `enum DataType` (src/utils/tensor.h:19-28): FP32 = 0, FP16 = 1. */
+#define ONELLM_FP32 0
+#define ONELLM_FP16 1
+
+/* argument-rejection codes (negative so they never collide with hipError_t) */
+#define ONELLM_EINVAL      (-1)  /* null pointer, non-positive size, bad enum  */
+#define ONELLM_EUNSUPPORTED (-2) /* shape outside what the kernels are built for */
+#define ONELLM_EWORKSPACE  (-3)  /* workspace missing or too small              */
+
+/* flags for onellm_decode_attn */
+#define ONELLM_ATTN_NO_V_BIAS     0x1u /* skip the v-bias add (reference decode kernel behaviour,
+                                          src/kernels/decoder_masked_attn.cu:257-258)            */
+#define ONELLM_ATTN_NO_CACHE_WRITE 0x2u /* do not store the new k/v row (read-only caches)        */
+
+typedef void* onellm_stream_t;
+
+/* Library/ABI version: major*1000 + minor. */
+int onellm_hip_version(void);
+
+/* Human-readable text for any code returned by this library.  Never NULL. */
+const char* onellm_error_string(int code);
+
+/*
+ * Fused masked decoder self-attention for ONE new token per sequence.
+ * Replaces launchDecoderMaskedMHA + masked_MHA_kernel
+ * (src/kernels/decoder_masked_attn.h:7-14, src/kernels/decoder_masked_attn.cu:136-327).
+ *
+ *   qkv        [B, Hq+2*Hkv, D]   fused projection output, q|k|v head-major per token
+ *   qkv_bias   [(Hq+2*Hkv)*D] or NULL (treated as zeros); q at h*D, k at Hq*D+kvh*D,
+ *              v at (Hq+Hkv)*D+kvh*D (src/kernels/qkv_bias_and_RoPE.cu:116,125,131)
+ *   k_cache,
+ *   v_cache    [num_layers, B, Hkv, S, D]; slab `layer` is used; rows 0..t-2 are history
+ *              and row t-1 is written by this call (roped+biased k, biased v)
+ *   out        [B, Hq*D]
+ *   t_host     number of attended positions (the reference's `step`,
+ *              decoder_masked_attn.cu:294) used for every sequence when t_dev == NULL
+ *   t_dev      optional device int32[B]: per-sequence t (1 <= t_dev[b] <= max_t)
+ *   max_t      upper bound of all t (<= S); sizes the sequence split.  With t_dev == NULL
+ *              pass t_host.
+ *   rotary_dim, rope_base   LLaMAAttentionStaticParams (src/models/llama/llama_params.h:2-7),
+ *              in the declared order; pairs (2i,2i+1) with 2i < rotary_dim are rotated by
+ *              angle = pos / base^(2i/rotary_dim), pos = t + rope_pos_offset
+ *              (offset 0 reproduces decoder_masked_attn.cu:186; -1 is the 0-based position
+ *              that the prefill kernel uses, qkv_bias_and_RoPE.cu:140)
+ *   workspace  device scratch of at least onellm_decode_attn_workspace_bytes() bytes, 256-byte
+ *              aligned; contents on entry are irrelevant and nothing is carried between calls
+ *
+ * Arithmetic is fp32 throughout; with ONELLM_FP16 the cache, qkv, bias and out are fp16 and the
+ * new k/v rows are rounded to fp16 before they take part in this step's scores.
+ * Supported shapes: D*sizeof(elt) a power of two in [16, 1024] bytes, Hq % Hkv == 0,
+ * Hq/Hkv <= 8, 1 <= t <= S.
+ */
+int onellm_decode_attn(int dtype,
+                       const void* qkv, const void* qkv_bias,
+                       void* k_cache, void* v_cache, void* out,
+                       int B, int Hq, int Hkv, int D, int S,
+                       int layer, int num_layers,
+                       int t_host, const int* t_dev, int max_t,
+                       int rotary_dim, float rope_base, int rope_pos_offset,
+                       unsigned flags,
+                       void* workspace, size_t workspace_bytes,
+                       onellm_stream_t stream);
+
+/* Bytes of workspace onellm_decode_attn needs for these sizes (0 never; at least 256). */
+size_t onellm_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int max_t);
+
+/*
+ * In-place RMSNorm over rows: x <- gamma * x * rsqrt(mean(x^2) + eps).
+ * Replaces launchRMSNorm + RMSNorm (src/kernels/rmsnorm_kernel.h:6-9,
+ * src/kernels/rmsnorm_kernel.cu:47-103).  x [N, H], gamma [H], both of `dtype`.
+ */
+int onellm_rmsnorm(int dtype, void* x, const void* gamma, float eps,
+                   int N, int H, onellm_stream_t stream);
+
+/*
+ * Fused add-bias-residual + RMSNorm.  Replaces launchFusedAddBiasResidualRMSNorm
+ * (src/kernels/fused_addresidual_norm.h:4-12, src/kernels/fused_addresidual_norm.cu:51-132):
+ *   r = out + residual + bias;  residual <- r;  out <- gamma * r * rsqrt(mean(r^2) + eps)
+ * residual, out [N, H]; bias [H] or NULL; gamma [H]; all of `dtype`.
+ */
+int onellm_fused_add_bias_residual_rmsnorm(int dtype, void* residual, void* out,
+                                           const void* bias, const void* gamma, float eps,
+                                           int N, int H, onellm_stream_t stream);
+
+/*
+ * KV-cache concat.  Replaces launchAppendKVCache (src/kernels/append_to_kvcache.h:20-26,
+ * src/kernels/append_to_kvcache.cu:8-114):
+ *   cache[layer, b, kvh, history_len[b] + tau, :] = src[b, kvh, tau, :]   for tau < cur_len[b]
+ * k_src, v_src [B, Hkv, max_q_len, D]; caches [num_layers, B, Hkv, S, D];
+ * cur_len, history_len device int32[B].  Rows that would land at or beyond S are dropped.
+ */
+int onellm_kv_append(int dtype, const void* k_src, const void* v_src,
+                     void* k_cache, void* v_cache,
+                     const int* cur_len, const int* history_len,
+                     int B, int Hkv, int max_q_len, int S, int D,
+                     int layer, int num_layers, onellm_stream_t stream);
+
+/*
+ * KV repeat (broadcast of KV heads to query heads).  Replaces launchTransposeKVCache
+ * (src/kernels/transpose_kernel.h:5-11, src/kernels/transpose_kernel.cu:7-88):
+ *   dst[b, h, s, :] = cache[layer, b, h / (Hq/Hkv), s, :]   for s < min(context_len[b], max_k_len)
+ * caches [num_layers, B, Hkv, S, D]; k_dst, v_dst [B, Hq, max_k_len, D];
+ * context_len device int32[B].  Rows at or beyond the length are left untouched.
+ */
+int onellm_kv_repeat(int dtype, const void* k_cache, const void* v_cache,
+                     void* k_dst, void* v_dst, const int* context_len,
+                     int B, int Hq, int Hkv, int S, int max_k_len, int D,
+                     int layer, int num_layers, onellm_stream_t stream);
+
+/*
+ * Beam-search top-K.  Replaces launchTopKforBeamSearch (src/kernels/beamsearch_topK.h:35-38,
+ * src/kernels/beamsearch_topK.cu:20-119).  logits [B*beam, V] fp32.
+ * Order: larger value first; equal values: smaller global flat index (row*V + token) first.
+ * Stage 1 keeps the K best of every (row, block) pair, stage 2 the K best of each batch entry.
+ * workspace (fp32 words), the reference's layout generalised:
+ *   vals[B*beam*nblk*K] | ids[B*beam*nblk*K] (int32) | final_vals[B*K] | final_ids[B*K] (int32)
+ * nblk = onellm_beam_topk_blocks_per_row(V) (8 for any V >= 2048, as in the reference).
+ * 1 <= K <= 8.  Slots with no candidate (V*beam < K) hold value -inf and id -1.
+ */
+int onellm_beam_topk(const float* logits, int B, int beam, int V, int K,
+                     float* workspace, onellm_stream_t stream);
+int onellm_beam_topk_blocks_per_row(int V);
+size_t onellm_beam_topk_workspace_bytes(int B, int beam, int V, int K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ONELLM_HIP_H */

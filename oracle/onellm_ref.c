@@ -1,0 +1,460 @@
+/*
+ * onellm_ref.c — CPU oracle for the decode hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file is the checker, never the product: only the test-suite, the smoke check and the
+ * benchmark's CPU-baseline leg may build, load or call it.  The HIP library does not link it
+ * and has no CPU fallback.
+ *
+ * It restates, in plain C, what the oneLLM decode-path kernels are meant to compute.  Each
+ * function cites the reference lines it follows (paths relative to the oneLLM tree).  Where the
+ * reference snapshot contradicts itself the choice made is written beside the citation.
+ *
+ * Numeric model (all functions): element-wise work (bias add, RoPE, exp, scale, gamma) is done
+ * in fp32 exactly as written; dot products and running sums are accumulated in double so that
+ * the oracle is the value the fp32 inputs define, not one particular summation order.  With
+ * dtype FP16 the buffers hold IEEE binary16 and every load widens / every store rounds once
+ * (round-to-nearest-even).
+ *
+ * The RoPE sine/cosine are NOT libm's: they are a fixed sequence of IEEE fp32 operations
+ * (3-term Cody-Waite reduction + degree-7/8 polynomials) so that a GPU kernel performing the
+ * same sequence produces the same bits; onellm_ref_sincosf is pinned against double-precision
+ * sin/cos in the test-suite.
+ *
+ * Parity status: every function below is pinned by known-answer tests taken from the reference's
+ * own unit tests and by independent float64 formulations (tests/test_oracle_*.py); none is
+ * "parity unpinned".  Tie order of the beam top-K is fixed by the task statement (lower index
+ * wins), not by a reference test.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <immintrin.h>
+
+#define REF_FP32 0
+#define REF_FP16 1
+
+#define REF_ATTN_NO_V_BIAS      0x1u
+#define REF_ATTN_NO_CACHE_WRITE 0x2u
+
+/* ---------------------------------------------------------------- fp16 <-> fp32 */
+
+static inline float h2f(uint16_t h) { return _cvtsh_ss(h); }
+static inline uint16_t f2h(float f) { return _cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC); }
+
+static inline float ld(const void* p, size_t i, int dtype)
+{
+    return dtype == REF_FP16 ? h2f(((const uint16_t*)p)[i]) : ((const float*)p)[i];
+}
+static inline void st(void* p, size_t i, int dtype, float v)
+{
+    if (dtype == REF_FP16) ((uint16_t*)p)[i] = f2h(v);
+    else ((float*)p)[i] = v;
+}
+/* value after one round trip through the storage type */
+static inline float rnd(float v, int dtype) { return dtype == REF_FP16 ? h2f(f2h(v)) : v; }
+
+static void ld_row(float* dst, const void* p, size_t off, int n, int dtype)
+{
+    if (dtype == REF_FP16) {
+        const uint16_t* s = (const uint16_t*)p + off;
+        int i = 0;
+        for (; i + 8 <= n; i += 8)
+            _mm256_storeu_ps(dst + i, _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)(s + i))));
+        for (; i < n; ++i) dst[i] = h2f(s[i]);
+    } else {
+        memcpy(dst, (const float*)p + off, (size_t)n * sizeof(float));
+    }
+}
+
+/* ---------------------------------------------------------------- deterministic sin/cos */
+
+/*
+ * sin and cos of an fp32 angle as a fixed sequence of fp32 IEEE operations.
+ * Reduction: j = rint(x * 2/pi); r = x - j*pi/2 with pi/2 split in three fp32 terms, each
+ * step one fused multiply-add.  Polynomials: the classic single-precision minimax pair on
+ * [-pi/4, pi/4].  Quadrant from j & 3.  Valid for |x| < ~1e5 (positions of any KV cache).
+ */
+void onellm_ref_sincosf(float x, float* s_out, float* c_out)
+{
+    const float TWO_OVER_PI = 0x1.45f306p-1f;
+    const float PIO2_HI = 0x1.921fb6p+0f;
+    const float PIO2_MID = -0x1.777a5cp-25f;
+    const float PIO2_LO = -0x1.0p-49f;
+    float j = rintf(x * TWO_OVER_PI);
+    float r = fmaf(-j, PIO2_HI, x);
+    r = fmaf(-j, PIO2_MID, r);
+    r = fmaf(-j, PIO2_LO, r);
+    float r2 = r * r;
+    float ps = fmaf(-1.9515295891e-4f, r2, 8.3321608736e-3f);
+    ps = fmaf(ps, r2, -1.6666654611e-1f);
+    float sr = fmaf(r * r2, ps, r);
+    float pc = fmaf(2.443315711809948e-5f, r2, -1.388731625493765e-3f);
+    pc = fmaf(pc, r2, 4.166664568298827e-2f);
+    float cr = fmaf(r2 * r2, pc, fmaf(-0.5f, r2, 1.0f));
+    int q = (int)j & 3;
+    float s = (q & 1) ? cr : sr;
+    float c = (q & 1) ? sr : cr;
+    if (q & 2) s = -s;
+    if ((q + 1) & 2) c = -c;
+    *s_out = s;
+    *c_out = c;
+}
+
+/*
+ * Rotation frequencies of RoPE: freq[i] = base^(2i/rotary_dim), 2i < min(rotary_dim, D), and the angle
+ * of pair i at position p is p / freq[i]  (src/kernels/decoder_masked_attn.cu:95-99 `GetRoPEfreq`:
+ * `t_step / powf(base, zid / (float)rot_embed_dim)` with zid = 2i;
+ * restated independently at tests/unittests/test_qkv_bias_and_rope.cu:56-66).
+ */
+void onellm_ref_rope_freqs(float* freq, int D, int rotary_dim, float base)
+{
+    /* rotary_dim may exceed D (the example drivers run rotary_dim 128 with D 8): the exponent
+       keeps rotary_dim in the denominator and only the pairs that exist are rotated. */
+    for (int i = 0; 2 * i < rotary_dim && 2 * i + 1 < D; ++i)
+        freq[i] = powf(base, (float)(2 * i) / (float)rotary_dim);
+}
+
+/*
+ * Rotate adjacent pairs (x[2i], x[2i+1]), 2i < rotary_dim, in place
+ * (src/kernels/decoder_masked_attn.cu:102-131 `GetRoPEres` / `apply_RoPE`):
+ *   x'[2i]   = cos*x[2i]   - sin*x[2i+1]
+ *   x'[2i+1] = cos*x[2i+1] + sin*x[2i]
+ * written as fma(x0, c, -(x1*s)) and fma(x1, c, x0*s) so the rounding sequence is fixed.
+ */
+void onellm_ref_rope_row(float* x, int D, int rotary_dim, const float* freq, int pos)
+{
+    for (int i = 0; 2 * i + 1 < D && 2 * i < rotary_dim; ++i) {
+        float ang = (float)pos / freq[i];
+        float s, c;
+        onellm_ref_sincosf(ang, &s, &c);
+        float x0 = x[2 * i], x1 = x[2 * i + 1];
+        x[2 * i]     = fmaf(x0, c, -(x1 * s));
+        x[2 * i + 1] = fmaf(x1, c, x0 * s);
+    }
+}
+
+/* ---------------------------------------------------------------- decode attention */
+
+/*
+ * One decode step of fused masked self-attention
+ * (src/kernels/decoder_masked_attn.cu:136-268 kernel, :280-327 launcher).
+ *
+ * Flow per (b, q-head h), kvh = h / (Hq/Hkv):
+ *   q = qkv[b, h] + bias[h*D..]                      (:175-180)
+ *   k = qkv[b, Hq+kvh] + bias[Hq*D + kvh*D..]        (:181-185)
+ *   v = qkv[b, Hq+Hkv+kvh] + bias[(Hq+Hkv)*D+kvh*D..]  (v bias as the prefill kernel adds it,
+ *        src/kernels/qkv_bias_and_RoPE.cu:130-134; the decode kernel as written skips it,
+ *        :257-258 — flag REF_ATTN_NO_V_BIAS reproduces that)
+ *   RoPE(q), RoPE(k) at position pos = t + rope_pos_offset   (:186 uses `step`, i.e. offset 0)
+ *   cache row t-1 <- k, v (rounded to the storage type)      (:208-214, :255-259)
+ *   s_j = (q . K_j) / sqrt(D), j < t                          (:218-224, scale :301)
+ *   p = softmax(s) with the true row maximum                  (:228-244; the kernel as written
+ *        is only valid for t <= D — not reproduced)
+ *   out[b, h*D + d] = sum_j p_j V_j[d]                        (:247-267)
+ *
+ * Layout choices where the snapshot disagrees with itself: the fused buffer has batch stride
+ * (Hq+2Hkv)*D (:296-299 slices one [B, Hq+2Hkv, D] buffer); the cache is
+ * [num_layers, B, Hkv, S, D] as the layer allocates it (examples/cpp/decoder/self_decoder_example.cpp:186-187)
+ * and as the concat kernel writes it (src/kernels/append_to_kvcache.cu:32-34); GQA maps q-head h
+ * to kv-head h/G as the repeat kernel does (src/kernels/transpose_kernel.cu:32).
+ *
+ * t_arr (host int[B]) gives a per-sequence t; NULL means t_host for all.
+ */
+int onellm_ref_decode_attn(int dtype, const void* qkv, const void* qkv_bias,
+                           void* k_cache, void* v_cache, void* out,
+                           int B, int Hq, int Hkv, int D, int S, int layer, int num_layers,
+                           int t_host, const int* t_arr,
+                           int rotary_dim, float rope_base, int rope_pos_offset, unsigned flags)
+{
+    if (!qkv || !k_cache || !v_cache || !out || B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || S <= 0) return -1;
+    if (Hq % Hkv || layer < 0 || layer >= num_layers) return -1;
+    const int G = Hq / Hkv;
+    const int QKVH = Hq + 2 * Hkv;
+    const float scale = 1.0f / sqrtf((float)D);
+    float* freq = (float*)malloc(sizeof(float) * (size_t)(D / 2 + 1));
+    onellm_ref_rope_freqs(freq, D, rotary_dim, rope_base);
+    const size_t slab = (size_t)layer * B * Hkv * S * D;
+    int bad = 0;
+
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int b = 0; b < B; ++b) {
+        for (int kvh = 0; kvh < Hkv; ++kvh) {
+            const int t = t_arr ? t_arr[b] : t_host;
+            if (t < 1 || t > S) {
+#pragma omp atomic write
+                bad = 1;
+                continue;
+            }
+            const int pos = t + rope_pos_offset;
+            float* kn = (float*)malloc(sizeof(float) * (size_t)D * 4);
+            float* vn = kn + D;
+            float* q = vn + D;
+            float* row = q + D;
+            float* sc = (float*)malloc(sizeof(float) * (size_t)t);
+            double* acc = (double*)malloc(sizeof(double) * (size_t)D);
+            const size_t tok = (size_t)b * QKVH * D;
+            /* new k / v rows */
+            for (int d = 0; d < D; ++d) {
+                float kb = qkv_bias ? ld(qkv_bias, (size_t)(Hq + kvh) * D + d, dtype) : 0.0f;
+                float vb = (qkv_bias && !(flags & REF_ATTN_NO_V_BIAS)) ? ld(qkv_bias, (size_t)(Hq + Hkv + kvh) * D + d, dtype) : 0.0f;
+                kn[d] = ld(qkv, tok + (size_t)(Hq + kvh) * D + d, dtype) + kb;
+                vn[d] = ld(qkv, tok + (size_t)(Hq + Hkv + kvh) * D + d, dtype) + vb;
+            }
+            onellm_ref_rope_row(kn, D, rotary_dim, freq, pos);
+            for (int d = 0; d < D; ++d) {
+                kn[d] = rnd(kn[d], dtype);
+                vn[d] = rnd(vn[d], dtype);
+            }
+            const size_t base = slab + ((size_t)b * Hkv + kvh) * (size_t)S * D;
+            if (!(flags & REF_ATTN_NO_CACHE_WRITE)) {
+                for (int d = 0; d < D; ++d) {
+                    st(k_cache, base + (size_t)(t - 1) * D + d, dtype, kn[d]);
+                    st(v_cache, base + (size_t)(t - 1) * D + d, dtype, vn[d]);
+                }
+            }
+            for (int g = 0; g < G; ++g) {
+                const int h = kvh * G + g;
+                for (int d = 0; d < D; ++d) {
+                    float qb = qkv_bias ? ld(qkv_bias, (size_t)h * D + d, dtype) : 0.0f;
+                    q[d] = ld(qkv, tok + (size_t)h * D + d, dtype) + qb;
+                }
+                onellm_ref_rope_row(q, D, rotary_dim, freq, pos);
+                float smax = -INFINITY;
+                for (int j = 0; j < t; ++j) {
+                    const float* kr;
+                    if (j == t - 1) kr = kn;
+                    else { ld_row(row, k_cache, base + (size_t)j * D, D, dtype); kr = row; }
+                    double a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+                    int d = 0;
+                    for (; d + 4 <= D; d += 4) {
+                        a0 += (double)q[d] * kr[d];
+                        a1 += (double)q[d + 1] * kr[d + 1];
+                        a2 += (double)q[d + 2] * kr[d + 2];
+                        a3 += (double)q[d + 3] * kr[d + 3];
+                    }
+                    for (; d < D; ++d) a0 += (double)q[d] * kr[d];
+                    sc[j] = (float)((a0 + a1) + (a2 + a3)) * scale;
+                    if (sc[j] > smax) smax = sc[j];
+                }
+                double denom = 0;
+                for (int d = 0; d < D; ++d) acc[d] = 0;
+                for (int j = 0; j < t; ++j) {
+                    const float p = expf(sc[j] - smax);
+                    denom += p;
+                    const float* vr;
+                    if (j == t - 1) vr = vn;
+                    else { ld_row(row, v_cache, base + (size_t)j * D, D, dtype); vr = row; }
+                    for (int d = 0; d < D; ++d) acc[d] += (double)p * vr[d];
+                }
+                for (int d = 0; d < D; ++d)
+                    st(out, (size_t)b * Hq * D + (size_t)h * D + d, dtype, (float)(acc[d] / denom));
+            }
+            free(acc);
+            free(sc);
+            free(kn);
+        }
+    }
+    free(freq);
+    return bad ? -1 : 0;
+}
+
+/* ---------------------------------------------------------------- norms */
+
+/*
+ * In-place RMSNorm (src/kernels/rmsnorm_kernel.cu:47-83): per row
+ *   inv = rsqrt(sum(x^2)/H + eps)   (:61-72)      x <- gamma * x * inv   (:76-82)
+ * The multiplication order gamma*x then *inv follows :78-81.
+ */
+int onellm_ref_rmsnorm(int dtype, void* x, const void* gamma, float eps, int N, int H)
+{
+    if (!x || !gamma || N < 0 || H <= 0) return -1;
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; ++n) {
+        const size_t o = (size_t)n * H;
+        double ss = 0;
+        for (int i = 0; i < H; ++i) {
+            float v = ld(x, o + i, dtype);
+            ss += (double)v * v;
+        }
+        const float inv = (float)(1.0 / sqrt(ss / H + (double)eps));
+        for (int i = 0; i < H; ++i)
+            st(x, o + i, dtype, ld(gamma, i, dtype) * ld(x, o + i, dtype) * inv);
+    }
+    return 0;
+}
+
+/*
+ * Fused add-bias-residual-RMSNorm (src/kernels/fused_addresidual_norm.cu:51-107).
+ * Intended semantics (what the calling layer relies on, src/layers/decoder/self_decoder.cpp:49-56
+ * "decoder_output += decoder_input", and what the kernel's first loop computes, :78-82):
+ *   r = out + residual + bias;  residual <- r (rounded to storage);
+ *   out <- gamma * r * rsqrt(mean(r^2) + eps), r taken un-rounded.
+ * as_written != 0 reproduces the snapshot instead (:99-105): the sum is used only for the
+ * mean, `out` is scaled from its un-added value and residual is left alone.
+ */
+int onellm_ref_fused_add_bias_residual_rmsnorm(int dtype, void* residual, void* out,
+                                               const void* bias, const void* gamma, float eps,
+                                               int N, int H, int as_written)
+{
+    if (!residual || !out || !gamma || N < 0 || H <= 0) return -1;
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; ++n) {
+        const size_t o = (size_t)n * H;
+        float* r = (float*)malloc(sizeof(float) * (size_t)H);
+        double ss = 0;
+        for (int i = 0; i < H; ++i) {
+            float b = bias ? ld(bias, i, dtype) : 0.0f;
+            r[i] = ld(out, o + i, dtype) + ld(residual, o + i, dtype) + b;
+            ss += (double)r[i] * r[i];
+        }
+        const float inv = (float)(1.0 / sqrt(ss / H + (double)eps));
+        for (int i = 0; i < H; ++i) {
+            if (as_written) {
+                st(out, o + i, dtype, ld(gamma, i, dtype) * ld(out, o + i, dtype) * inv);
+            } else {
+                st(residual, o + i, dtype, r[i]);
+                st(out, o + i, dtype, ld(gamma, i, dtype) * r[i] * inv);
+            }
+        }
+        free(r);
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------- KV cache concat / repeat */
+
+static size_t esize(int dtype) { return dtype == REF_FP16 ? 2 : 4; }
+
+/*
+ * KV concat (src/kernels/append_to_kvcache.cu:27-36 index math, :81-87 shapes):
+ *   cache[layer, b, kvh, history[b]+tau, :] = src[b, kvh, tau, :]   for tau < cur_len[b]
+ * The layer slab offset is the one the launcher comment gives (:75) and hard-codes to 0 (:87).
+ * Rows that would fall outside [0, S) are dropped (the reference has no guard).
+ */
+int onellm_ref_kv_append(int dtype, const void* k_src, const void* v_src, void* k_cache, void* v_cache,
+                         const int* cur_len, const int* history_len,
+                         int B, int Hkv, int max_q_len, int S, int D, int layer, int num_layers)
+{
+    if (!k_src || !v_src || !k_cache || !v_cache || !cur_len || !history_len) return -1;
+    if (B <= 0 || Hkv <= 0 || max_q_len <= 0 || S <= 0 || D <= 0 || layer < 0 || layer >= num_layers) return -1;
+    const size_t e = esize(dtype), rowb = (size_t)D * e;
+    const size_t slab = (size_t)layer * B * Hkv * S * D;
+    for (int b = 0; b < B; ++b)
+        for (int h = 0; h < Hkv; ++h)
+            for (int tau = 0; tau < max_q_len && tau < cur_len[b]; ++tau) {
+                const long drow = (long)history_len[b] + tau;
+                if (drow < 0 || drow >= S) continue;
+                const size_t so = (((size_t)b * Hkv + h) * max_q_len + tau) * D;
+                const size_t d_o = slab + (((size_t)b * Hkv + h) * S + (size_t)drow) * D;
+                memcpy((char*)k_cache + d_o * e, (const char*)k_src + so * e, rowb);
+                memcpy((char*)v_cache + d_o * e, (const char*)v_src + so * e, rowb);
+            }
+    return 0;
+}
+
+/*
+ * KV repeat for grouped-query heads (src/kernels/transpose_kernel.cu:30-41 index math,
+ * :53-62 shapes):  dst[b, h, s, :] = cache[layer, b, h/G, s, :]  for s < context_len[b];
+ * dst is [B, Hq, max_k_len, D]; rows >= length are not written.  Lengths above max_k_len are
+ * clipped (the reference grid simply has no threads there, :65).
+ */
+int onellm_ref_kv_repeat(int dtype, const void* k_cache, const void* v_cache, void* k_dst, void* v_dst,
+                         const int* context_len, int B, int Hq, int Hkv, int S, int max_k_len, int D,
+                         int layer, int num_layers)
+{
+    if (!k_cache || !v_cache || !k_dst || !v_dst || !context_len) return -1;
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || S <= 0 || max_k_len <= 0 || D <= 0) return -1;
+    if (layer < 0 || layer >= num_layers) return -1;
+    const int G = Hq / Hkv;
+    const size_t e = esize(dtype), rowb = (size_t)D * e;
+    const size_t slab = (size_t)layer * B * Hkv * S * D;
+    for (int b = 0; b < B; ++b) {
+        int len = context_len[b];
+        if (len > max_k_len) len = max_k_len;
+        if (len > S) len = S;
+        for (int h = 0; h < Hq; ++h)
+            for (int s = 0; s < len; ++s) {
+                const size_t so = slab + (((size_t)b * Hkv + h / G) * S + s) * D;
+                const size_t d_o = (((size_t)b * Hq + h) * max_k_len + s) * D;
+                memcpy((char*)k_dst + d_o * e, (const char*)k_cache + so * e, rowb);
+                memcpy((char*)v_dst + d_o * e, (const char*)v_cache + so * e, rowb);
+            }
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------- beam-search top-K */
+
+/* candidate order: larger value first, then smaller id (global flat index) */
+static inline int better(float v1, int i1, float v2, int i2)
+{
+    return v1 > v2 || (v1 == v2 && (unsigned)i1 < (unsigned)i2);
+}
+
+/*
+ * Sorted-K insertion list (src/kernels/beamsearch_topK.h:3-33 `topK<K>::insertHeap`): the
+ * candidate replaces the last slot when it is better, then one bubble pass restores order.
+ * Unlike the reference's strict `>` on values alone (:16-31), the comparison is the total
+ * order above, so the result does not depend on insertion order.  Empty slots are id -1.
+ */
+static void topk_insert(float* val, int* id, int K, float v, int i)
+{
+    if (id[K - 1] != -1 && !better(v, i, val[K - 1], id[K - 1])) return;
+    val[K - 1] = v;
+    id[K - 1] = i;
+    for (int s = K - 2; s >= 0; --s) {
+        if (id[s] == -1 || better(val[s + 1], id[s + 1], val[s], id[s])) {
+            float tv = val[s]; val[s] = val[s + 1]; val[s + 1] = tv;
+            int ti = id[s]; id[s] = id[s + 1]; id[s + 1] = ti;
+        } else break;
+    }
+}
+
+/*
+ * Two-round beam top-K (src/kernels/beamsearch_topK.cu:20-52 round 1, :57-83 round 2,
+ * :85-119 launcher and workspace plan).
+ * Round 1: row r = [b, beam] is scanned by nblk blocks of 256 lanes; block `lane` owns tokens
+ *   tid + lane*256 + m*nblk*256 (:35); candidate id = global flat index r*V + token (:36-38);
+ *   output [B*beam, nblk, K] (:45-49).
+ * Round 2: the beam*nblk*K candidates of each batch entry are merged into [B, K] (:70-81).
+ * Workspace (fp32 words): vals | ids | final_vals | final_ids (:92-99).
+ * Empty slots: value -inf, id -1.
+ */
+int onellm_ref_beam_topk(const float* logits, int B, int beam, int V, int K, int nblk, float* workspace)
+{
+    if (!logits || !workspace || B <= 0 || beam <= 0 || V <= 0 || K <= 0 || K > 64 || nblk <= 0) return -1;
+    const size_t n1 = (size_t)B * beam * nblk * K;
+    float* vals = workspace;
+    int* ids = (int*)(vals + n1);
+    float* fvals = (float*)(ids + n1);
+    int* fids = (int*)(fvals + (size_t)B * K);
+    const int rows = B * beam;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int r = 0; r < rows; ++r)
+        for (int lane = 0; lane < nblk; ++lane) {
+            float v[64]; int id[64];
+            for (int k = 0; k < K; ++k) { v[k] = -INFINITY; id[k] = -1; }
+            for (int base = lane * 256; base < V; base += nblk * 256)
+                for (int tok = base; tok < base + 256 && tok < V; ++tok)
+                    topk_insert(v, id, K, logits[(size_t)r * V + tok], r * V + tok);
+            for (int k = 0; k < K; ++k) {
+                vals[((size_t)r * nblk + lane) * K + k] = v[k];
+                ids[((size_t)r * nblk + lane) * K + k] = id[k];
+            }
+        }
+    for (int b = 0; b < B; ++b) {
+        float v[64]; int id[64];
+        for (int k = 0; k < K; ++k) { v[k] = -INFINITY; id[k] = -1; }
+        const size_t n = (size_t)beam * nblk * K;
+        for (size_t i = 0; i < n; ++i) {
+            const int cid = ids[(size_t)b * n + i];
+            if (cid != -1) topk_insert(v, id, K, vals[(size_t)b * n + i], cid);
+        }
+        for (int k = 0; k < K; ++k) {
+            fvals[(size_t)b * K + k] = v[k];
+            fids[(size_t)b * K + k] = id[k];
+        }
+    }
+    return 0;
+}

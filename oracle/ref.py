@@ -1,0 +1,174 @@
+"""ctypes binding of the CPU oracle (oracle/libonellm_ref.so).  TEST INFRASTRUCTURE ONLY.
+
+Only the test-suite, the smoke check and the benchmark's CPU-baseline leg import this module;
+the product package never does.  Every function works on numpy arrays in place, exactly as the
+C functions do, and raises on a non-zero return code.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libonellm_ref.so")
+
+FP32, FP16 = 0, 1
+ATTN_NO_V_BIAS = 0x1
+ATTN_NO_CACHE_WRITE = 0x2
+
+
+def build(force=False):
+    """Compile the oracle with gcc (a few hundred ms)."""
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(
+            os.path.join(_HERE, "onellm_ref.c")):
+        subprocess.run(["make", "-C", _HERE, "-B", "libonellm_ref.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        vp, ci, cf, cu = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_uint
+        L.onellm_ref_sincosf.argtypes = [cf, ctypes.POINTER(cf), ctypes.POINTER(cf)]
+        L.onellm_ref_sincosf.restype = None
+        L.onellm_ref_rope_freqs.argtypes = [vp, ci, ci, cf]
+        L.onellm_ref_rope_freqs.restype = None
+        L.onellm_ref_rope_row.argtypes = [vp, ci, ci, vp, ci]
+        L.onellm_ref_rope_row.restype = None
+        L.onellm_ref_decode_attn.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, ci, cf, ci, cu]
+        L.onellm_ref_rmsnorm.argtypes = [ci, vp, vp, cf, ci, ci]
+        L.onellm_ref_fused_add_bias_residual_rmsnorm.argtypes = [ci, vp, vp, vp, vp, cf, ci, ci, ci]
+        L.onellm_ref_kv_append.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci]
+        L.onellm_ref_kv_repeat.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci]
+        L.onellm_ref_beam_topk.argtypes = [vp, ci, ci, ci, ci, ci, vp]
+        _lib = L
+    return _lib
+
+
+def _dt(a):
+    if a.dtype == np.float32:
+        return FP32
+    if a.dtype == np.float16:
+        return FP16
+    raise TypeError(f"unsupported dtype {a.dtype}")
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"], "oracle needs C-contiguous arrays"
+    return a.ctypes.data
+
+
+def _chk(rc, name):
+    if rc != 0:
+        raise RuntimeError(f"oracle {name} rejected its arguments (rc={rc})")
+
+
+def sincosf(x):
+    s, c = ctypes.c_float(), ctypes.c_float()
+    lib().onellm_ref_sincosf(ctypes.c_float(x), ctypes.byref(s), ctypes.byref(c))
+    return s.value, c.value
+
+
+def sincosf_array(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    s = np.empty_like(x)
+    c = np.empty_like(x)
+    L = lib()
+    cs, cc = ctypes.c_float(), ctypes.c_float()
+    for i, v in enumerate(x.ravel()):
+        L.onellm_ref_sincosf(ctypes.c_float(float(v)), ctypes.byref(cs), ctypes.byref(cc))
+        s.ravel()[i] = cs.value
+        c.ravel()[i] = cc.value
+    return s, c
+
+
+def rope_freqs(rotary_dim, base, D=None):
+    D = rotary_dim if D is None else D
+    f = np.zeros(D // 2 + 1, dtype=np.float32)
+    lib().onellm_ref_rope_freqs(_p(f), D, rotary_dim, base)
+    return f[: min(rotary_dim, D) // 2]
+
+
+def rope_row(x, rotary_dim, base, pos):
+    """Rotate one fp32 row in place."""
+    assert x.dtype == np.float32 and x.ndim == 1
+    f = np.zeros(x.shape[0] // 2 + 1, dtype=np.float32)
+    lib().onellm_ref_rope_freqs(_p(f), x.shape[0], rotary_dim, base)
+    lib().onellm_ref_rope_row(_p(x), x.shape[0], rotary_dim, _p(f), pos)
+    return x
+
+
+def decode_attn(qkv, bias, k_cache, v_cache, Hq, t, rotary_dim, rope_base, layer=0,
+                rope_pos_offset=0, flags=0):
+    """qkv [B, Hq+2Hkv, D]; caches [L, B, Hkv, S, D] (modified in place); t int or int array [B].
+    Returns out [B, Hq*D]."""
+    B, QKVH, D = qkv.shape
+    L, Bc, Hkv, S, Dc = k_cache.shape
+    assert Bc == B and Dc == D and QKVH == Hq + 2 * Hkv and v_cache.shape == k_cache.shape
+    assert k_cache.dtype == qkv.dtype == v_cache.dtype
+    out = np.zeros((B, Hq * D), dtype=qkv.dtype)
+    if np.isscalar(t) or isinstance(t, (int, np.integer)):
+        t_host, t_arr = int(t), None
+    else:
+        t_arr = np.ascontiguousarray(t, dtype=np.int32)
+        t_host = int(t_arr.max())
+    rc = lib().onellm_ref_decode_attn(_dt(qkv), _p(qkv), _p(bias), _p(k_cache), _p(v_cache), _p(out),
+                                      B, Hq, Hkv, D, S, layer, L, t_host, _p(t_arr),
+                                      rotary_dim, rope_base, rope_pos_offset, flags)
+    _chk(rc, "decode_attn")
+    return out
+
+
+def rmsnorm(x, gamma, eps):
+    N, H = x.shape
+    assert gamma.dtype == x.dtype
+    _chk(lib().onellm_ref_rmsnorm(_dt(x), _p(x), _p(gamma), eps, N, H), "rmsnorm")
+    return x
+
+
+def fused_add_bias_residual_rmsnorm(residual, out, bias, gamma, eps, as_written=False):
+    N, H = out.shape
+    assert residual.shape == out.shape and residual.dtype == out.dtype == gamma.dtype
+    _chk(lib().onellm_ref_fused_add_bias_residual_rmsnorm(_dt(out), _p(residual), _p(out), _p(bias), _p(gamma),
+                                                          eps, N, H, int(as_written)), "fused_norm")
+    return residual, out
+
+
+def kv_append(k_src, v_src, k_cache, v_cache, cur_len, history_len, layer=0):
+    B, Hkv, max_q_len, D = k_src.shape
+    L, _, _, S, _ = k_cache.shape
+    cur_len = np.ascontiguousarray(cur_len, dtype=np.int32)
+    history_len = np.ascontiguousarray(history_len, dtype=np.int32)
+    _chk(lib().onellm_ref_kv_append(_dt(k_src), _p(k_src), _p(v_src), _p(k_cache), _p(v_cache), _p(cur_len),
+                                    _p(history_len), B, Hkv, max_q_len, S, D, layer, L), "kv_append")
+
+
+def kv_repeat(k_cache, v_cache, k_dst, v_dst, context_len, layer=0):
+    L, B, Hkv, S, D = k_cache.shape
+    _, Hq, max_k_len, _ = k_dst.shape
+    context_len = np.ascontiguousarray(context_len, dtype=np.int32)
+    _chk(lib().onellm_ref_kv_repeat(_dt(k_cache), _p(k_cache), _p(v_cache), _p(k_dst), _p(v_dst), _p(context_len),
+                                    B, Hq, Hkv, S, max_k_len, D, layer, L), "kv_repeat")
+
+
+def beam_topk(logits, B, beam, K, nblk=8):
+    """Returns (round1_vals [B*beam,nblk,K], round1_ids, final_vals [B,K], final_ids [B,K])."""
+    rows, V = logits.shape
+    assert rows == B * beam and logits.dtype == np.float32
+    n1 = B * beam * nblk * K
+    ws = np.zeros(2 * n1 + 2 * B * K, dtype=np.float32)
+    _chk(lib().onellm_ref_beam_topk(_p(logits), B, beam, V, K, nblk, _p(ws)), "beam_topk")
+    vals = ws[:n1].reshape(B * beam, nblk, K).copy()
+    ids = ws[n1:2 * n1].view(np.int32).reshape(B * beam, nblk, K).copy()
+    fv = ws[2 * n1:2 * n1 + B * K].reshape(B, K).copy()
+    fi = ws[2 * n1 + B * K:].view(np.int32).reshape(B, K).copy()
+    return vals, ids, fv, fi
