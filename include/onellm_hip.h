@@ -73,8 +73,8 @@ const char* onellm_error_string(int code);
  *
  * Arithmetic is fp32 throughout; with ONELLM_FP16 the cache, qkv, bias and out are fp16 and the
  * new k/v rows are rounded to fp16 before they take part in this step's scores.
- * Supported shapes: D*sizeof(elt) a power of two in [16, 1024] bytes, Hq % Hkv == 0,
- * Hq/Hkv <= 8, 1 <= t <= S.
+ * Supported shapes: D*sizeof(elt) a power of two in [16, 1024] bytes, Hq % Hkv == 0, 1 <= t <= S,
+ * caches 16-byte aligned.
  */
 int onellm_decode_attn(int dtype,
                        const void* qkv, const void* qkv_bias,
@@ -140,13 +140,15 @@ int onellm_kv_repeat(int dtype, const void* k_cache, const void* v_cache,
  * Stage 1 keeps the K best of every (row, block) pair, stage 2 the K best of each batch entry.
  * workspace (fp32 words), the reference's layout generalised:
  *   vals[B*beam*nblk*K] | ids[B*beam*nblk*K] (int32) | final_vals[B*K] | final_ids[B*K] (int32)
- * nblk = onellm_beam_topk_blocks_per_row(V) (8 for any V >= 2048, as in the reference).
- * 1 <= K <= 8.  Slots with no candidate (V*beam < K) hold value -inf and id -1.
+ * nblk = ONELLM_TOPK_BLOCKS_PER_ROW (8, the reference's BlockPerBeam, beamsearch_topK.cu:105), so
+ * with K = beam = 2 the final results sit exactly where the reference's unit test reads them
+ * (tests/unittests/test_beamsearch_topK.cu:33-35).
+ * 1 <= K <= 8.  Slots with no candidate hold value -inf and id -1.
  */
+#define ONELLM_TOPK_BLOCKS_PER_ROW 8
 int onellm_beam_topk(const float* logits, int B, int beam, int V, int K,
                      float* workspace, onellm_stream_t stream);
-int onellm_beam_topk_blocks_per_row(int V);
-size_t onellm_beam_topk_workspace_bytes(int B, int beam, int V, int K);
+size_t onellm_beam_topk_workspace_bytes(int B, int beam, int K);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,81 @@
+"""Compiles the gfx950 HIP kernels and the C++ launcher shims into in-tree shared libraries.
+
+    python -m onellm_amd.build            # build what is out of date
+    python -m onellm_amd.build --force    # rebuild everything
+
+Outputs (next to this file): libonellm_hip.so (the C ABI of include/onellm_hip.h) and
+libonellm_launchers.so (the six launch* functions with oneLLM's own signatures).
+hipcc cross-compiles for gfx950 without a GPU.
+"""
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+INCLUDE = os.path.join(ROOT, "include")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+LIB_HIP = os.path.join(HERE, "libonellm_hip.so")
+LIB_LAUNCH = os.path.join(HERE, "libonellm_launchers.so")
+
+KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "tuning.cpp"]
+LAUNCHER_SOURCES = ["launchers.cpp"]
+
+# packed fp32 VALU forms are switched off on purpose (code generation only; scalar fp32 code is
+# what the kernels are written in)
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC, "-Wall", "-Wno-unused-function"]
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _newer(target, deps):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def _headers():
+    hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".h"))]
+    for d, _, fs in os.walk(INCLUDE):
+        hs += [os.path.join(d, f) for f in fs if f.endswith(".h")]
+    return hs
+
+
+def _compile(src, force):
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    path = os.path.join(CSRC, src)
+    if not force and not _newer(obj, [path] + _headers()):
+        return obj
+    cmd = [HIPCC, "-c", path, "-o", obj] + COMMON
+    if src.endswith(".hip"):
+        cmd += DEVICE
+    else:
+        cmd += ["-x", "hip", "--offload-arch=gfx950"] if False else []
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr[-4000:]))
+    return obj
+
+
+def build(force=False, verbose=False):
+    os.makedirs(OBJ, exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=6) as ex:
+        kobjs = list(ex.map(lambda s: _compile(s, force), KERNEL_SOURCES))
+        lobjs = list(ex.map(lambda s: _compile(s, force), LAUNCHER_SOURCES))
+    if force or _newer(LIB_HIP, kobjs):
+        cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_HIP] + kobjs
+        subprocess.run(cmd, check=True, capture_output=not verbose)
+    if force or _newer(LIB_LAUNCH, lobjs + [LIB_HIP]):
+        cmd = [HIPCC, "-shared", "-fPIC", "-o", LIB_LAUNCH] + lobjs + \
+              ["-L" + HERE, "-lonellm_hip", "-Wl,-rpath,$ORIGIN"]
+        subprocess.run(cmd, check=True, capture_output=not verbose)
+    return LIB_HIP, LIB_LAUNCH
+
+
+if __name__ == "__main__":
+    libs = build(force="--force" in sys.argv, verbose=True)
+    print("\n".join(libs))

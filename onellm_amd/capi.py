@@ -1,0 +1,165 @@
+"""ctypes binding of libonellm_hip.so (the C ABI in include/onellm_hip.h) for torch tensors.
+
+Every wrapper passes raw device pointers and launches on torch's current stream.  There is no
+fallback: if the library is not built, loading raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libonellm_hip.so")
+LAUNCHERS_PATH = os.path.join(_HERE, "libonellm_launchers.so")
+
+FP32, FP16 = 0, 1
+EINVAL, EUNSUPPORTED, EWORKSPACE = -1, -2, -3
+ATTN_NO_V_BIAS = 0x1
+ATTN_NO_CACHE_WRITE = 0x2
+TOPK_BLOCKS_PER_ROW = 8
+
+# every symbol include/onellm_hip.h declares: name -> (restype, argtypes)
+_vp, _ci, _cf, _cu, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_uint, ctypes.c_size_t
+SYMBOLS = {
+    "onellm_hip_version": (_ci, []),
+    "onellm_error_string": (ctypes.c_char_p, [_ci]),
+    "onellm_decode_attn": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp, _ci,
+                                 _ci, _cf, _ci, _cu, _vp, _sz, _vp]),
+    "onellm_decode_attn_workspace_bytes": (_sz, [_ci, _ci, _ci, _ci, _ci]),
+    "onellm_rmsnorm": (_ci, [_ci, _vp, _vp, _cf, _ci, _ci, _vp]),
+    "onellm_fused_add_bias_residual_rmsnorm": (_ci, [_ci, _vp, _vp, _vp, _vp, _cf, _ci, _ci, _vp]),
+    "onellm_kv_append": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp]),
+    "onellm_kv_repeat": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp]),
+    "onellm_beam_topk": (_ci, [_vp, _ci, _ci, _ci, _ci, _vp, _vp]),
+    "onellm_beam_topk_workspace_bytes": (_sz, [_ci, _ci, _ci]),
+}
+
+_lib = None
+
+
+class OnellmError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        msg = lib().onellm_error_string(code).decode()
+        super().__init__(f"{what} failed with code {code}: {msg}")
+
+
+def lib():
+    """Load the HIP library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m onellm_amd.build` "
+                               "(there is no CPU fallback)")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        L.onellm_tune_set.restype = _ci
+        L.onellm_tune_set.argtypes = [ctypes.c_char_p, _ci]
+        _lib = L
+    return _lib
+
+
+def tune_set(key, value):
+    """Internal tuning knob (benchmarks only); -1 restores the automatic choice."""
+    rc = lib().onellm_tune_set(key.encode(), int(value))
+    if rc:
+        raise OnellmError(rc, f"tune_set({key})")
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dt(t):
+    import torch
+    if t.dtype == torch.float32:
+        return FP32
+    if t.dtype == torch.float16:
+        return FP16
+    raise TypeError(f"unsupported dtype {t.dtype}")
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensors only"
+    return t.data_ptr()
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise OnellmError(rc, what)
+
+
+def decode_attn_workspace_bytes(B, Hq, Hkv, D, max_t):
+    return lib().onellm_decode_attn_workspace_bytes(B, Hq, Hkv, D, max_t)
+
+
+def decode_attn(qkv, bias, k_cache, v_cache, out, Hq, t, rotary_dim, rope_base, layer=0, t_dev=None,
+                max_t=None, rope_pos_offset=0, flags=0, workspace=None):
+    """qkv [B, Hq+2Hkv, D]; caches [L, B, Hkv, S, D]; out [B, Hq*D]; t host int (or max of t_dev).
+    `workspace` is a uint8 device tensor; allocated here when None."""
+    import torch
+    B, QKVH, D = qkv.shape
+    L, _, Hkv, S, _ = k_cache.shape
+    assert QKVH == Hq + 2 * Hkv
+    if max_t is None:
+        max_t = t
+    if workspace is None:
+        workspace = torch.empty(decode_attn_workspace_bytes(B, Hq, Hkv, D, max_t), dtype=torch.uint8, device=qkv.device)
+    rc = lib().onellm_decode_attn(_dt(qkv), _ptr(qkv), _ptr(bias), _ptr(k_cache), _ptr(v_cache), _ptr(out),
+                                  B, Hq, Hkv, D, S, layer, L, int(t), _ptr(t_dev), int(max_t),
+                                  rotary_dim, rope_base, rope_pos_offset, flags,
+                                  _ptr(workspace), workspace.numel(), _stream())
+    _check(rc, "onellm_decode_attn")
+    return out
+
+
+def rmsnorm(x, gamma, eps):
+    N, H = x.shape
+    _check(lib().onellm_rmsnorm(_dt(x), _ptr(x), _ptr(gamma), eps, N, H, _stream()), "onellm_rmsnorm")
+    return x
+
+
+def fused_add_bias_residual_rmsnorm(residual, out, bias, gamma, eps):
+    N, H = out.shape
+    _check(lib().onellm_fused_add_bias_residual_rmsnorm(_dt(out), _ptr(residual), _ptr(out), _ptr(bias), _ptr(gamma),
+                                                        eps, N, H, _stream()), "onellm_fused_add_bias_residual_rmsnorm")
+    return residual, out
+
+
+def kv_append(k_src, v_src, k_cache, v_cache, cur_len, history_len, layer=0):
+    B, Hkv, max_q_len, D = k_src.shape
+    L, _, _, S, _ = k_cache.shape
+    _check(lib().onellm_kv_append(_dt(k_src), _ptr(k_src), _ptr(v_src), _ptr(k_cache), _ptr(v_cache), _ptr(cur_len),
+                                  _ptr(history_len), B, Hkv, max_q_len, S, D, layer, L, _stream()), "onellm_kv_append")
+
+
+def kv_repeat(k_cache, v_cache, k_dst, v_dst, context_len, layer=0):
+    L, B, Hkv, S, D = k_cache.shape
+    _, Hq, max_k_len, _ = k_dst.shape
+    _check(lib().onellm_kv_repeat(_dt(k_cache), _ptr(k_cache), _ptr(v_cache), _ptr(k_dst), _ptr(v_dst),
+                                  _ptr(context_len), B, Hq, Hkv, S, max_k_len, D, layer, L, _stream()),
+           "onellm_kv_repeat")
+
+
+def beam_topk_workspace_bytes(B, beam, K):
+    return lib().onellm_beam_topk_workspace_bytes(B, beam, K)
+
+
+def beam_topk(logits, B, beam, K, workspace=None):
+    """logits [B*beam, V] fp32.  Returns (workspace, round1_vals, round1_ids, final_vals, final_ids) as views."""
+    import torch
+    rows, V = logits.shape
+    assert rows == B * beam and logits.dtype == torch.float32
+    if workspace is None:
+        workspace = torch.empty(beam_topk_workspace_bytes(B, beam, K) // 4, dtype=torch.float32, device=logits.device)
+    _check(lib().onellm_beam_topk(_ptr(logits), B, beam, V, K, _ptr(workspace), _stream()), "onellm_beam_topk")
+    n1 = B * beam * TOPK_BLOCKS_PER_ROW * K
+    vals = workspace[:n1].view(B * beam, TOPK_BLOCKS_PER_ROW, K)
+    ids = workspace[n1:2 * n1].view(torch.int32).view(B * beam, TOPK_BLOCKS_PER_ROW, K)
+    fv = workspace[2 * n1:2 * n1 + B * K].view(B, K)
+    fi = workspace[2 * n1 + B * K:2 * n1 + 2 * B * K].view(torch.int32).view(B, K)
+    return workspace, vals, ids, fv, fi

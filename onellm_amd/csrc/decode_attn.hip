@@ -1,0 +1,461 @@
+// Fused masked decoder self-attention for one new token per sequence, gfx950 (wave64).
+//
+// One launch fuses: q/k/v bias add, RoPE of q and k, the KV-cache write of row t-1, the scaled
+// scores against rows 0..t-1, the softmax and the weighted V sum.  The work is memory-bound (the
+// K and V history is read exactly once: 2*Hkv*(t-1)*D*e bytes per sequence), so the design is
+// about bytes in flight, not matrix cores:
+//
+//   * split over the sequence ("flash-decoding"): grid = (splits, kv-head x head-tile, batch); each
+//     workgroup streams one contiguous chunk of cache rows of one (sequence, kv-head) and keeps an
+//     online-softmax state (running max m, sum l, weighted V accumulator) per query head;
+//   * grouped-query heads are fused on the read side: a workgroup applies every K/V row it loads to
+//     up to GT query heads of the group, so the cache is never repeated in memory;
+//   * lane mapping: a cache row of D elements is LPR = D*sizeof(T)/16 lanes x 16 bytes, so a wave
+//     reads 64/LPR whole rows per global_load_dwordx4 (fully coalesced 1 KiB per instruction); the
+//     q.k dot product is finished by an LPR-lane DPP reduction, no LDS;
+//   * every group of LPR lanes owns an independent softmax state for the rows it sees; the states
+//     of a workgroup are merged once, through LDS, at the end of the chunk;
+//   * partial results (m, l, unnormalised acc) go to a workspace and a second tiny kernel merges
+//     the splits; with a single split the first kernel writes the output directly.
+//
+// Arithmetic is fp32 throughout; T is only the storage type of qkv, bias, cache and output.
+#include <math.h>
+#include "common.hpp"
+
+namespace onellm {
+namespace {
+
+constexpr int kMaxPairs = 256;                 // D <= 512
+struct RopeFreqs { float f[kMaxPairs]; };      // f[i] = base^(2i/rotary_dim), filled on the host
+
+struct AttnArgs {
+    const void* qkv;
+    const void* bias;
+    void* k_cache;
+    void* v_cache;
+    void* out;
+    float* part_o;        // [B, Hq, nsplit, D]
+    float* part_ml;       // [B, Hq, nsplit, 2]
+    const int* t_dev;
+    int t_host;
+    int B, Hq, Hkv, G, S;
+    int chunk;            // cache rows per split
+    int nsplit;           // grid.x
+    int rotary_dim;
+    int pos_offset;
+    unsigned flags;
+    float qscale;         // log2(e) / sqrt(D), folded into q
+    size_t slab;          // element offset of the layer slab inside the cache
+};
+
+// sin/cos as a fixed sequence of fp32 IEEE operations: 3-term Cody-Waite reduction by pi/2, the
+// single-precision minimax polynomials on [-pi/4, pi/4], quadrant from the multiple.  Every
+// multiply-add is an explicit fma so that a host implementation of the same sequence gives the
+// same bits (the K row written to the cache is bit-reproducible on a CPU).
+__device__ __forceinline__ void sincos_fixed(float x, float& s_out, float& c_out)
+{
+    const float j = __builtin_rintf(x * 0x1.45f306p-1f);
+    float r = __builtin_fmaf(-j, 0x1.921fb6p+0f, x);
+    r = __builtin_fmaf(-j, -0x1.777a5cp-25f, r);
+    r = __builtin_fmaf(-j, -0x1.0p-49f, r);
+    const float r2 = r * r;
+    float ps = __builtin_fmaf(-1.9515295891e-4f, r2, 8.3321608736e-3f);
+    ps = __builtin_fmaf(ps, r2, -1.6666654611e-1f);
+    const float sr = __builtin_fmaf(r * r2, ps, r);
+    float pc = __builtin_fmaf(2.443315711809948e-5f, r2, -1.388731625493765e-3f);
+    pc = __builtin_fmaf(pc, r2, 4.166664568298827e-2f);
+    const float cr = __builtin_fmaf(r2 * r2, pc, __builtin_fmaf(-0.5f, r2, 1.0f));
+    const int q = (int)j & 3;
+    float s = (q & 1) ? cr : sr;
+    float c = (q & 1) ? sr : cr;
+    if (q & 2) s = -s;
+    if ((q + 1) & 2) c = -c;
+    s_out = s;
+    c_out = c;
+}
+
+// rotate the pair (x0, x1) of index `pair` at position pos
+__device__ __forceinline__ void rope_pair(float& x0, float& x1, int pair, int pos, const RopeFreqs& fr)
+{
+    const float ang = (float)pos / fr.f[pair];
+    float s, c;
+    sincos_fixed(ang, s, c);
+    const float a = __builtin_fmaf(x0, c, -(x1 * s));
+    const float b = __builtin_fmaf(x1, c, x0 * s);
+    x0 = a;
+    x1 = b;
+}
+
+template <typename T, int LPR, int GT, int U, int NW>
+__global__ __launch_bounds__(NW * kWave)
+void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
+{
+    constexpr int VEC = Elt<T>::kVec;
+    constexpr int D = LPR * VEC;
+    constexpr int RPW = kWave / LPR;            // cache rows per wave per load instruction
+    constexpr int NRG = NW * RPW;               // row groups (independent softmax states) per workgroup
+    constexpr int NTHR = NW * kWave;
+
+    extern __shared__ float lds[];
+    float* sq = lds;                            // [GT][D]   roped q * qscale
+    float* sk = sq + GT * D;                    // [D]       new k row (as stored)
+    float* sv = sk + D;                         // [D]       new v row (as stored)
+    float* snew = sv + D;                       // [GT]      score of the new row
+    float* st_ml = snew + GT;                   // [NRG][GT][2]
+    float* st_acc = st_ml + NRG * GT * 2;       // [NRG][GT][D]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int split = blockIdx.x;
+    const int ngt = (a.G + GT - 1) / GT;
+    const int kvh = blockIdx.y / ngt;
+    const int g0 = (blockIdx.y % ngt) * GT;
+    const int b = blockIdx.z;
+
+    const int t = a.t_dev ? a.t_dev[b] : a.t_host;
+    if (t < 1 || t > a.S) return;               // out-of-contract length: touch nothing
+    const int last = (t - 1) / a.chunk;
+    if (split > last) return;
+    const bool is_last = split == last;
+    const int r0 = split * a.chunk;
+    const int r1 = min(r0 + a.chunk, t - 1);    // history rows [r0, r1)
+    const int pos = t + a.pos_offset;
+
+    const T* qkv = static_cast<const T*>(a.qkv) + (size_t)b * (a.Hq + 2 * a.Hkv) * D;
+    const T* bias = static_cast<const T*>(a.bias);
+    const size_t head_off = a.slab + ((size_t)b * a.Hkv + kvh) * (size_t)a.S * D;
+    T* kc = static_cast<T*>(a.k_cache) + head_off;
+    T* vc = static_cast<T*>(a.v_cache) + head_off;
+
+    // ---- q (and, in the last split, the new k/v row): bias, RoPE, staging in LDS
+    for (int i = tid; i < GT * (D / 2); i += NTHR) {
+        const int g = i / (D / 2), p = i % (D / 2);
+        float x0 = 0.f, x1 = 0.f;
+        if (g0 + g < a.G) {
+            const int h = kvh * a.G + g0 + g;
+            x0 = to_f32(qkv[h * D + 2 * p]);
+            x1 = to_f32(qkv[h * D + 2 * p + 1]);
+            if (bias) {
+                x0 += to_f32(bias[h * D + 2 * p]);
+                x1 += to_f32(bias[h * D + 2 * p + 1]);
+            }
+            if (2 * p < a.rotary_dim) rope_pair(x0, x1, p, pos, fr);
+        }
+        sq[g * D + 2 * p] = x0 * a.qscale;
+        sq[g * D + 2 * p + 1] = x1 * a.qscale;
+    }
+    if (is_last) {
+        const bool store = g0 == 0 && !(a.flags & ONELLM_ATTN_NO_CACHE_WRITE);
+        for (int p = tid; p < D / 2; p += NTHR) {
+            const int o = (a.Hq + kvh) * D + 2 * p;
+            float x0 = to_f32(qkv[o]), x1 = to_f32(qkv[o + 1]);
+            if (bias) {
+                x0 += to_f32(bias[o]);
+                x1 += to_f32(bias[o + 1]);
+            }
+            if (2 * p < a.rotary_dim) rope_pair(x0, x1, p, pos, fr);
+            const T k0 = from_f32<T>(x0), k1 = from_f32<T>(x1);
+            sk[2 * p] = to_f32(k0);
+            sk[2 * p + 1] = to_f32(k1);
+            if (store) {
+                kc[(size_t)(t - 1) * D + 2 * p] = k0;
+                kc[(size_t)(t - 1) * D + 2 * p + 1] = k1;
+            }
+        }
+        for (int d = tid; d < D; d += NTHR) {
+            const int o = (a.Hq + a.Hkv + kvh) * D + d;
+            float x = to_f32(qkv[o]);
+            if (bias && !(a.flags & ONELLM_ATTN_NO_V_BIAS)) x += to_f32(bias[o]);
+            const T v = from_f32<T>(x);
+            sv[d] = to_f32(v);
+            if (store) vc[(size_t)(t - 1) * D + d] = v;
+        }
+    }
+    __syncthreads();
+
+    const int col = (lane % LPR) * VEC;         // first of this lane's VEC columns
+    float qr[GT][VEC];
+#pragma unroll
+    for (int g = 0; g < GT; ++g)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) qr[g][e] = sq[g * D + col + e];
+
+    if (is_last && wave == 0) {
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+            float part = 0.f;
+            for (int d = lane; d < D; d += kWave) part = fmaf(sq[g * D + d], sk[d], part);
+            part = wave_sum(part);
+            if (lane == 0) snew[g] = part;
+        }
+    }
+
+    // ---- stream the history rows of this chunk
+    float m[GT], l[GT], acc[GT][VEC];
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+        m[g] = -INFINITY;
+        l[g] = 0.f;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[g][e] = 0.f;
+    }
+
+    const int rg = wave * RPW + lane / LPR;     // row group of this lane
+    constexpr int RPI = U * NRG;                // rows per workgroup iteration
+    const T* kp = kc + col;
+    const T* vp = vc + col;
+
+    auto body = [&](int rbase, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        Vec16<T> kv[U], vv[U];
+        bool valid[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int row = rbase + u * NRG + rg;
+            if constexpr (MASKED) {
+                valid[u] = row < r1;
+                row = min(row, r1 - 1);
+            }
+            kv[u] = load16(kp + (size_t)row * D);
+            vv[u] = load16(vp + (size_t)row * D);
+        }
+        float s[GT][U];
+#pragma unroll
+        for (int g = 0; g < GT; ++g)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float part = 0.f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) part = fmaf(qr[g][e], kv[u].get(e), part);
+                part = group_sum<LPR>(part);
+                if constexpr (MASKED) part = valid[u] ? part : -INFINITY;
+                s[g][u] = part;
+            }
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+            float mx = m[g];
+#pragma unroll
+            for (int u = 0; u < U; ++u) mx = fmaxf(mx, s[g][u]);
+            float mref = mx;
+            if constexpr (MASKED) mref = (mx == -INFINITY) ? 0.f : mx;   // nothing seen yet: keep zeros
+            const float alpha = __builtin_amdgcn_exp2f(m[g] - mref);
+            float psum = 0.f;
+            float p[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                p[u] = __builtin_amdgcn_exp2f(s[g][u] - mref);
+                psum += p[u];
+            }
+            l[g] = fmaf(l[g], alpha, psum);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float v = acc[g][e] * alpha;
+#pragma unroll
+                for (int u = 0; u < U; ++u) v = fmaf(p[u], vv[u].get(e), v);
+                acc[g][e] = v;
+            }
+            m[g] = mx;
+        }
+    };
+
+    if (r1 > r0) {
+        const int nfull = (r1 - r0) / RPI;
+        int rbase = r0;
+        for (int it = 0; it < nfull; ++it, rbase += RPI) body(rbase, std::false_type{});
+        if (rbase < r1) body(rbase, std::true_type{});
+    }
+
+    // ---- merge the row-group states of the workgroup
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+        if (lane % LPR == 0) {
+            st_ml[(rg * GT + g) * 2] = m[g];
+            st_ml[(rg * GT + g) * 2 + 1] = l[g];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) st_acc[(size_t)(rg * GT + g) * D + col + e] = acc[g][e];
+    }
+    __syncthreads();
+
+    for (int i = tid; i < GT * D; i += NTHR) {
+        const int g = i / D, d = i % D;
+        if (g0 + g >= a.G) continue;
+        float M = is_last ? snew[g] : -INFINITY;
+        for (int r = 0; r < NRG; ++r) M = fmaxf(M, st_ml[(r * GT + g) * 2]);
+        float L = 0.f, O = 0.f;
+        for (int r = 0; r < NRG; ++r) {
+            const float w = __builtin_amdgcn_exp2f(st_ml[(r * GT + g) * 2] - M);
+            L = fmaf(st_ml[(r * GT + g) * 2 + 1], w, L);
+            O = fmaf(st_acc[(size_t)(r * GT + g) * D + d], w, O);
+        }
+        if (is_last) {
+            const float w = __builtin_amdgcn_exp2f(snew[g] - M);
+            L += w;
+            O = fmaf(sv[d], w, O);
+        }
+        const int h = kvh * a.G + g0 + g;
+        if (a.nsplit == 1) {
+            static_cast<T*>(a.out)[((size_t)b * a.Hq + h) * D + d] = from_f32<T>(O / L);
+        } else {
+            const size_t pi = ((size_t)b * a.Hq + h) * a.nsplit + split;
+            a.part_o[pi * D + d] = O;
+            if (d == 0) {
+                a.part_ml[pi * 2] = M;
+                a.part_ml[pi * 2 + 1] = L;
+            }
+        }
+    }
+}
+
+// Merge the per-split partial states of one (sequence, query head) and normalise.
+template <typename T>
+__global__ __launch_bounds__(128)
+void decode_attn_merge_kernel(const AttnArgs a, int D)
+{
+    const int bh = blockIdx.x;
+    const int b = bh / a.Hq;
+    const int t = a.t_dev ? a.t_dev[b] : a.t_host;
+    if (t < 1 || t > a.S) return;
+    const int nvalid = min((t - 1) / a.chunk + 1, a.nsplit);   // t above max_t is out of contract: stay in bounds
+    const float* ml = a.part_ml + (size_t)bh * a.nsplit * 2;
+    const float* po = a.part_o + (size_t)bh * a.nsplit * D;
+    float M = -INFINITY;
+    for (int s = 0; s < nvalid; ++s) M = fmaxf(M, ml[s * 2]);
+    float L = 0.f;
+    for (int s = 0; s < nvalid; ++s) L = fmaf(ml[s * 2 + 1], __builtin_amdgcn_exp2f(ml[s * 2] - M), L);
+    const float invL = 1.0f / L;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float O = 0.f;
+        for (int s = 0; s < nvalid; ++s) O = fmaf(po[(size_t)s * D + d], __builtin_amdgcn_exp2f(ml[s * 2] - M), O);
+        static_cast<T*>(a.out)[(size_t)bh * D + d] = from_f32<T>(O * invL);
+    }
+}
+
+constexpr int kNW = 4;              // waves per workgroup
+constexpr int kMaxSplits = 64;      // upper bound of splits the workspace is sized for
+constexpr int kMinChunk = 64;       // never split finer than this many cache rows
+
+template <typename T, int LPR, int GT>
+int launch_split(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    constexpr int U = GT >= 4 ? 2 : 4;
+    constexpr int D = LPR * Elt<T>::kVec;
+    constexpr int NRG = kNW * (kWave / LPR);
+    const size_t lds_bytes = sizeof(float) * (size_t)(GT * D + 2 * D + GT + NRG * GT * 2 + (size_t)NRG * GT * D);
+    if (lds_bytes > 64 * 1024) return ONELLM_EUNSUPPORTED;
+    const int ngt = (a.G + GT - 1) / GT;
+    const dim3 grid(a.nsplit, a.Hkv * ngt, a.B), block(kNW * kWave);
+    hipLaunchKernelGGL((decode_attn_split_kernel<T, LPR, GT, U, kNW>), grid, block, lds_bytes, st, a, fr);
+    return launch_status();
+}
+
+template <typename T, int LPR>
+int launch_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    if (a.G == 1) return launch_split<T, LPR, 1>(a, fr, st);
+    if (a.G == 2) return launch_split<T, LPR, 2>(a, fr, st);
+    return launch_split<T, LPR, 4>(a, fr, st);
+}
+
+template <typename T>
+int launch_lpr(int lpr, const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    switch (lpr) {
+        case 1: return launch_gt<T, 1>(a, fr, st);
+        case 2: return launch_gt<T, 2>(a, fr, st);
+        case 4: return launch_gt<T, 4>(a, fr, st);
+        case 8: return launch_gt<T, 8>(a, fr, st);
+        case 16: return launch_gt<T, 16>(a, fr, st);
+        case 32: return launch_gt<T, 32>(a, fr, st);
+        case 64: return launch_gt<T, 64>(a, fr, st);
+        default: return ONELLM_EUNSUPPORTED;
+    }
+}
+
+int max_splits(int max_t)
+{
+    int n = (max_t + kMinChunk - 1) / kMinChunk;
+    return n < 1 ? 1 : (n > kMaxSplits ? kMaxSplits : n);
+}
+
+}  // namespace
+}  // namespace onellm
+
+extern "C" size_t onellm_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int max_t)
+{
+    (void)Hkv;
+    if (B <= 0 || Hq <= 0 || D <= 0 || max_t <= 0) return 256;
+    const size_t n = (size_t)B * Hq * onellm::max_splits(max_t) * (size_t)(D + 2) * sizeof(float);
+    return (n + 255) & ~(size_t)255;
+}
+
+extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bias, void* k_cache, void* v_cache,
+                                  void* out, int B, int Hq, int Hkv, int D, int S, int layer, int num_layers,
+                                  int t_host, const int* t_dev, int max_t, int rotary_dim, float rope_base,
+                                  int rope_pos_offset, unsigned flags, void* workspace, size_t workspace_bytes,
+                                  onellm_stream_t stream)
+{
+    using namespace onellm;
+    if (!qkv || !k_cache || !v_cache || !out) return ONELLM_EINVAL;
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || S <= 0 || num_layers <= 0) return ONELLM_EINVAL;
+    if (layer < 0 || layer >= num_layers || Hq % Hkv) return ONELLM_EINVAL;
+    if (dtype != ONELLM_FP32 && dtype != ONELLM_FP16) return ONELLM_EINVAL;
+    if (!t_dev) max_t = t_host;
+    if (max_t < 1 || max_t > S || (!t_dev && (t_host < 1 || t_host > S))) return ONELLM_EINVAL;
+    if (rotary_dim < 0 || (rotary_dim > 0 && !(rope_base > 0.f))) return ONELLM_EINVAL;
+    const int esz = dtype == ONELLM_FP16 ? 2 : 4;
+    const int row_bytes = D * esz;
+    if (row_bytes < 16 || row_bytes > 1024 || (row_bytes & (row_bytes - 1))) return ONELLM_EUNSUPPORTED;
+    if (!aligned16(k_cache) || !aligned16(v_cache)) return ONELLM_EUNSUPPORTED;
+    const int lpr = row_bytes / 16;
+
+    AttnArgs a{};
+    a.qkv = qkv; a.bias = qkv_bias; a.k_cache = k_cache; a.v_cache = v_cache; a.out = out;
+    a.t_dev = t_dev; a.t_host = t_host;
+    a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.G = Hq / Hkv; a.S = S;
+    a.rotary_dim = rotary_dim; a.pos_offset = rope_pos_offset; a.flags = flags;
+    a.qscale = (1.0f / sqrtf((float)D)) * 1.4426950408889634f;
+    a.slab = (size_t)layer * B * Hkv * (size_t)S * D;
+
+    // sequence split: enough workgroups to cover the chip several times over, chunks not below kMinChunk
+    const int G = a.G;
+    const int gt = G == 1 ? 1 : (G == 2 ? 2 : 4);
+    const int ngt = (G + gt - 1) / gt;
+    const long base_wgs = (long)B * Hkv * ngt;
+    int target = tune_get("attn_target_wgs");
+    if (target <= 0) target = 2048;
+    int nsplit = (int)((target + base_wgs - 1) / base_wgs);
+    const int cap = max_splits(max_t);
+    if (nsplit > cap) nsplit = cap;
+    if (nsplit < 1) nsplit = 1;
+    const int forced = tune_get("attn_nsplit");
+    if (forced > 0) nsplit = forced > cap ? cap : forced;
+    int chunk = (max_t + nsplit - 1) / nsplit;
+    chunk = (chunk + kMinChunk - 1) / kMinChunk * kMinChunk;
+    nsplit = (max_t + chunk - 1) / chunk;
+    a.chunk = chunk;
+    a.nsplit = nsplit;
+
+    if (nsplit > 1) {
+        const size_t need = (size_t)B * Hq * nsplit * (size_t)(D + 2) * sizeof(float);
+        if (!workspace || workspace_bytes < need) return ONELLM_EWORKSPACE;
+        a.part_o = static_cast<float*>(workspace);
+        a.part_ml = a.part_o + (size_t)B * Hq * nsplit * D;
+    }
+
+    RopeFreqs fr;
+    for (int i = 0; 2 * i < rotary_dim && 2 * i + 1 < D; ++i) fr.f[i] = powf(rope_base, (float)(2 * i) / (float)rotary_dim);
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int rc = dtype == ONELLM_FP16 ? launch_lpr<__half>(lpr, a, fr, st) : launch_lpr<float>(lpr, a, fr, st);
+    if (rc != 0) return rc;
+    if (nsplit > 1) {
+        if (dtype == ONELLM_FP16)
+            hipLaunchKernelGGL((decode_attn_merge_kernel<__half>), dim3(B * Hq), dim3(128), 0, st, a, D);
+        else
+            hipLaunchKernelGGL((decode_attn_merge_kernel<float>), dim3(B * Hq), dim3(128), 0, st, a, D);
+        rc = launch_status();
+    }
+    return rc;
+}

@@ -1,0 +1,56 @@
+// Library version, error strings and the internal tuning table.
+#include <string.h>
+#include <atomic>
+#include <hip/hip_runtime_api.h>
+#include "onellm_hip.h"
+
+namespace onellm {
+
+namespace {
+struct Knob {
+    const char* key;
+    std::atomic<int> value;
+};
+// -1 = let the launcher decide.  Meant for benchmarks and sweeps, not part of the stable ABI.
+Knob g_knobs[] = {
+    {"norm_tpr", {-1}},          // threads per row of the norm kernels: 64, 256 or 1024
+    {"attn_target_wgs", {-1}},   // workgroups the sequence split of decode attention aims for
+    {"attn_nsplit", {-1}},       // force the number of sequence splits
+    {"topk_single", {-1}},       // reserved
+};
+}  // namespace
+
+int tune_get(const char* key)
+{
+    for (auto& k : g_knobs)
+        if (strcmp(k.key, key) == 0) return k.value.load(std::memory_order_relaxed);
+    return -1;
+}
+
+}  // namespace onellm
+
+extern "C" int onellm_hip_version(void) { return 1000; }
+
+extern "C" int onellm_tune_set(const char* key, int value)
+{
+    if (!key) return ONELLM_EINVAL;
+    for (auto& k : onellm::g_knobs)
+        if (strcmp(k.key, key) == 0) {
+            k.value.store(value, std::memory_order_relaxed);
+            return 0;
+        }
+    return ONELLM_EINVAL;
+}
+
+extern "C" const char* onellm_error_string(int code)
+{
+    switch (code) {
+        case 0: return "success";
+        case ONELLM_EINVAL: return "onellm: invalid argument (null pointer, non-positive size or unknown enum)";
+        case ONELLM_EUNSUPPORTED: return "onellm: shape or alignment not supported by the gfx950 kernels";
+        case ONELLM_EWORKSPACE: return "onellm: workspace missing or too small";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "onellm: unknown error code";
+}

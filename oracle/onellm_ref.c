@@ -196,10 +196,10 @@ int onellm_ref_decode_attn(int dtype, const void* qkv, const void* qkv_bias,
             const size_t tok = (size_t)b * QKVH * D;
             /* new k / v rows */
             for (int d = 0; d < D; ++d) {
-                float kb = qkv_bias ? ld(qkv_bias, (size_t)(Hq + kvh) * D + d, dtype) : 0.0f;
-                float vb = (qkv_bias && !(flags & REF_ATTN_NO_V_BIAS)) ? ld(qkv_bias, (size_t)(Hq + Hkv + kvh) * D + d, dtype) : 0.0f;
-                kn[d] = ld(qkv, tok + (size_t)(Hq + kvh) * D + d, dtype) + kb;
-                vn[d] = ld(qkv, tok + (size_t)(Hq + Hkv + kvh) * D + d, dtype) + vb;
+                kn[d] = ld(qkv, tok + (size_t)(Hq + kvh) * D + d, dtype);
+                vn[d] = ld(qkv, tok + (size_t)(Hq + Hkv + kvh) * D + d, dtype);
+                if (qkv_bias) kn[d] += ld(qkv_bias, (size_t)(Hq + kvh) * D + d, dtype);
+                if (qkv_bias && !(flags & REF_ATTN_NO_V_BIAS)) vn[d] += ld(qkv_bias, (size_t)(Hq + Hkv + kvh) * D + d, dtype);
             }
             onellm_ref_rope_row(kn, D, rotary_dim, freq, pos);
             for (int d = 0; d < D; ++d) {
@@ -216,8 +216,8 @@ int onellm_ref_decode_attn(int dtype, const void* qkv, const void* qkv_bias,
             for (int g = 0; g < G; ++g) {
                 const int h = kvh * G + g;
                 for (int d = 0; d < D; ++d) {
-                    float qb = qkv_bias ? ld(qkv_bias, (size_t)h * D + d, dtype) : 0.0f;
-                    q[d] = ld(qkv, tok + (size_t)h * D + d, dtype) + qb;
+                    q[d] = ld(qkv, tok + (size_t)h * D + d, dtype);
+                    if (qkv_bias) q[d] += ld(qkv_bias, (size_t)h * D + d, dtype);
                 }
                 onellm_ref_rope_row(q, D, rotary_dim, freq, pos);
                 float smax = -INFINITY;
@@ -304,8 +304,8 @@ int onellm_ref_fused_add_bias_residual_rmsnorm(int dtype, void* residual, void* 
         float* r = (float*)malloc(sizeof(float) * (size_t)H);
         double ss = 0;
         for (int i = 0; i < H; ++i) {
-            float b = bias ? ld(bias, i, dtype) : 0.0f;
-            r[i] = ld(out, o + i, dtype) + ld(residual, o + i, dtype) + b;
+            r[i] = ld(out, o + i, dtype) + ld(residual, o + i, dtype);
+            if (bias) r[i] += ld(bias, i, dtype);          /* no "+ 0" when absent: keeps -0 */
             ss += (double)r[i] * r[i];
         }
         const float inv = (float)(1.0 / sqrt(ss / H + (double)eps));

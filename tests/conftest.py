@@ -19,3 +19,25 @@ def ref():
     _ref.build()
     _ref.lib()
     return _ref
+
+
+def announce(*parts):
+    """Name the case on the real stderr (unbuffered, not captured) before a GPU step, so a run that
+    dies inside the GPU call still shows which case it was."""
+    sys.__stderr__.write("[case] " + " ".join(str(p) for p in parts) + "\n")
+    sys.__stderr__.flush()
+
+
+@pytest.fixture(scope="session")
+def capi():
+    """The HIP library through its C ABI.  Raises (never skips) if it is not built."""
+    from onellm_amd import capi as _capi
+    _capi.lib()
+    return _capi
+
+
+@pytest.fixture(scope="session")
+def dev():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return torch.device("cuda:0")

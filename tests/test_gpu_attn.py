@@ -1,0 +1,215 @@
+"""GPU parity of the fused decode attention against the CPU oracle, through the C ABI.
+
+Tolerances (written once, used everywhere): fp32 outputs 1e-5 relative (plus 1e-6 absolute for
+values that cancel to near zero); fp16 outputs 2e-3 absolute / 1e-2 relative.  The cache row the
+step writes is compared bit for bit: v is one fp32 add rounded once, k goes through the same fixed
+sequence of fp32 operations on both sides."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.float32: dict(rtol=1e-5, atol=1e-6), np.float16: dict(rtol=1e-2, atol=2e-3)}
+
+
+def _bits(a):
+    return a.view(np.uint16 if a.dtype == np.float16 else np.uint32)
+
+
+def _case(dtype, B, Hq, Hkv, D, S, L, seed, std=1.0):
+    rng = np.random.default_rng(seed)
+    qkv = (rng.standard_normal((B, Hq + 2 * Hkv, D)) * std).astype(dtype)
+    bias = (rng.standard_normal((Hq + 2 * Hkv) * D) * std).astype(dtype)
+    kc = (rng.standard_normal((L, B, Hkv, S, D)) * std).astype(dtype)
+    vc = (rng.standard_normal((L, B, Hkv, S, D)) * std).astype(dtype)
+    return qkv, bias, kc, vc
+
+
+def _run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, rotary_dim, base=10000.0, layer=0, pos_offset=0, flags=0):
+    """Runs GPU and oracle on the same inputs; returns (gpu_out, ref_out, gpu_kc, gpu_vc, ref_kc, ref_vc)."""
+    d_qkv = torch.from_numpy(qkv).to(dev)
+    d_bias = torch.from_numpy(bias).to(dev) if bias is not None else None
+    d_kc, d_vc = torch.from_numpy(kc).to(dev), torch.from_numpy(vc).to(dev)
+    B, _, D = qkv.shape
+    d_out = torch.zeros(B, Hq * D, dtype=d_qkv.dtype, device=dev)
+    if isinstance(t, np.ndarray):
+        t_dev = torch.from_numpy(t.astype(np.int32)).to(dev)
+        capi.decode_attn(d_qkv, d_bias, d_kc, d_vc, d_out, Hq, int(t.max()), rotary_dim, base, layer=layer,
+                         t_dev=t_dev, max_t=int(t.max()), rope_pos_offset=pos_offset, flags=flags)
+    else:
+        capi.decode_attn(d_qkv, d_bias, d_kc, d_vc, d_out, Hq, t, rotary_dim, base, layer=layer,
+                         rope_pos_offset=pos_offset, flags=flags)
+    r_kc, r_vc = kc.copy(), vc.copy()
+    r_out = ref.decode_attn(qkv, bias, r_kc, r_vc, Hq, t, rotary_dim, base, layer=layer, rope_pos_offset=pos_offset,
+                            flags=flags)
+    return d_out.cpu().numpy(), r_out, d_kc.cpu().numpy(), d_vc.cpu().numpy(), r_kc, r_vc
+
+
+def _assert_parity(res, dtype):
+    g_out, r_out, g_kc, g_vc, r_kc, r_vc = res
+    np.testing.assert_allclose(g_out.astype(np.float64), r_out.astype(np.float64), **TOL[dtype])
+    np.testing.assert_array_equal(_bits(g_kc), _bits(r_kc))      # whole cache, including the new row
+    np.testing.assert_array_equal(_bits(g_vc), _bits(r_vc))
+
+
+def test_config1_fp32_small(capi, ref, dev):
+    # BASELINE config 1: fp32, B1, 8 heads x 64, 16 cached steps + the current token, rotary 64, seed 0
+    announce("attn config1")
+    qkv, bias, kc, vc = _case(np.float32, 1, 8, 8, 64, 32, 1, seed=0)
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 17, 64), np.float32)
+
+
+def test_reference_unit_test_shape(capi, ref, dev):
+    # tests/unittests/test_decoder_masked_attn.cu:113-176 of the reference: B1 Hq2 Hkv1 D16 step4
+    announce("attn unit-test shape")
+    B, Hq, Hkv, D, t, S = 1, 2, 1, 16, 4, 32
+    qkv = np.ones((B, Hq + 2 * Hkv, D), np.float32)
+    bias = np.full(((Hq + 2 * Hkv) * D,), 2.0, np.float32)
+    kc = np.zeros((1, B, Hkv, S, D), np.float32)
+    vc = np.zeros((1, B, Hkv, S, D), np.float32)
+    kc[:, :, :, :t] = 1.0
+    vc[:, :, :, :t] = 1.0
+    res = _run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, 128, flags=capi.ATTN_NO_V_BIAS)
+    _assert_parity(res, np.float32)
+    np.testing.assert_allclose(res[0], 1.0, rtol=1e-6)            # all V rows are 1
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, 128), np.float32)
+
+
+def test_example_driver_shape_two_layers(capi, ref, dev):
+    # examples/cpp/decoder/self_decoder_example.cpp:10-27: Hq4 Hkv2 D8 B2 step3 max_seq12 rotary 128
+    announce("attn example driver shape")
+    qkv, bias, kc, vc = _case(np.float32, 2, 4, 2, 8, 12, 2, seed=3)
+    for layer in (0, 1):
+        _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 4, 3, 128, layer=layer), np.float32)
+
+
+@pytest.mark.parametrize("dtype,Hq,Hkv,D", [
+    (np.float16, 4, 4, 128), (np.float16, 8, 2, 128), (np.float16, 8, 1, 64), (np.float16, 6, 3, 32),
+    (np.float16, 12, 2, 256), (np.float16, 2, 2, 8), (np.float16, 4, 2, 16), (np.float16, 2, 1, 512),
+    (np.float32, 4, 4, 128), (np.float32, 8, 2, 64), (np.float32, 3, 1, 32), (np.float32, 2, 2, 256),
+    (np.float32, 4, 1, 4), (np.float32, 10, 2, 16),
+])
+@pytest.mark.parametrize("t", [1, 2, 63, 64, 65, 300])
+def test_shapes_and_lengths(capi, ref, dev, dtype, Hq, Hkv, D, t):
+    announce("attn", dtype.__name__, Hq, Hkv, D, "t", t)
+    qkv, bias, kc, vc = _case(dtype, 3, Hq, Hkv, D, 304, 1, seed=Hq * 1000 + D + t, std=0.5)
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("nsplit", [1, 2, 5, 64])
+def test_sequence_split_counts_and_ragged_lengths(capi, ref, dev, dtype, nsplit):
+    announce("attn ragged", dtype.__name__, "nsplit", nsplit)
+    B, Hq, Hkv, D, S = 6, 8, 2, 128 if dtype == np.float16 else 64, 1100
+    qkv, bias, kc, vc = _case(dtype, B, Hq, Hkv, D, S, 1, seed=11 + nsplit, std=0.5)
+    t = np.array([1, 1100, 64, 513, 2, 777])
+    capi.tune_set("attn_nsplit", nsplit)
+    try:
+        _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), dtype)
+    finally:
+        capi.tune_set("attn_nsplit", -1)
+
+
+def test_options(capi, ref, dev):
+    announce("attn options")
+    qkv, bias, kc, vc = _case(np.float16, 2, 4, 2, 64, 40, 1, seed=21, std=0.5)
+    _assert_parity(_run_both(capi, ref, dev, qkv, None, kc, vc, 4, 33, 64), np.float16)               # no bias
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 4, 33, 0), np.float16)                # no rotation
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 4, 33, 32), np.float16)               # partial rotation
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 4, 33, 64, pos_offset=-1), np.float16)
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 4, 33, 64, base=500000.0), np.float16)
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 4, 33, 64, flags=capi.ATTN_NO_V_BIAS), np.float16)
+    res = _run_both(capi, ref, dev, qkv, bias, kc, vc, 4, 33, 64, flags=capi.ATTN_NO_CACHE_WRITE)
+    _assert_parity(res, np.float16)
+    np.testing.assert_array_equal(_bits(res[2]), _bits(kc))                                          # untouched
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 4, 40, 64), np.float16)               # t == S
+
+
+def test_config2_llama7b_full_size(capi, ref, dev):
+    # BASELINE config 2: fp16, B16, 32 x 128, cache [1,16,32,4096,128] ~ N(0,0.5); contexts 512..4096
+    torch.manual_seed(2)
+    B, H, D, S = 16, 32, 128, 4096
+    d_kc = torch.randn(1, B, H, S, D, device=dev).mul_(0.5).half()
+    d_vc = torch.randn(1, B, H, S, D, device=dev).mul_(0.5).half()
+    d_qkv = torch.randn(B, 3 * H, D, device=dev).mul_(0.5).half()
+    d_bias = torch.randn(3 * H * D, device=dev).mul_(0.5).half()
+    kc, vc = d_kc.cpu().numpy(), d_vc.cpu().numpy()
+    qkv, bias = d_qkv.cpu().numpy(), d_bias.cpu().numpy()
+    ws = torch.empty(capi.decode_attn_workspace_bytes(B, H, H, D, S), dtype=torch.uint8, device=dev)
+    for t in (512, 1024, 2048, 4096):
+        announce("attn config2 t", t)
+        g_kc, g_vc = d_kc.clone(), d_vc.clone()
+        out = torch.zeros(B, H * D, dtype=torch.float16, device=dev)
+        capi.decode_attn(d_qkv, d_bias, g_kc, g_vc, out, H, t, D, 10000.0, workspace=ws)
+        r_kc, r_vc = kc.copy(), vc.copy()
+        want = ref.decode_attn(qkv, bias, r_kc, r_vc, H, t, D, 10000.0)
+        np.testing.assert_allclose(out.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[np.float16])
+        np.testing.assert_array_equal(_bits(g_kc[0, :, :, t - 1].cpu().numpy()), _bits(r_kc[0, :, :, t - 1]))
+        np.testing.assert_array_equal(_bits(g_vc[0, :, :, t - 1].cpu().numpy()), _bits(r_vc[0, :, :, t - 1]))
+        g_kc[0, :, :, t - 1] = d_kc[0, :, :, t - 1]
+        g_vc[0, :, :, t - 1] = d_vc[0, :, :, t - 1]
+        assert torch.equal(g_kc, d_kc) and torch.equal(g_vc, d_vc)              # nothing else was written
+        # run-to-run: bit-identical output
+        out2 = torch.zeros_like(out)
+        capi.decode_attn(d_qkv, d_bias, d_kc.clone(), d_vc.clone(), out2, H, t, D, 10000.0, workspace=ws)
+        assert torch.equal(out, out2)
+
+
+def test_config3_gqa_fused_equals_repeat_path(capi, ref, dev):
+    # BASELINE config 3: fp16, B32, 32 q heads over 8 kv heads x 128, S 8192, lengths U[1024, 8192].
+    # (i) reference-style: concat the new row, repeat KV to 32 heads, attend with Hkv == Hq;
+    # (ii) fused: attend straight from the [B, 8, S, 128] cache.  Both against the oracle.
+    announce("attn config3 setup")
+    torch.manual_seed(3)
+    B, Hq, Hkv, D, S = 32, 32, 8, 128, 8192
+    G = Hq // Hkv
+    d_kc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+    d_vc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+    d_qkv = torch.randn(B, Hq + 2 * Hkv, D, device=dev).mul_(0.5).half()
+    d_bias = torch.randn((Hq + 2 * Hkv) * D, device=dev).mul_(0.5).half()
+    t = np.random.default_rng(3).integers(1024, 8193, size=B).astype(np.int32)
+    t[0], t[1] = 8192, 1024
+    d_t = torch.from_numpy(t).to(dev)
+    # oracle
+    r_kc, r_vc = d_kc.cpu().numpy(), d_vc.cpu().numpy()
+    want = ref.decode_attn(d_qkv.cpu().numpy(), d_bias.cpu().numpy(), r_kc, r_vc, Hq, t, D, 10000.0)
+    # (ii) fused
+    announce("attn config3 fused")
+    f_kc, f_vc = d_kc.clone(), d_vc.clone()
+    out_f = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+    capi.decode_attn(d_qkv, d_bias, f_kc, f_vc, out_f, Hq, int(t.max()), D, 10000.0, t_dev=d_t, max_t=int(t.max()))
+    np.testing.assert_allclose(out_f.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[np.float16])
+    assert np.array_equal(_bits(f_kc.cpu().numpy()), _bits(r_kc)) and np.array_equal(_bits(f_vc.cpu().numpy()), _bits(r_vc))
+    # (i) repeat path on the cache that already holds the new rows: broadcast to 32 heads, then a
+    # 32-head attention that re-derives the same new row (written again, same bits)
+    announce("attn config3 repeat path")
+    rk = torch.zeros(1, B, Hq, S, D, dtype=torch.float16, device=dev)
+    rv = torch.zeros(1, B, Hq, S, D, dtype=torch.float16, device=dev)
+    capi.kv_repeat(f_kc, f_vc, rk[0], rv[0], d_t)
+    # MHA over the repeated cache: q heads as they are, k/v heads repeated in the fused buffer too
+    qkv_r = torch.cat([d_qkv[:, :Hq], d_qkv[:, Hq:Hq + Hkv].repeat_interleave(G, 1),
+                       d_qkv[:, Hq + Hkv:].repeat_interleave(G, 1)], 1).contiguous()
+    b3 = d_bias.view(Hq + 2 * Hkv, D)
+    bias_r = torch.cat([b3[:Hq], b3[Hq:Hq + Hkv].repeat_interleave(G, 0), b3[Hq + Hkv:].repeat_interleave(G, 0)], 0).contiguous().view(-1)
+    out_r = torch.zeros_like(out_f)
+    capi.decode_attn(qkv_r, bias_r, rk, rv, out_r, Hq, int(t.max()), D, 10000.0, t_dev=d_t, max_t=int(t.max()))
+    np.testing.assert_allclose(out_r.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[np.float16])
+    # same rows, same arithmetic per row group => the two paths agree far inside the tolerance
+    assert (out_r.float() - out_f.float()).abs().max().item() <= 2e-3
+
+
+def test_constant_value_rows_at_full_size(capi, dev):
+    # size-independent property at config-2 size: if every V row (cache and new) equals c, out == c
+    announce("attn constant V")
+    torch.manual_seed(7)
+    B, H, D, S, t = 16, 32, 128, 4096, 4096
+    kc = torch.randn(1, B, H, S, D, device=dev).mul_(0.5).half()
+    vc = torch.full((1, B, H, S, D), 0.375, dtype=torch.float16, device=dev)
+    qkv = torch.randn(B, 3 * H, D, device=dev).mul_(0.5).half()
+    qkv[:, 2 * H:] = 0.375
+    out = torch.zeros(B, H * D, dtype=torch.float16, device=dev)
+    capi.decode_attn(qkv, None, kc, vc, out, H, t, D, 10000.0)
+    assert (out.float() - 0.375).abs().max().item() <= 1e-3

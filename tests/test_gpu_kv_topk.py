@@ -1,0 +1,165 @@
+"""GPU parity of KV concat, KV repeat and beam top-K against the CPU oracle (bit-exact), through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(a):
+    return a.view(np.uint16 if a.dtype == np.float16 else np.uint32)
+
+
+# ---------------------------------------------------------------- KV concat
+
+def test_append_reference_unit_vector(capi, dev):
+    announce("append unit vector")
+    ks = torch.ones(1, 2, 16, 8, device=dev)
+    kc = torch.full((1, 1, 2, 32, 8), -9.0, device=dev)
+    vc = torch.full((1, 1, 2, 32, 8), -9.0, device=dev)
+    capi.kv_append(ks, ks.clone(), kc, vc, torch.tensor([16], dtype=torch.int32, device=dev),
+                   torch.tensor([1], dtype=torch.int32, device=dev))
+    for c in (kc.cpu().numpy(), vc.cpu().numpy()):
+        np.testing.assert_array_equal(c[0, 0, :, 1:17], 1.0)
+        np.testing.assert_array_equal(c[0, 0, :, 0], -9.0)
+        np.testing.assert_array_equal(c[0, 0, :, 17:], -9.0)
+
+
+@pytest.mark.parametrize("dtype,D", [(np.float16, 128), (np.float32, 64), (np.float16, 12), (np.float32, 5)])
+@pytest.mark.parametrize("Q", [1, 7])
+def test_append_matches_oracle(capi, ref, dev, dtype, D, Q):
+    announce("append", dtype.__name__, D, Q)
+    rng = np.random.default_rng(3)
+    L, B, Hkv, S = 2, 5, 3, 40
+    ks = rng.standard_normal((B, Hkv, Q, D)).astype(dtype)
+    vs = rng.standard_normal((B, Hkv, Q, D)).astype(dtype)
+    kc = rng.standard_normal((L, B, Hkv, S, D)).astype(dtype)
+    vc = rng.standard_normal((L, B, Hkv, S, D)).astype(dtype)
+    cur = np.minimum(rng.integers(0, Q + 1, B), Q).astype(np.int32)
+    cur[0] = Q
+    hist = rng.integers(0, S - Q + 1, B).astype(np.int32)
+    hist[1] = S - 1          # spills over the end when cur > 1: those rows are dropped
+    d = [torch.from_numpy(a).to(dev) for a in (ks, vs, kc, vc, cur, hist)]
+    capi.kv_append(*d, layer=1)
+    ref.kv_append(ks, vs, kc, vc, cur, hist, layer=1)
+    np.testing.assert_array_equal(_bits(d[2].cpu().numpy()), _bits(kc))
+    np.testing.assert_array_equal(_bits(d[3].cpu().numpy()), _bits(vc))
+
+
+def test_append_decode_shape_of_gqa_config(capi, ref, dev):
+    # BASELINE config 3, the per-token concat: B32, Hkv8, D128, S8192, one new row per sequence
+    announce("append cfg3 decode")
+    torch.manual_seed(3)
+    B, Hkv, S, D = 32, 8, 8192, 128
+    kc = torch.zeros(1, B, Hkv, S, D, dtype=torch.float16, device=dev)
+    vc = torch.zeros(1, B, Hkv, S, D, dtype=torch.float16, device=dev)
+    ks = torch.randn(B, Hkv, 1, D, device=dev).mul(0.5).half()
+    vs = torch.randn(B, Hkv, 1, D, device=dev).mul(0.5).half()
+    hist = torch.randint(1023, 8191, (B,), dtype=torch.int32, device=dev)
+    capi.kv_append(ks, vs, kc, vc, torch.ones(B, dtype=torch.int32, device=dev), hist)
+    idx = hist.long()
+    got_k = kc[0, torch.arange(B, device=dev), :, idx]          # [B, Hkv, D]
+    got_v = vc[0, torch.arange(B, device=dev), :, idx]
+    assert torch.equal(got_k, ks[:, :, 0]) and torch.equal(got_v, vs[:, :, 0])
+    assert int(kc.count_nonzero().item()) == int(ks.count_nonzero().item())     # nothing else was written
+    assert int(vc.count_nonzero().item()) == int(vs.count_nonzero().item())
+
+
+# ---------------------------------------------------------------- KV repeat
+
+def test_repeat_reference_unit_vector(capi, dev):
+    announce("repeat unit vector")
+    src = torch.arange(32, dtype=torch.float32, device=dev).view(2, 1, 2, 4, 2)
+    kd = torch.full((1, 2, 2, 2), -1.0, device=dev)
+    vd = torch.full((1, 2, 2, 2), -1.0, device=dev)
+    capi.kv_repeat(src, src.clone(), kd, vd, torch.tensor([2], dtype=torch.int32, device=dev))
+    np.testing.assert_array_equal(kd.cpu().numpy().ravel(), [0, 1, 2, 3, 8, 9, 10, 11])
+    np.testing.assert_array_equal(vd.cpu().numpy().ravel(), [0, 1, 2, 3, 8, 9, 10, 11])
+
+
+@pytest.mark.parametrize("dtype,Hq,Hkv,D", [(np.float16, 32, 8, 128), (np.float32, 4, 4, 64), (np.float16, 6, 1, 12),
+                                            (np.float32, 8, 2, 3)])
+def test_repeat_matches_oracle(capi, ref, dev, dtype, Hq, Hkv, D):
+    announce("repeat", dtype.__name__, Hq, Hkv, D)
+    rng = np.random.default_rng(8)
+    L, B, S, MK = 2, 4, 50, 44
+    kc = rng.standard_normal((L, B, Hkv, S, D)).astype(dtype)
+    vc = rng.standard_normal((L, B, Hkv, S, D)).astype(dtype)
+    lens = np.array([44, 1, 49, 0], np.int32)      # 49 > max_k_len: clipped; 0: nothing written
+    kd = np.full((B, Hq, MK, D), 5.0, dtype)
+    vd = np.full((B, Hq, MK, D), 5.0, dtype)
+    d = [torch.from_numpy(a).to(dev) for a in (kc, vc, kd, vd, lens)]
+    capi.kv_repeat(*d, layer=1)
+    ref.kv_repeat(kc, vc, kd, vd, lens, layer=1)
+    np.testing.assert_array_equal(_bits(d[2].cpu().numpy()), _bits(kd))
+    np.testing.assert_array_equal(_bits(d[3].cpu().numpy()), _bits(vd))
+
+
+# ---------------------------------------------------------------- beam top-K
+
+def _lexsort_topk(flat_vals, flat_ids, K):
+    order = np.lexsort((flat_ids, -flat_vals.astype(np.float64)))[:K]
+    return flat_vals[order], flat_ids[order]
+
+
+def test_topk_reference_unit_vector(capi, dev):
+    announce("topk unit vector")
+    logits = torch.arange(60000, dtype=torch.float32, device=dev).view(2, 30000)
+    ws, _, _, fv, fi = capi.beam_topk(logits, 1, 2, 2)
+    np.testing.assert_array_equal(fi.cpu().numpy(), [[59999, 59998]])
+    np.testing.assert_array_equal(fv.cpu().numpy(), [[59999.0, 59998.0]])
+    # where the reference's unit test reads them: vals at 2*B*beam*8*beam, ids B*beam further
+    w = ws.cpu().numpy()
+    assert w[2 * 1 * 2 * 8 * 2] == 59999.0 and w.view(np.int32)[2 * 1 * 2 * 8 * 2 + 1 * 2] == 59999
+
+
+def test_topk_config5_planted_ties(capi, ref, dev):
+    announce("topk cfg5")
+    rng = np.random.default_rng(5)
+    B, beam, V, K = 8, 4, 32000, 4
+    logits = (rng.standard_normal((B * beam, V)) * 2.0).astype(np.float32)
+    for b in range(B):
+        top = logits[b * beam:(b + 1) * beam].max() + 1.0
+        for r in (b * beam, b * beam + 3):
+            logits[r, [17, 16000, 31999]] = top
+    _, v1, i1, fv, fi = capi.beam_topk(torch.from_numpy(logits).to(dev), B, beam, K)
+    w1v, w1i, wfv, wfi = ref.beam_topk(logits, B, beam, K)
+    np.testing.assert_array_equal(i1.cpu().numpy(), w1i)
+    np.testing.assert_array_equal(v1.cpu().numpy().view(np.uint32), w1v.view(np.uint32))
+    np.testing.assert_array_equal(fi.cpu().numpy(), wfi)
+    np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), wfv.view(np.uint32))
+    # and against numpy's lexsort directly
+    flat = logits.reshape(B, beam * V)
+    for b in range(B):
+        v, i = _lexsort_topk(flat[b], np.arange(beam * V) + b * beam * V, K)
+        np.testing.assert_array_equal(fi.cpu().numpy()[b], i)
+
+
+@pytest.mark.parametrize("B,beam,V,K", [(1, 1, 1, 1), (2, 3, 100, 8), (3, 2, 257, 5), (1, 4, 2049, 3), (5, 1, 50000, 2),
+                                        (2, 2, 128256, 4), (1, 1, 3, 8)])
+def test_topk_shapes_with_heavy_ties(capi, ref, dev, B, beam, V, K):
+    announce("topk", B, beam, V, K)
+    rng = np.random.default_rng(V + K)
+    # few distinct values => many ties, the order of equal values is what is being checked
+    logits = rng.integers(-3, 4, size=(B * beam, V)).astype(np.float32)
+    _, v1, i1, fv, fi = capi.beam_topk(torch.from_numpy(logits).to(dev), B, beam, K)
+    w1v, w1i, wfv, wfi = ref.beam_topk(logits, B, beam, K)
+    np.testing.assert_array_equal(i1.cpu().numpy(), w1i)
+    np.testing.assert_array_equal(fi.cpu().numpy(), wfi)
+    np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), wfv.view(np.uint32))
+
+
+def test_topk_negative_infinity_and_run_to_run(capi, ref, dev):
+    announce("topk -inf")
+    logits = np.full((2, 1000), -np.inf, np.float32)
+    logits[0, 500] = 1.0
+    d = torch.from_numpy(logits).to(dev)
+    _, _, _, fv, fi = capi.beam_topk(d, 1, 2, 4)
+    _, _, wfv, wfi = ref.beam_topk(logits, 1, 2, 4)
+    np.testing.assert_array_equal(fi.cpu().numpy(), wfi)
+    np.testing.assert_array_equal(fi.cpu().numpy(), [[500, 0, 1, 2]])
+    a = fi.clone()
+    _, _, _, _, fi2 = capi.beam_topk(d, 1, 2, 4)
+    assert torch.equal(a, fi2)

@@ -1,0 +1,135 @@
+"""GPU parity of RMSNorm and fused add-bias-residual-RMSNorm against the CPU oracle, through the C ABI.
+Tolerances: fp32 1e-5 relative; fp16 2e-3 absolute / 1e-2 relative; the updated residual is one
+fp32 add chain rounded once, so it is compared bit for bit."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.float32: dict(rtol=1e-5, atol=1e-6), np.float16: dict(rtol=1e-2, atol=2e-3)}
+TORCH = {np.float32: torch.float32, np.float16: torch.float16}
+
+
+def _inputs(N, H, dtype, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((N, H), dtype=np.float32).astype(dtype)
+    res = rng.standard_normal((N, H), dtype=np.float32).astype(dtype)
+    bias = rng.standard_normal(H, dtype=np.float32).astype(dtype)
+    gamma = rng.uniform(0.5, 1.5, H).astype(dtype)
+    return x, res, bias, gamma
+
+
+def test_rmsnorm_reference_unit_vector(capi, dev):
+    announce("rmsnorm unit vector 2x32")
+    x = torch.ones(2, 32, device=dev)
+    capi.rmsnorm(x, torch.ones(32, device=dev), 0.5)
+    np.testing.assert_allclose(x.cpu().numpy(), 1.0 / math.sqrt(1.5), rtol=1e-6)
+
+
+def test_fused_reference_unit_vector(capi, dev):
+    announce("fused norm unit vector 2x32")
+    out = torch.ones(2, 32, device=dev)
+    res = torch.zeros(2, 32, device=dev)
+    capi.fused_add_bias_residual_rmsnorm(res, out, torch.zeros(32, device=dev), torch.ones(32, device=dev), 0.5)
+    np.testing.assert_allclose(out.cpu().numpy(), 1.0 / math.sqrt(1.5), rtol=1e-6)
+    np.testing.assert_array_equal(res.cpu().numpy(), 1.0)
+
+
+SHAPES = [(16, 4096), (512, 4096), (8192, 4096), (8192, 8192),      # BASELINE config 4
+          (3, 32), (5, 100), (7, 4100), (2, 16384), (1, 40960), (2050, 1024), (4, 70000)]
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("N,H", SHAPES)
+def test_rmsnorm_matches_oracle(capi, ref, dev, dtype, N, H):
+    if N * H > 8192 * 4096 and dtype == np.float32:
+        pytest.skip("fp32 at this size adds nothing over fp16 + the smaller fp32 cases")
+    announce("rmsnorm", dtype.__name__, N, H)
+    x, _, _, gamma = _inputs(N, H, dtype, seed=4)
+    d_x = torch.from_numpy(x).to(dev)
+    capi.rmsnorm(d_x, torch.from_numpy(gamma).to(dev), 1e-5)
+    want = ref.rmsnorm(x.copy(), gamma, 1e-5)
+    np.testing.assert_allclose(d_x.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("with_bias", [True, False])
+@pytest.mark.parametrize("N,H", SHAPES)
+def test_fused_norm_matches_oracle(capi, ref, dev, dtype, with_bias, N, H):
+    if N * H > 8192 * 4096 and (dtype == np.float32 or not with_bias):
+        pytest.skip("largest shape is covered once, in fp16 with bias")
+    announce("fused_norm", dtype.__name__, "bias" if with_bias else "nobias", N, H)
+    out, res, bias, gamma = _inputs(N, H, dtype, seed=4)
+    if not with_bias:
+        bias = None
+    d_out, d_res = torch.from_numpy(out).to(dev), torch.from_numpy(res).to(dev)
+    d_bias = torch.from_numpy(bias).to(dev) if with_bias else None
+    capi.fused_add_bias_residual_rmsnorm(d_res, d_out, d_bias, torch.from_numpy(gamma).to(dev), 1e-5)
+    w_res, w_out = ref.fused_add_bias_residual_rmsnorm(res.copy(), out.copy(), bias, gamma, 1e-5)
+    itype = np.uint16 if dtype == np.float16 else np.uint32
+    np.testing.assert_array_equal(d_res.cpu().numpy().view(itype), w_res.view(itype))
+    np.testing.assert_allclose(d_out.cpu().numpy().astype(np.float64), w_out.astype(np.float64), **TOL[dtype])
+
+
+@pytest.mark.parametrize("tpr", [64, 256, 1024])
+def test_every_row_team_size_gives_the_same_answer(capi, ref, dev, tpr):
+    announce("norm team size", tpr)
+    x, res, bias, gamma = _inputs(33, 4096, np.float16, seed=9)
+    capi.tune_set("norm_tpr", tpr)
+    try:
+        d_x = torch.from_numpy(x).to(dev)
+        capi.rmsnorm(d_x, torch.from_numpy(gamma).to(dev), 1e-5)
+        d_out, d_res = torch.from_numpy(x).to(dev), torch.from_numpy(res).to(dev)
+        capi.fused_add_bias_residual_rmsnorm(d_res, d_out, torch.from_numpy(bias).to(dev), torch.from_numpy(gamma).to(dev), 1e-5)
+    finally:
+        capi.tune_set("norm_tpr", -1)
+    np.testing.assert_allclose(d_x.cpu().numpy().astype(np.float64), ref.rmsnorm(x.copy(), gamma, 1e-5).astype(np.float64),
+                               **TOL[np.float16])
+    w_res, w_out = ref.fused_add_bias_residual_rmsnorm(res.copy(), x.copy(), bias, gamma, 1e-5)
+    np.testing.assert_array_equal(d_res.cpu().numpy().view(np.uint16), w_res.view(np.uint16))
+    np.testing.assert_allclose(d_out.cpu().numpy().astype(np.float64), w_out.astype(np.float64), **TOL[np.float16])
+
+
+def test_unaligned_rows_take_the_scalar_path(capi, ref, dev):
+    announce("norm unaligned")
+    x, res, bias, gamma = _inputs(6, 1000, np.float16, seed=10)
+    # a view that starts 2 bytes into an allocation: not 16-byte aligned
+    buf = torch.zeros(6 * 1000 + 8, dtype=torch.float16, device=dev)
+    d_x = buf[1:1 + 6000].view(6, 1000)
+    d_x.copy_(torch.from_numpy(x))
+    capi.rmsnorm(d_x, torch.from_numpy(gamma).to(dev), 1e-5)
+    np.testing.assert_allclose(d_x.cpu().numpy().astype(np.float64), ref.rmsnorm(x.copy(), gamma, 1e-5).astype(np.float64),
+                               **TOL[np.float16])
+    assert buf[0].item() == 0 and buf[6001].item() == 0
+
+
+def test_empty_batch_is_a_no_op(capi, dev):
+    x = torch.zeros(0, 64, device=dev)
+    capi.rmsnorm(x, torch.ones(64, device=dev), 1e-5)
+    torch.cuda.synchronize()
+
+
+def test_full_size_properties(capi, dev):
+    # size-independent checks at 8192 x 8192 fp16: unit mean square with gamma = 1, and the fused
+    # kernel with zero residual and no bias reproducing the plain kernel bit for bit
+    announce("norm properties 8192x8192")
+    torch.manual_seed(4)
+    x = torch.randn(8192, 8192, device=dev, dtype=torch.float16)
+    g = torch.ones(8192, device=dev, dtype=torch.float16)
+    a = x.clone()
+    capi.rmsnorm(a, g, 0.0)
+    ms = a.float().pow(2).mean(dim=1)
+    assert (ms - 1.0).abs().max().item() < 2e-3
+    b = x.clone()
+    r = torch.zeros_like(x)
+    capi.fused_add_bias_residual_rmsnorm(r, b, None, g, 0.0)
+    assert torch.equal(a, b)
+    assert torch.equal(r, x)
+    c = x.clone()
+    capi.rmsnorm(c, g, 0.0)
+    assert torch.equal(a, c)          # run-to-run determinism
