@@ -1,0 +1,187 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A step is one fused decode-attention call at the Llama-2-7B shape (batch 16, 32 heads x 128, fp16 KV
+cache, context 4096): bias + RoPE + cache write + softmax + V sum for one new token per sequence.
+Inputs are synthetic, resident in HBM before the timed region, and each step uses the next of several
+distinct cache sets so that the 256 MB Infinity Cache cannot serve the stream.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X, published
+
+
+def attn_bytes(B, Hq, Hkv, D, t_list, e):
+    """Algorithmic bytes of one decode step: history K+V read once, new row written, qkv + bias read, out written."""
+    hist = sum(2 * Hkv * (t - 1) * D * e for t in t_list)
+    return hist + 2 * B * Hkv * D * e + B * (Hq + 2 * Hkv) * D * e + (Hq + 2 * Hkv) * D * e + B * Hq * D * e
+
+
+def time_steps(fn, steps, warmup):
+    """fn(i) launches step i on torch's current stream; returns average ms per step measured with HIP events
+    recorded on that same stream."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn(i)
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=None):
+    import torch
+    torch.manual_seed(2)
+    sets = []
+    for _ in range(nsets):
+        kc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+        vc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+        sets.append((kc, vc))
+    qkv = torch.randn(B, Hq + 2 * Hkv, D, device=dev).mul_(0.5).half()
+    bias = torch.randn((Hq + 2 * Hkv) * D, device=dev).mul_(0.5).half()
+    out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+    max_t = t if t_dev is None else int(t_dev.max().item())
+    ws = torch.empty(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, max_t), dtype=torch.uint8, device=dev)
+
+    def step(i):
+        kc, vc = sets[i % nsets]
+        capi.decode_attn(qkv, bias, kc, vc, out, Hq, max_t, D, 10000.0, t_dev=t_dev, max_t=max_t, workspace=ws)
+
+    ms = time_steps(step, steps, warmup)
+    return ms, (qkv, bias, sets[0], out)
+
+
+def bench_norms(capi, dev, steps, warmup, N, H, fused):
+    import torch
+    torch.manual_seed(4)
+    nsets = max(3, int(1.2e9 // (N * H * 2 * (2 if fused else 1))) if N * H * 2 < 4e8 else 3)
+    nsets = min(nsets, 64)
+    xs = [torch.randn(N, H, device=dev).half() for _ in range(nsets)]
+    rs = [torch.randn(N, H, device=dev).half() for _ in range(nsets)] if fused else None
+    g = torch.rand(H, device=dev).add_(0.5).half()
+    b = torch.randn(H, device=dev).half()
+
+    def step(i):
+        if fused:
+            capi.fused_add_bias_residual_rmsnorm(rs[i % nsets], xs[i % nsets], b, g, 1e-5)
+        else:
+            capi.rmsnorm(xs[i % nsets], g, 1e-5)
+
+    ms = time_steps(step, steps, warmup)
+    nbytes = (4 * N * H * 2 + 2 * H * 2) if fused else (2 * N * H * 2 + H * 2)
+    return ms, nbytes
+
+
+def cpu_baseline_attention(qkv, bias, kc, vc, Hq, t, D):
+    """The CPU oracle (a port of the reference semantics, OpenMP over (sequence, kv-head)) on the same
+    inputs, on this host's cores.  Checker used as a reported baseline only."""
+    import numpy as np
+    from oracle import ref
+    ref.build()
+    h_qkv, h_bias = qkv.cpu().numpy(), bias.cpu().numpy()
+    h_kc, h_vc = kc.cpu().numpy(), vc.cpu().numpy()
+    cores = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
+    cores = min(cores, os.cpu_count() or cores)
+    times = []
+    budget = time.time() + 25.0
+    for _ in range(5):
+        t0 = time.time()
+        ref.decode_attn(h_qkv, h_bias, h_kc, h_vc, Hq, t, D, 10000.0)
+        times.append(time.time() - t0)
+        if time.time() + times[-1] > budget:
+            break
+    times.sort()
+    return {"value": round(times[len(times) // 2] * 1e6, 1), "unit": "us/step", "cores": cores, "kind": "port",
+            "sample": "the full batch-16 ctx-4096 step (1.07 GB of fp16 KV), median of %d runs, OpenMP over "
+                      "(sequence, kv-head)" % len(times)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--ctx", type=int, default=4096)
+    ap.add_argument("--no-extras", action="store_true", help="skip the context sweep, GQA, norm and top-K lines")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); --gpus %d is not supported" % args.gpus)
+
+    import torch
+    from onellm_amd import capi
+    capi.lib()                      # raises if the HIP library is not built: there is no fallback
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    B, H, D, S, t = 16, 32, 128, 4096, args.ctx
+    ms, (qkv, bias, (kc, vc), out) = bench_attention(capi, dev, args.steps, args.warmup, B, H, H, D, S, t, nsets=4)
+    nbytes = attn_bytes(B, H, H, D, [t] * B, 2)
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    line = {
+        "metric": "decode-attn us/step at Llama-2-7B shape, ctx %d (fused masked MHA: qkv bias + RoPE + KV-cache write + softmax + V sum)" % t,
+        "value": round(ms * 1e3, 2), "unit": "us/step", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: batch 16, 32 heads x 128, MHA, fp16 KV cache [1,16,32,4096,128], ctx %d, "
+                               "RoPE base 10000; 4 cache sets rotated per step" % t,
+                   "storage": "fp16", "arithmetic": "fp32"},
+        "hbm_gbps": round(gbps, 1), "hbm_frac_of_8TBps": round(gbps / HBM_PEAK_GBPS, 4),
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "decode_attn_split_kernel<__half,16,1,4,4>",
+                     "algorithmic_bytes_per_launch": nbytes,
+                     "note": "duration = HIP-event time of the whole step (split kernel + merge kernel) / steps"},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_attention(qkv, bias, kc, vc, H, t, D)
+
+    if not args.no_extras:
+        extras = {}
+        for c in (512, 1024, 2048):
+            m, _ = bench_attention(capi, dev, args.steps, args.warmup, B, H, H, D, S, c, nsets=4)
+            nb = attn_bytes(B, H, H, D, [c] * B, 2)
+            extras["decode_attn_ctx%d" % c] = {"us": round(m * 1e3, 2), "gbps": round(nb / m / 1e6, 1),
+                                               "frac": round(nb / m / 1e6 / HBM_PEAK_GBPS, 4)}
+        del kc, vc
+        torch.cuda.empty_cache()
+        # BASELINE configs[2]: fused grouped-query read, ragged lengths
+        import numpy as np
+        tl = np.random.default_rng(3).integers(1024, 8193, size=32).astype(np.int32)
+        m, _ = bench_attention(capi, dev, max(args.steps // 3, 10), args.warmup, 32, 32, 8, 128, 8192, 8192, nsets=3,
+                               t_dev=torch.from_numpy(tl).to(dev))
+        nb = attn_bytes(32, 32, 8, 128, tl.tolist(), 2)
+        extras["decode_attn_gqa_b32_q32_kv8_len1024-8192"] = {"us": round(m * 1e3, 2), "gbps": round(nb / m / 1e6, 1),
+                                                             "frac": round(nb / m / 1e6 / HBM_PEAK_GBPS, 4)}
+        torch.cuda.empty_cache()
+        for (N, Hd) in ((16, 4096), (512, 4096), (8192, 4096), (8192, 8192)):
+            for fused in (False, True):
+                m, nb = bench_norms(capi, dev, args.steps, args.warmup, N, Hd, fused)
+                extras["%s_%dx%d" % ("fused_norm" if fused else "rmsnorm", N, Hd)] = {
+                    "us": round(m * 1e3, 2), "gbps": round(nb / m / 1e6, 1), "frac": round(nb / m / 1e6 / HBM_PEAK_GBPS, 4)}
+            torch.cuda.empty_cache()
+        logits = torch.randn(32, 32000, device=dev).mul_(2.0)
+        wsk = torch.empty(capi.beam_topk_workspace_bytes(8, 4, 4) // 4, dtype=torch.float32, device=dev)
+        m = time_steps(lambda i: capi.beam_topk(logits, 8, 4, 4, workspace=wsk), args.steps, args.warmup)
+        extras["beam_topk_b8_beam4_v32000_k4"] = {"us": round(m * 1e3, 2), "gbps": round(4096000 / m / 1e6, 1)}
+        line["extras"] = extras
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -217,8 +217,8 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
                 valid[u] = row < r1;
                 row = min(row, r1 - 1);
             }
-            kv[u] = load16(kp + (size_t)row * D);
-            vv[u] = load16(vp + (size_t)row * D);
+            kv[u] = load16_stream(kp + (size_t)row * D);
+            vv[u] = load16_stream(vp + (size_t)row * D);
         }
         float s[GT][U];
 #pragma unroll
@@ -332,30 +332,45 @@ void decode_attn_merge_kernel(const AttnArgs a, int D)
     }
 }
 
-constexpr int kNW = 4;              // waves per workgroup
 constexpr int kMaxSplits = 64;      // upper bound of splits the workspace is sized for
 constexpr int kMinChunk = 64;       // never split finer than this many cache rows
 
-template <typename T, int LPR, int GT>
+template <typename T, int LPR, int GT, int U, int NW>
 int launch_split(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
-    constexpr int U = GT >= 4 ? 2 : 4;
     constexpr int D = LPR * Elt<T>::kVec;
-    constexpr int NRG = kNW * (kWave / LPR);
+    constexpr int NRG = NW * (kWave / LPR);
     const size_t lds_bytes = sizeof(float) * (size_t)(GT * D + 2 * D + GT + NRG * GT * 2 + (size_t)NRG * GT * D);
     if (lds_bytes > 64 * 1024) return ONELLM_EUNSUPPORTED;
     const int ngt = (a.G + GT - 1) / GT;
-    const dim3 grid(a.nsplit, a.Hkv * ngt, a.B), block(kNW * kWave);
-    hipLaunchKernelGGL((decode_attn_split_kernel<T, LPR, GT, U, kNW>), grid, block, lds_bytes, st, a, fr);
+    const dim3 grid(a.nsplit, a.Hkv * ngt, a.B), block(NW * kWave);
+    hipLaunchKernelGGL((decode_attn_split_kernel<T, LPR, GT, U, NW>), grid, block, lds_bytes, st, a, fr);
     return launch_status();
+}
+
+template <typename T, int LPR, int GT>
+int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    constexpr int U0 = GT >= 4 ? 2 : 4;
+    if constexpr (LPR == 16 && GT == 1) {
+        const int u = tune_get("attn_unroll"), nw = tune_get("attn_waves");
+        if (nw == 8 && u == 8) return launch_split<T, LPR, GT, 8, 8>(a, fr, st);
+        if (nw == 8) return launch_split<T, LPR, GT, 4, 8>(a, fr, st);
+        if (nw == 16 && u == 2) return launch_split<T, LPR, GT, 2, 16>(a, fr, st);
+        if (nw == 16) return launch_split<T, LPR, GT, 4, 16>(a, fr, st);
+        if (nw == 2) return launch_split<T, LPR, GT, 8, 2>(a, fr, st);
+        if (u == 8) return launch_split<T, LPR, GT, 8, 4>(a, fr, st);
+        if (u == 2) return launch_split<T, LPR, GT, 2, 4>(a, fr, st);
+    }
+    return launch_split<T, LPR, GT, U0, 4>(a, fr, st);
 }
 
 template <typename T, int LPR>
 int launch_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
-    if (a.G == 1) return launch_split<T, LPR, 1>(a, fr, st);
-    if (a.G == 2) return launch_split<T, LPR, 2>(a, fr, st);
-    return launch_split<T, LPR, 4>(a, fr, st);
+    if (a.G == 1) return launch_shape<T, LPR, 1>(a, fr, st);
+    if (a.G == 2) return launch_shape<T, LPR, 2>(a, fr, st);
+    return launch_shape<T, LPR, 4>(a, fr, st);
 }
 
 template <typename T>
@@ -418,13 +433,14 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     a.qscale = (1.0f / sqrtf((float)D)) * 1.4426950408889634f;
     a.slab = (size_t)layer * B * Hkv * (size_t)S * D;
 
-    // sequence split: enough workgroups to cover the chip several times over, chunks not below kMinChunk
+    // sequence split: about two workgroups (eight waves) per compute unit measured best on MI355X —
+    // long contiguous streams per workgroup, and with one split there is no merge pass at all
     const int G = a.G;
     const int gt = G == 1 ? 1 : (G == 2 ? 2 : 4);
     const int ngt = (G + gt - 1) / gt;
     const long base_wgs = (long)B * Hkv * ngt;
     int target = tune_get("attn_target_wgs");
-    if (target <= 0) target = 2048;
+    if (target <= 0) target = 512;
     int nsplit = (int)((target + base_wgs - 1) / base_wgs);
     const int cap = max_splits(max_t);
     if (nsplit > cap) nsplit = cap;

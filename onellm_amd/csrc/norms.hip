@@ -50,14 +50,14 @@ void norm_rows_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         const int idx = lane + j * TPR;
-        if (idx < nvec) x[j] = load16(orow + idx * VEC);
+        if (idx < nvec) x[j] = load16_stream(orow + idx * VEC);
     }
     if constexpr (FUSED) {
         Vec16<T> y[NV];
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int idx = lane + j * TPR;
-            if (idx < nvec) y[j] = load16(rrow + idx * VEC);
+            if (idx < nvec) y[j] = load16_stream(rrow + idx * VEC);
         }
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
@@ -73,7 +73,7 @@ void norm_rows_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __
                     y[j].set(e, v);
                     ss = fmaf(v, v, ss);
                 }
-                store16(rrow + idx * VEC, y[j]);
+                store16_stream(rrow + idx * VEC, y[j]);
             }
         }
     } else {
@@ -98,7 +98,7 @@ void norm_rows_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __
             const Vec16<T> g = load16(gamma + idx * VEC);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) x[j].set(e, g.get(e) * r[j][e] * inv);
-            store16(orow + idx * VEC, x[j]);
+            store16_stream(orow + idx * VEC, x[j]);
         }
     }
 }
