@@ -21,6 +21,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 LIB_HIP = os.path.join(HERE, "libonellm_hip.so")
 LIB_LAUNCH = os.path.join(HERE, "libonellm_launchers.so")
+# test-only: a C wrapper that drives the launcher shims with oneLLM-style Tensor objects
+HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "launcher_harness.cpp")
+LIB_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
 
 KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "tuning.cpp"]
 LAUNCHER_SOURCES = ["launchers.cpp"]
@@ -53,8 +56,6 @@ def _compile(src, force):
     cmd = [HIPCC, "-c", path, "-o", obj] + COMMON
     if src.endswith(".hip"):
         cmd += DEVICE
-    else:
-        cmd += ["-x", "hip", "--offload-arch=gfx950"] if False else []
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr[-4000:]))
@@ -73,6 +74,12 @@ def build(force=False, verbose=False):
         cmd = [HIPCC, "-shared", "-fPIC", "-o", LIB_LAUNCH] + lobjs + \
               ["-L" + HERE, "-lonellm_hip", "-Wl,-rpath,$ORIGIN"]
         subprocess.run(cmd, check=True, capture_output=not verbose)
+    if os.path.exists(HARNESS_SRC) and (force or _newer(LIB_HARNESS, [HARNESS_SRC, LIB_LAUNCH] + _headers())):
+        cmd = [HIPCC, "-shared", "-fPIC", "-O2", "-std=c++17", "-I" + INCLUDE, HARNESS_SRC, "-o", LIB_HARNESS,
+               "-L" + HERE, "-lonellm_launchers", "-lonellm_hip", "-Wl,-rpath,$ORIGIN/../../onellm_amd"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for the launcher harness:\n" + r.stderr[-4000:])
     return LIB_HIP, LIB_LAUNCH
 
 

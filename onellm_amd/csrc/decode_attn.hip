@@ -5,7 +5,7 @@
 // K and V history is read exactly once: 2*Hkv*(t-1)*D*e bytes per sequence), so the design is
 // about bytes in flight, not matrix cores:
 //
-//   * split over the sequence ("flash-decoding"): grid = (splits, kv-head x head-tile, batch); each
+//   * split over the sequence ("flash-decoding"): grid = (kv-head x head-tile, splits, batch); each
 //     workgroup streams one contiguous chunk of cache rows of one (sequence, kv-head) and keeps an
 //     online-softmax state (running max m, sum l, weighted V accumulator) per query head;
 //   * grouped-query heads are fused on the read side: a workgroup applies every K/V row it loads to
@@ -107,11 +107,15 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    const int split = blockIdx.x;
+    // Workgroups are dealt to the 8 XCDs round-robin in linear block order.  The kv-head index is
+    // the fastest grid dimension so that every XCD sees the same mix of sequences and splits, and
+    // the split index is rotated by the sequence index so that, with ragged lengths, the splits
+    // every sequence has (the low ones) do not all land on the same XCDs.
     const int ngt = (a.G + GT - 1) / GT;
-    const int kvh = blockIdx.y / ngt;
-    const int g0 = (blockIdx.y % ngt) * GT;
+    const int kvh = blockIdx.x / ngt;
+    const int g0 = (blockIdx.x % ngt) * GT;
     const int b = blockIdx.z;
+    const int split = (blockIdx.y + b) % a.nsplit;
 
     const int t = a.t_dev ? a.t_dev[b] : a.t_host;
     if (t < 1 || t > a.S) return;               // out-of-contract length: touch nothing
@@ -206,20 +210,19 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     const T* kp = kc + col;
     const T* vp = vc + col;
 
-    auto body = [&](int rbase, auto masked_tag) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
-        Vec16<T> kv[U], vv[U];
-        bool valid[U];
+    // loads of one iteration: U cache rows of K and of V per row group
+    auto issue = [&](Vec16<T> (&kv)[U], Vec16<T> (&vv)[U], int rbase) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            int row = rbase + u * NRG + rg;
-            if constexpr (MASKED) {
-                valid[u] = row < r1;
-                row = min(row, r1 - 1);
-            }
+            const int row = rbase + u * NRG + rg;
             kv[u] = load16_stream(kp + (size_t)row * D);
             vv[u] = load16_stream(vp + (size_t)row * D);
         }
+    };
+    // scores, online softmax and weighted V sum for the rows held in (kv, vv); `valid` masks rows
+    // past the end of the chunk in the tail iteration
+    auto consume = [&](const Vec16<T> (&kv)[U], const Vec16<T> (&vv)[U], const bool (&valid)[U], auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
         float s[GT][U];
 #pragma unroll
         for (int g = 0; g < GT; ++g)
@@ -260,10 +263,36 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     };
 
     if (r1 > r0) {
+        // Full iterations are software-pipelined over two register buffers: the loads of the next
+        // iteration are in flight while the current one is consumed, so a wave never sits with an
+        // empty memory queue.  The (at most one) partial iteration at the end is masked.
         const int nfull = (r1 - r0) / RPI;
+        const bool none[U] = {};
+        Vec16<T> ka[U], va[U], kb[U], vb[U];
         int rbase = r0;
-        for (int it = 0; it < nfull; ++it, rbase += RPI) body(rbase, std::false_type{});
-        if (rbase < r1) body(rbase, std::true_type{});
+        if (nfull > 0) issue(ka, va, rbase);
+        for (int it = 0; it < nfull; it += 2) {
+            if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
+            consume(ka, va, none, std::false_type{});
+            if (it + 1 < nfull) {
+                if (it + 2 < nfull) issue(ka, va, rbase + 2 * RPI);
+                consume(kb, vb, none, std::false_type{});
+            }
+            rbase += 2 * RPI;
+        }
+        rbase = r0 + nfull * RPI;
+        if (rbase < r1) {
+            bool valid[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                int row = rbase + u * NRG + rg;
+                valid[u] = row < r1;
+                row = min(row, r1 - 1);
+                ka[u] = load16_stream(kp + (size_t)row * D);
+                va[u] = load16_stream(vp + (size_t)row * D);
+            }
+            consume(ka, va, valid, std::true_type{});
+        }
     }
 
     // ---- merge the row-group states of the workgroup
@@ -343,7 +372,7 @@ int launch_split(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     const size_t lds_bytes = sizeof(float) * (size_t)(GT * D + 2 * D + GT + NRG * GT * 2 + (size_t)NRG * GT * D);
     if (lds_bytes > 64 * 1024) return ONELLM_EUNSUPPORTED;
     const int ngt = (a.G + GT - 1) / GT;
-    const dim3 grid(a.nsplit, a.Hkv * ngt, a.B), block(NW * kWave);
+    const dim3 grid(a.Hkv * ngt, a.nsplit, a.B), block(NW * kWave);
     hipLaunchKernelGGL((decode_attn_split_kernel<T, LPR, GT, U, NW>), grid, block, lds_bytes, st, a, fr);
     return launch_status();
 }
@@ -351,18 +380,9 @@ int launch_split(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 template <typename T, int LPR, int GT>
 int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
-    constexpr int U0 = GT >= 4 ? 2 : 4;
-    if constexpr (LPR == 16 && GT == 1) {
-        const int u = tune_get("attn_unroll"), nw = tune_get("attn_waves");
-        if (nw == 8 && u == 8) return launch_split<T, LPR, GT, 8, 8>(a, fr, st);
-        if (nw == 8) return launch_split<T, LPR, GT, 4, 8>(a, fr, st);
-        if (nw == 16 && u == 2) return launch_split<T, LPR, GT, 2, 16>(a, fr, st);
-        if (nw == 16) return launch_split<T, LPR, GT, 4, 16>(a, fr, st);
-        if (nw == 2) return launch_split<T, LPR, GT, 8, 2>(a, fr, st);
-        if (u == 8) return launch_split<T, LPR, GT, 8, 4>(a, fr, st);
-        if (u == 2) return launch_split<T, LPR, GT, 2, 4>(a, fr, st);
-    }
-    return launch_split<T, LPR, GT, U0, 4>(a, fr, st);
+    // 4 waves per workgroup and 4 cache rows per row group and iteration measured best on MI355X for
+    // both the single-head and the grouped-query form (8 or 16 waves, 2 or 8 rows: 3-30 % slower).
+    return launch_split<T, LPR, GT, 4, 4>(a, fr, st);
 }
 
 template <typename T, int LPR>
@@ -433,20 +453,23 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     a.qscale = (1.0f / sqrtf((float)D)) * 1.4426950408889634f;
     a.slab = (size_t)layer * B * Hkv * (size_t)S * D;
 
-    // sequence split: about two workgroups (eight waves) per compute unit measured best on MI355X —
-    // long contiguous streams per workgroup, and with one split there is no merge pass at all
+    // Sequence split.  Equal lengths (t_dev == NULL): about two workgroups (eight waves) per compute
+    // unit measured best on MI355X — long contiguous streams per workgroup, and with a single split
+    // there is no merge pass at all.  Per-sequence lengths: finer chunks (about 16 workgroups per
+    // compute unit, chunks of at least 256 rows) so that the dispatcher can balance ragged work.
     const int G = a.G;
     const int gt = G == 1 ? 1 : (G == 2 ? 2 : 4);
     const int ngt = (G + gt - 1) / gt;
     const long base_wgs = (long)B * Hkv * ngt;
     int target = tune_get("attn_target_wgs");
-    if (target <= 0) target = 512;
+    if (target <= 0) target = t_dev ? 4096 : 512;
     int nsplit = (int)((target + base_wgs - 1) / base_wgs);
-    const int cap = max_splits(max_t);
+    int cap = max_splits(max_t);
+    if (t_dev && tune_get("attn_target_wgs") <= 0) cap = (max_t + 255) / 256 < cap ? (max_t + 255) / 256 : cap;
     if (nsplit > cap) nsplit = cap;
     if (nsplit < 1) nsplit = 1;
     const int forced = tune_get("attn_nsplit");
-    if (forced > 0) nsplit = forced > cap ? cap : forced;
+    if (forced > 0) nsplit = forced > max_splits(max_t) ? max_splits(max_t) : forced;
     int chunk = (max_t + nsplit - 1) / nsplit;
     chunk = (chunk + kMinChunk - 1) / kMinChunk * kMinChunk;
     nsplit = (max_t + chunk - 1) / chunk;

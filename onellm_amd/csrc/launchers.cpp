@@ -91,13 +91,21 @@ void launchDecoderMaskedMHA(Tensor* qkv_buf, BaseWeight& qkv, Tensor* k_cache, T
     const int head_num = qkv_head_num - 2 * kv_head_num;   // :292
     const int cur_step = *(const int*)step->data;      // :294
     ONELLM_CHECK_WITH_INFO(cs.B == batch_size && cs.D == head_size, "KV cache does not match qkv_buf");
-    const size_t ws_bytes = onellm_decode_attn_workspace_bytes(batch_size, head_num, kv_head_num, head_size, cur_step);
-    void* ws = g_attn_ws.get(ws_bytes);
-    const int rc = onellm_decode_attn(dtype, qkv_buf->data, qkv.bias, k_cache->data, v_cache->data, mha_output->data,
-                                      batch_size, head_num, kv_head_num, head_size, cs.S, /*layer=*/0, cs.layers,
-                                      cur_step, nullptr, cur_step,
-                                      static_params.rotary_embedding_dim, static_params.rotary_embedding_base,
-                                      /*rope_pos_offset=*/0, /*flags=*/0u, ws, ws_bytes, nullptr);
+    ONELLM_CHECK_WITH_INFO(head_num > 0 && cur_step >= 1 && cur_step <= cs.S, "step outside [1, max_seq_len]");
+    // Most shapes need no scratch (a single sequence split); the buffer is only created when the
+    // entry point asks for one.
+    auto call = [&](void* ws, size_t ws_bytes) {
+        return onellm_decode_attn(dtype, qkv_buf->data, qkv.bias, k_cache->data, v_cache->data, mha_output->data,
+                                  batch_size, head_num, kv_head_num, head_size, cs.S, /*layer=*/0, cs.layers,
+                                  cur_step, nullptr, cur_step,
+                                  static_params.rotary_embedding_dim, static_params.rotary_embedding_base,
+                                  /*rope_pos_offset=*/0, /*flags=*/0u, ws, ws_bytes, nullptr);
+    };
+    int rc = call(nullptr, 0);
+    if (rc == ONELLM_EWORKSPACE) {
+        const size_t ws_bytes = onellm_decode_attn_workspace_bytes(batch_size, head_num, kv_head_num, head_size, cur_step);
+        rc = call(g_attn_ws.get(ws_bytes), ws_bytes);
+    }
     throw_on_error(rc, "launchDecoderMaskedMHA");
 }
 

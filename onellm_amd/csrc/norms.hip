@@ -10,95 +10,149 @@
 namespace onellm {
 namespace {
 
-template <int TPR>
-__device__ __forceinline__ float row_sum(float v, float* smem, int tid)
+// Sums over the TPR threads that share a row, for RPT rows at once; smem holds RPT floats per
+// wave of the block.  Teams of a block reach the barrier together (callers keep whole blocks alive).
+template <int TPR, int RPT>
+__device__ __forceinline__ void row_sums(float (&v)[RPT], float* smem, int tid)
 {
-    v = wave_sum(v);
+#pragma unroll
+    for (int k = 0; k < RPT; ++k) v[k] = wave_sum(v[k]);
     if constexpr (TPR > kWave) {
         constexpr int NWAVE = TPR / kWave;
-        if ((tid & (kWave - 1)) == 0) smem[tid / kWave] = v;
-        __syncthreads();
-        float s = 0.f;
+        const int wave = tid / kWave;
+        if ((tid & (kWave - 1)) == 0) {
 #pragma unroll
-        for (int w = 0; w < NWAVE; ++w) s += smem[w];
-        v = s;
+            for (int k = 0; k < RPT; ++k) smem[wave * RPT + k] = v[k];
+        }
+        __syncthreads();
+        const int first = wave / NWAVE * NWAVE;
+#pragma unroll
+        for (int k = 0; k < RPT; ++k) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < NWAVE; ++w) s += smem[(first + w) * RPT + k];
+            v[k] = s;
+        }
     }
-    return v;
 }
 
-// residual == nullptr-free: FUSED selects the add-bias-residual form at compile time.
-template <typename T, int NV, int TPR, bool FUSED>
+// A team of TPR threads owns RPT rows at a time and each thread holds NV 16-byte vectors of each:
+// all RPT*NV loads (twice that when FUSED) are issued before anything is consumed, so a thread
+// keeps up to 8 KiB-per-wave-sized bursts in flight; then one reduction serves the RPT rows.
+// FUSED selects the add-bias-residual form at compile time.
+template <typename T, int NV, int TPR, int RPT, bool FUSED>
 __global__ __launch_bounds__(TPR > 256 ? TPR : 256)
 void norm_rows_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __restrict__ bias,
                       const T* __restrict__ gamma, float eps, int N, int H)
 {
     constexpr int VEC = Elt<T>::kVec;
     constexpr int BLOCK = TPR > 256 ? TPR : 256;
-    constexpr int RPB = BLOCK / TPR;
-    __shared__ float smem[TPR > kWave ? TPR / kWave : 1];
+    constexpr int TPB = BLOCK / TPR;             // teams per block
+    __shared__ float smem[BLOCK / kWave * RPT];
     const int tid = threadIdx.x;
-    const int row = blockIdx.x * RPB + tid / TPR;
     const int lane = tid % TPR;
-    if (row >= N) return;   // whole row-teams leave together; TPR > 64 means one team per block
+    const int row0 = (blockIdx.x * TPB + tid / TPR) * RPT;
+    // one wave per team: a wave past the end simply leaves (no barrier is ever used);
+    // several waves per team: every team stays for the barrier, rows past the end are empty
+    if (TPR <= kWave && row0 >= N) return;
     const int nvec = H / VEC;
-    T* orow = out + (size_t)row * H;
-    T* rrow = FUSED ? residual + (size_t)row * H : nullptr;
 
-    Vec16<T> x[NV];
-    float r[NV][VEC];
-    float ss = 0.f;
+    Vec16<T> x[RPT][NV];
+    float ss[RPT];
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        const int idx = lane + j * TPR;
-        if (idx < nvec) x[j] = load16_stream(orow + idx * VEC);
-    }
-    if constexpr (FUSED) {
-        Vec16<T> y[NV];
+    for (int k = 0; k < RPT; ++k) {
+        ss[k] = 0.f;
+        const bool live = row0 + k < N;
+        const T* orow = out + (size_t)(live ? row0 + k : 0) * H;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int idx = lane + j * TPR;
-            if (idx < nvec) y[j] = load16_stream(rrow + idx * VEC);
+            if (live && idx < nvec) x[k][j] = load16_stream(orow + idx * VEC);
         }
+    }
+    if constexpr (FUSED) {
+        // r = (out + residual) + bias is kept in fp32 in place of the raw inputs
+        float r[RPT][NV][VEC];
+        {
+            Vec16<T> y[RPT][NV];
+#pragma unroll
+            for (int k = 0; k < RPT; ++k) {
+                const bool live = row0 + k < N;
+                const T* rrow = residual + (size_t)(live ? row0 + k : 0) * H;
+#pragma unroll
+                for (int j = 0; j < NV; ++j) {
+                    const int idx = lane + j * TPR;
+                    if (live && idx < nvec) y[k][j] = load16_stream(rrow + idx * VEC);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NV; ++j) {
+                const int idx = lane + j * TPR;
+                Vec16<T> b;
+                if (bias && idx < nvec) b = load16(bias + idx * VEC);
+#pragma unroll
+                for (int k = 0; k < RPT; ++k) {
+                    if (row0 + k < N && idx < nvec) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) {
+                            float v = x[k][j].get(e) + y[k][j].get(e);        // (out + residual) + bias, in this order
+                            if (bias) v += b.get(e);
+                            r[k][j][e] = v;
+                            y[k][j].set(e, v);
+                            ss[k] = fmaf(v, v, ss[k]);
+                        }
+                        store16_stream(residual + (size_t)(row0 + k) * H + idx * VEC, y[k][j]);
+                    }
+                }
+            }
+        }
+        row_sums<TPR, RPT>(ss, smem, tid);
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int idx = lane + j * TPR;
             if (idx < nvec) {
-                Vec16<T> b;
-                if (bias) b = load16(bias + idx * VEC);
+                const Vec16<T> g = load16(gamma + idx * VEC);
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    float v = x[j].get(e) + y[j].get(e);        // (out + residual) + bias, in this order
-                    if (bias) v += b.get(e);
-                    r[j][e] = v;
-                    y[j].set(e, v);
-                    ss = fmaf(v, v, ss);
+                for (int k = 0; k < RPT; ++k) {
+                    if (row0 + k < N) {
+                        const float inv = rsqrtf(ss[k] / (float)H + eps);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) x[k][j].set(e, g.get(e) * r[k][j][e] * inv);
+                        store16_stream(out + (size_t)(row0 + k) * H + idx * VEC, x[k][j]);
+                    }
                 }
-                store16_stream(rrow + idx * VEC, y[j]);
             }
         }
     } else {
 #pragma unroll
+        for (int k = 0; k < RPT; ++k)
+#pragma unroll
+            for (int j = 0; j < NV; ++j) {
+                const int idx = lane + j * TPR;
+                if (row0 + k < N && idx < nvec) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const float v = x[k][j].get(e);
+                        ss[k] = fmaf(v, v, ss[k]);
+                    }
+                }
+            }
+        row_sums<TPR, RPT>(ss, smem, tid);
+#pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int idx = lane + j * TPR;
             if (idx < nvec) {
+                const Vec16<T> g = load16(gamma + idx * VEC);
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    r[j][e] = x[j].get(e);
-                    ss = fmaf(r[j][e], r[j][e], ss);
+                for (int k = 0; k < RPT; ++k) {
+                    if (row0 + k < N) {
+                        const float inv = rsqrtf(ss[k] / (float)H + eps);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) x[k][j].set(e, g.get(e) * x[k][j].get(e) * inv);
+                        store16_stream(out + (size_t)(row0 + k) * H + idx * VEC, x[k][j]);
+                    }
                 }
             }
-        }
-    }
-    ss = row_sum<TPR>(ss, smem, tid);
-    const float inv = rsqrtf(ss / (float)H + eps);
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        const int idx = lane + j * TPR;
-        if (idx < nvec) {
-            const Vec16<T> g = load16(gamma + idx * VEC);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) x[j].set(e, g.get(e) * r[j][e] * inv);
-            store16_stream(orow + idx * VEC, x[j]);
         }
     }
 }
@@ -122,8 +176,9 @@ void norm_rows_generic_kernel(T* __restrict__ out, T* __restrict__ residual, con
         }
         ss = fmaf(v, v, ss);
     }
-    ss = row_sum<256>(ss, smem, tid);
-    const float inv = rsqrtf(ss / (float)H + eps);
+    float sv[1] = {ss};
+    row_sums<256, 1>(sv, smem, tid);
+    const float inv = rsqrtf(sv[0] / (float)H + eps);
     for (int i = tid; i < H; i += 256) {
         float v = to_f32(orow[i]);
         if constexpr (FUSED) {
@@ -135,17 +190,17 @@ void norm_rows_generic_kernel(T* __restrict__ out, T* __restrict__ residual, con
     }
 }
 
-template <typename T, int TPR, bool FUSED>
-int launch_tpr(T* out, T* residual, const T* bias, const T* gamma, float eps, int N, int H, hipStream_t st)
+template <typename T, int TPR, int RPT, bool FUSED>
+int launch_team(T* out, T* residual, const T* bias, const T* gamma, float eps, int N, int H, hipStream_t st)
 {
     constexpr int VEC = Elt<T>::kVec;
     constexpr int BLOCK = TPR > 256 ? TPR : 256;
-    constexpr int RPB = BLOCK / TPR;
+    constexpr int RPB = BLOCK / TPR * RPT;       // rows per block
     const int nvec = H / VEC;
     const int need = (nvec + TPR - 1) / TPR;
     const dim3 grid((N + RPB - 1) / RPB), block(BLOCK);
-#define ONELLM_NORM_CASE(nv)                                                                                     \
-    hipLaunchKernelGGL((norm_rows_kernel<T, nv, TPR, FUSED>), grid, block, 0, st, out, residual, bias, gamma, eps, N, H)
+#define ONELLM_NORM_CASE(nv)                                                                                          \
+    hipLaunchKernelGGL((norm_rows_kernel<T, nv, TPR, RPT, FUSED>), grid, block, 0, st, out, residual, bias, gamma, eps, N, H)
     if (need <= 1) ONELLM_NORM_CASE(1);
     else if (need <= 2) ONELLM_NORM_CASE(2);
     else if (need <= 4) ONELLM_NORM_CASE(4);
@@ -154,6 +209,16 @@ int launch_tpr(T* out, T* residual, const T* bias, const T* gamma, float eps, in
     else return ONELLM_EUNSUPPORTED;
 #undef ONELLM_NORM_CASE
     return launch_status();
+}
+
+template <typename T, int RPT, bool FUSED>
+int launch_tpr(int tpr, T* out, T* residual, const T* bias, const T* gamma, float eps, int N, int H, hipStream_t st)
+{
+    if (tpr == 64) return launch_team<T, 64, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
+    if (tpr == 128) return launch_team<T, 128, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
+    if (tpr == 256) return launch_team<T, 256, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
+    if (tpr == 512) return launch_team<T, 512, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
+    return launch_team<T, 1024, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
 }
 
 template <typename T, bool FUSED>
@@ -168,20 +233,17 @@ int launch_norm(T* out, T* residual, const T* bias, const T* gamma, float eps, i
         return launch_status();
     }
     const int nvec = H / VEC;
+    // team size: two 16-byte vectors per thread and row measured best (8 KiB fp16 rows -> 256
+    // threads, 16 KiB -> 512)
     int tpr = tune_get("norm_tpr");
-    if (tpr != 64 && tpr != 256 && tpr != 1024) {
-        // one wave per row once there are enough rows to fill the chip with independent waves and
-        // the row fits a wave's registers; otherwise a workgroup per row
-        const int wave_nv_cap = FUSED ? 8 : 16;
-        if (N >= 2048 && nvec <= kWave * wave_nv_cap) tpr = 64;
-        else if (nvec <= 256 * 16) tpr = 256;
-        else tpr = 1024;
+    if (tpr != 64 && tpr != 128 && tpr != 256 && tpr != 512 && tpr != 1024) {
+        tpr = 64;
+        while (tpr < 1024 && nvec > tpr * 2) tpr *= 2;
     }
-    if (tpr == 64 && nvec > 64 * 16) tpr = 256;
-    if (tpr == 256 && nvec > 256 * 16) tpr = 1024;
-    if (tpr == 64) return launch_tpr<T, 64, FUSED>(out, residual, bias, gamma, eps, N, H, st);
-    if (tpr == 256) return launch_tpr<T, 256, FUSED>(out, residual, bias, gamma, eps, N, H, st);
-    return launch_tpr<T, 1024, FUSED>(out, residual, bias, gamma, eps, N, H, st);
+    while (tpr < 1024 && nvec > tpr * 16) tpr *= 2;
+    // several rows per team (2 or 4, all loads issued up front) were measured too and gave nothing
+    // over one row per team on MI355X: the plateau is the read/write mix at the memory, not latency
+    return launch_tpr<T, 1, FUSED>(tpr, out, residual, bias, gamma, eps, N, H, st);
 }
 
 }  // namespace

@@ -13,11 +13,9 @@ struct Knob {
 };
 // -1 = let the launcher decide.  Meant for benchmarks and sweeps, not part of the stable ABI.
 Knob g_knobs[] = {
-    {"norm_tpr", {-1}},          // threads per row of the norm kernels: 64, 256 or 1024
+    {"norm_tpr", {-1}},          // threads per row of the norm kernels: 64 .. 1024
     {"attn_target_wgs", {-1}},   // workgroups the sequence split of decode attention aims for
     {"attn_nsplit", {-1}},       // force the number of sequence splits
-    {"attn_unroll", {-1}},       // cache rows per row group per iteration (exploration variants)
-    {"attn_waves", {-1}},        // waves per workgroup (exploration variants)
 };
 }  // namespace
 

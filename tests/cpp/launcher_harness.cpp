@@ -1,0 +1,144 @@
+// Test harness for the launcher shims: builds oneLLM-style Tensor / BaseWeight / LayerNormWeight
+// objects around raw pointers handed in from Python and calls the six launch* functions exactly as
+// the oneLLM layers and unit tests do.  C++ exceptions are turned into return code 1 + a message.
+#include <cstring>
+#include <exception>
+#include <string>
+#include "onellm/kernels.h"
+
+namespace {
+std::string g_last_error;
+
+template <typename F>
+int guarded(F&& f)
+{
+    try {
+        f();
+        g_last_error.clear();
+        return 0;
+    } catch (const std::exception& e) {
+        g_last_error = e.what();
+        return 1;
+    }
+}
+
+DataType dt(int dtype) { return dtype == 1 ? FP16 : (dtype == 0 ? FP32 : INT8); }
+
+Tensor cache_tensor(int dtype, void* p, int L, int B, int Hkv, int S, int D)
+{
+    if (L <= 0) return Tensor(GPU, dt(dtype), {B, Hkv, S, D}, p);        // 4-D, as the kernel unit tests build it
+    return Tensor(GPU, dt(dtype), {L, B, Hkv, S, D}, p);                 // 5-D, as the layers allocate it
+}
+}  // namespace
+
+extern "C" {
+
+const char* h_last_error() { return g_last_error.c_str(); }
+
+int h_decode_mha(int dtype, void* qkv, void* bias, void* kc, void* vc, void* out, int B, int Hq, int Hkv, int D, int S,
+                 int L, int step_value, int step_on_gpu, int rotary_dim, float base)
+{
+    return guarded([&] {
+        Tensor qkv_buf(GPU, dt(dtype), {B, Hq + 2 * Hkv, D}, qkv);
+        BaseWeight w;
+        w.data = nullptr;
+        w.type = dtype == 1 ? WeightType::FP16_W : WeightType::FP32_W;
+        w.bias = bias;
+        Tensor k_cache = cache_tensor(dtype, kc, L, B, Hkv, S, D);
+        Tensor v_cache = cache_tensor(dtype, vc, L, B, Hkv, S, D);
+        bool fin = false;
+        Tensor finished(GPU, BOOL, {B}, &fin);
+        int h_step = step_value;
+        Tensor step(step_on_gpu ? GPU : CPU, INT32, {1}, &h_step);
+        Tensor mha_output(GPU, dt(dtype), {B, Hq * D}, out);
+        LLaMAAttentionStaticParams params;
+        params.rotary_embedding_dim = rotary_dim;
+        params.rotary_embedding_base = base;
+        params.max_position_embeddings = 2048;
+        params.use_dynamic_ntk = false;
+        launchDecoderMaskedMHA(&qkv_buf, w, &k_cache, &v_cache, &finished, &step, &mha_output, params);
+    });
+}
+
+int h_rmsnorm(int dtype, void* x, void* gamma, int N, int H, float eps)
+{
+    return guarded([&] {
+        Tensor t(GPU, dt(dtype), {N, H}, x);
+        LayerNormWeight w;
+        w.gamma = (float*)gamma;
+        launchRMSNorm(&t, w, eps);
+    });
+}
+
+int h_fused_norm(int dtype, void* residual, void* out, void* bias, void* gamma, int N, int H, float eps)
+{
+    return guarded([&] {
+        if (dtype == 1)
+            launchFusedAddBiasResidualRMSNorm<half>((half*)residual, (half*)out, (const half*)bias, (const half*)gamma, eps, N, H);
+        else
+            launchFusedAddBiasResidualRMSNorm<float>((float*)residual, (float*)out, (const float*)bias, (const float*)gamma, eps, N, H);
+    });
+}
+
+int h_append(int dtype, void* ks, void* vs, void* kc, void* vc, void* cur, void* hist, int B, int Hkv, int Q, int S, int D,
+             int L, int host_layer_id)
+{
+    return guarded([&] {
+        Tensor k_src(GPU, dt(dtype), {B, Hkv, Q, D}, ks), v_src(GPU, dt(dtype), {B, Hkv, Q, D}, vs);
+        Tensor k_dst = cache_tensor(dtype, kc, L, B, Hkv, S, D), v_dst = cache_tensor(dtype, vc, L, B, Hkv, S, D);
+        Tensor cur_len(GPU, INT32, {B}, cur), history(GPU, INT32, {B}, hist);
+        int lid = host_layer_id;
+        Tensor layer_id(CPU, INT32, {1}, &lid);
+        launchAppendKVCache(&k_src, &v_src, host_layer_id >= 0 ? &layer_id : nullptr, &cur_len, &history, &k_dst, &v_dst);
+    });
+}
+
+int h_repeat(int dtype, void* kc, void* vc, void* kd, void* vd, void* ctx, int B, int Hq, int Hkv, int S, int MK, int D, int L,
+             int host_layer_id)
+{
+    return guarded([&] {
+        Tensor k_src = cache_tensor(dtype, kc, L, B, Hkv, S, D), v_src = cache_tensor(dtype, vc, L, B, Hkv, S, D);
+        Tensor k_dst(GPU, dt(dtype), {B, Hq, MK, D}, kd), v_dst(GPU, dt(dtype), {B, Hq, MK, D}, vd);
+        Tensor ctx_len(GPU, INT32, {B}, ctx);
+        int lid = host_layer_id;
+        Tensor layer_id(CPU, INT32, {1}, &lid);
+        launchTransposeKVCache(&k_src, &v_src, &ctx_len, host_layer_id >= 0 ? &layer_id : nullptr, &k_dst, &v_dst);
+    });
+}
+
+int h_topk(const float* probs, int B, int V, float* ws)
+{
+    return guarded([&] { launchTopKforBeamSearch(probs, B, V, ws); });
+}
+
+// the callers' pattern after every launch (src/layers/attention/masked_self_attention.cpp:73 in oneLLM)
+int h_sync_and_check()
+{
+    return guarded([] { DeviceSyncAndCheckCudaError(); });
+}
+
+// host-only behaviour of the carrier types
+int h_getval_requires_cpu_tensor()
+{
+    int v = 7;
+    Tensor on_cpu(CPU, INT32, {1}, &v), on_gpu(GPU, INT32, {1}, &v);
+    if (on_cpu.getVal<int>() != 7) return 2;
+    return guarded([&] { (void)on_gpu.getVal<int>(); });   // must throw -> 1
+}
+
+int h_tensor_size(int a, int b, int c)
+{
+    int dummy;
+    Tensor t(CPU, FP32, {a, b, c}, &dummy);
+    Tensor empty(CPU, FP32, {a, b, c});
+    return empty.size() == 0 ? t.size() : -1;
+}
+
+int h_type_tags()
+{
+    return (getTensorType<float>() == FP32) + 2 * (getTensorType<half>() == FP16) + 4 * (getTensorType<int>() == INT32)
+           + 8 * (getTensorType<const float>() == FP32) + 16 * (getWeightType<half>() == WeightType::FP16_W)
+           + 32 * (getBitNum(WeightType::INT8_W) == 8);
+}
+
+}  // extern "C"

@@ -1,0 +1,162 @@
+"""The six launch* shims with oneLLM's own signatures, driven through a small C harness that builds
+Tensor / BaseWeight / LayerNormWeight objects the way the oneLLM layers and unit tests do.
+Host-side behaviour (carrier types, argument errors -> exceptions) runs without a GPU; the parity
+checks against the CPU oracle are marked gpu."""
+import ctypes
+import math
+import os
+
+import numpy as np
+import pytest
+
+from conftest import announce
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
+
+
+@pytest.fixture(scope="module")
+def H():
+    assert os.path.exists(HARNESS), "build it with `python -m onellm_amd.build`"
+    L = ctypes.CDLL(HARNESS)
+    vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    L.h_last_error.restype = ctypes.c_char_p
+    L.h_decode_mha.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cf]
+    L.h_rmsnorm.argtypes = [ci, vp, vp, ci, ci, cf]
+    L.h_fused_norm.argtypes = [ci, vp, vp, vp, vp, ci, ci, cf]
+    L.h_append.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci]
+    L.h_repeat.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci]
+    L.h_topk.argtypes = [vp, ci, ci, vp]
+    return L
+
+
+# ---------------------------------------------------------------- host only
+
+def test_carrier_types(H):
+    assert H.h_type_tags() == 63
+    assert H.h_tensor_size(2, 3, 4) == 24
+    assert H.h_getval_requires_cpu_tensor() == 1          # getVal on a GPU tensor throws
+    assert b"[oneLLM][ERROR]" in H.h_last_error()
+
+
+def test_precondition_failures_throw_without_touching_the_gpu(H):
+    fake = ctypes.c_void_p(0x1000)
+    # step tensor on the GPU: the launcher must refuse to dereference it on the host
+    assert H.h_decode_mha(0, fake, None, fake, fake, fake, 1, 2, 1, 16, 32, 1, 4, 1, 128, 10000.0) == 1
+    assert b"step must be a host tensor" in H.h_last_error()
+    # unsupported element type
+    assert H.h_rmsnorm(5, fake, fake, 2, 32, 1e-5) == 1
+    assert b"only FP32 and FP16" in H.h_last_error()
+    # step beyond the cache
+    assert H.h_decode_mha(0, fake, None, fake, fake, fake, 1, 2, 1, 16, 32, 1, 33, 0, 128, 10000.0) == 1
+    assert b"step outside" in H.h_last_error()
+    # a head size the kernels are not built for: rejected by the C ABI before any launch, surfaces as [TM][ERROR]
+    assert H.h_decode_mha(0, fake, None, fake, fake, fake, 1, 2, 1, 24, 32, 1, 4, 0, 128, 10000.0) == 1
+    assert b"[TM][ERROR] launchDecoderMaskedMHA" in H.h_last_error()
+    assert H.h_topk(None, 1, 100, fake) == 1
+    assert b"launchTopKforBeamSearch" in H.h_last_error()
+
+
+# ---------------------------------------------------------------- GPU parity through the launchers
+
+def _dev(a, dev):
+    import torch
+    return torch.from_numpy(a).to(dev)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,five_d", [(np.float32, True), (np.float32, False), (np.float16, True)])
+def test_launchDecoderMaskedMHA(H, ref, dev, dtype, five_d):
+    announce("launchDecoderMaskedMHA", dtype.__name__, five_d)
+    rng = np.random.default_rng(1)
+    B, Hq, Hkv, D, S, t = 2, 4, 2, 64, 48, 37
+    L = 2 if five_d else 1
+    qkv = (rng.standard_normal((B, Hq + 2 * Hkv, D)) * 0.5).astype(dtype)
+    bias = (rng.standard_normal((Hq + 2 * Hkv) * D) * 0.5).astype(dtype)
+    kc = (rng.standard_normal((L, B, Hkv, S, D)) * 0.5).astype(dtype)
+    vc = (rng.standard_normal((L, B, Hkv, S, D)) * 0.5).astype(dtype)
+    import torch
+    d = [_dev(a, dev) for a in (qkv, bias, kc, vc)]
+    out = torch.zeros(B, Hq * D, dtype=d[0].dtype, device=dev)
+    code = 1 if dtype == np.float16 else 0
+    rc = H.h_decode_mha(code, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), out.data_ptr(),
+                        B, Hq, Hkv, D, S, L if five_d else 0, t, 0, D, 10000.0)
+    assert rc == 0, H.h_last_error()
+    assert H.h_sync_and_check() == 0, H.h_last_error()
+    want = ref.decode_attn(qkv, bias, kc, vc, Hq, t, D, 10000.0, layer=0)
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == np.float32 else dict(rtol=1e-2, atol=2e-3)
+    np.testing.assert_allclose(out.cpu().numpy().astype(np.float64), want.astype(np.float64), **tol)
+    it = np.uint32 if dtype == np.float32 else np.uint16
+    np.testing.assert_array_equal(d[2].cpu().numpy().view(it), kc.view(it))
+    np.testing.assert_array_equal(d[3].cpu().numpy().view(it), vc.view(it))
+
+
+@pytest.mark.gpu
+def test_launchRMSNorm_and_fused_norm(H, ref, dev):
+    import torch
+    announce("launchRMSNorm / launchFusedAddBiasResidualRMSNorm")
+    # the reference unit-test vectors: 2 x 32 ones, eps 0.5
+    x = torch.ones(2, 32, device=dev)
+    g = torch.ones(32, device=dev)
+    assert H.h_rmsnorm(0, x.data_ptr(), g.data_ptr(), 2, 32, 0.5) == 0, H.h_last_error()
+    np.testing.assert_allclose(x.cpu().numpy(), 1 / math.sqrt(1.5), rtol=1e-6)
+    rng = np.random.default_rng(2)
+    for dtype, code in ((np.float32, 0), (np.float16, 1)):
+        out = rng.standard_normal((9, 4096)).astype(dtype)
+        res = rng.standard_normal((9, 4096)).astype(dtype)
+        bias = rng.standard_normal(4096).astype(dtype)
+        gam = rng.uniform(0.5, 1.5, 4096).astype(dtype)
+        d = [_dev(a, dev) for a in (res, out, bias, gam)]
+        assert H.h_fused_norm(code, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), 9, 4096, 1e-5) == 0
+        w_res, w_out = ref.fused_add_bias_residual_rmsnorm(res, out, bias, gam, 1e-5)
+        it = np.uint32 if dtype == np.float32 else np.uint16
+        np.testing.assert_array_equal(d[0].cpu().numpy().view(it), w_res.view(it))
+        tol = dict(rtol=1e-5, atol=1e-6) if dtype == np.float32 else dict(rtol=1e-2, atol=2e-3)
+        np.testing.assert_allclose(d[1].cpu().numpy().astype(np.float64), w_out.astype(np.float64), **tol)
+    assert H.h_sync_and_check() == 0
+
+
+@pytest.mark.gpu
+def test_launchAppendKVCache_and_launchTransposeKVCache(H, ref, dev):
+    import torch
+    announce("launchAppendKVCache / launchTransposeKVCache")
+    rng = np.random.default_rng(3)
+    L, B, Hq, Hkv, Q, S, D, MK = 2, 3, 8, 2, 5, 24, 16, 20
+    ks = rng.standard_normal((B, Hkv, Q, D)).astype(np.float32)
+    vs = rng.standard_normal((B, Hkv, Q, D)).astype(np.float32)
+    kc = rng.standard_normal((L, B, Hkv, S, D)).astype(np.float32)
+    vc = rng.standard_normal((L, B, Hkv, S, D)).astype(np.float32)
+    cur = np.array([5, 2, 0], np.int32)
+    hist = np.array([3, 19, 7], np.int32)
+    d = [_dev(a, dev) for a in (ks, vs, kc, vc, cur, hist)]
+    assert H.h_append(0, *[t.data_ptr() for t in d], B, Hkv, Q, S, D, L, 1) == 0, H.h_last_error()
+    ref.kv_append(ks, vs, kc, vc, cur, hist, layer=1)
+    np.testing.assert_array_equal(d[2].cpu().numpy().view(np.uint32), kc.view(np.uint32))
+    np.testing.assert_array_equal(d[3].cpu().numpy().view(np.uint32), vc.view(np.uint32))
+    ctx = (hist + cur).astype(np.int32)
+    kd = np.full((B, Hq, MK, D), 9.0, np.float32)
+    vd = np.full((B, Hq, MK, D), 9.0, np.float32)
+    e = [_dev(a, dev) for a in (kd, vd, ctx)]
+    assert H.h_repeat(0, d[2].data_ptr(), d[3].data_ptr(), e[0].data_ptr(), e[1].data_ptr(), e[2].data_ptr(),
+                      B, Hq, Hkv, S, MK, D, L, 1) == 0, H.h_last_error()
+    ref.kv_repeat(kc, vc, kd, vd, ctx, layer=1)
+    np.testing.assert_array_equal(e[0].cpu().numpy().view(np.uint32), kd.view(np.uint32))
+    np.testing.assert_array_equal(e[1].cpu().numpy().view(np.uint32), vd.view(np.uint32))
+    assert H.h_sync_and_check() == 0
+
+
+@pytest.mark.gpu
+def test_launchTopKforBeamSearch_reference_layout(H, ref, dev):
+    import torch
+    announce("launchTopKforBeamSearch")
+    B, V = 3, 30000
+    rng = np.random.default_rng(4)
+    logits = rng.integers(-50, 50, size=(B * 2, V)).astype(np.float32)
+    ws = torch.zeros(2 * B * 2 + 2 * B * 2 * 8 * 2, dtype=torch.float32, device=dev)     # the reference test's size
+    assert H.h_topk(_dev(logits, dev).data_ptr(), B, V, ws.data_ptr()) == 0, H.h_last_error()
+    assert H.h_sync_and_check() == 0
+    w = ws.cpu().numpy()
+    off = 2 * B * 2 * 8 * 2                                                              # where the reference test reads
+    _, _, wfv, wfi = ref.beam_topk(logits, B, 2, 2)
+    np.testing.assert_array_equal(w[off:off + B * 2].reshape(B, 2), wfv)
+    np.testing.assert_array_equal(w.view(np.int32)[off + B * 2:off + 2 * B * 2].reshape(B, 2), wfi)
