@@ -20,6 +20,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0   # MI355X, published
 
+# HBM bytes per launch of the headline kernel as counted by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
+# each scaled by the same counter's reading for a 1 GiB device copy: x2.0000 and x1.0000), keyed by context.
+MEASURED_TRAFFIC_BYTES = {4096: 1074413568}
+
 
 def attn_bytes(B, Hq, Hkv, D, t_list, e):
     """Algorithmic bytes of one decode step: history K+V read once, new row written, qkv + bias read, out written."""
@@ -118,6 +122,9 @@ def main():
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--no-extras", action="store_true", help="skip the context sweep, GQA, norm and top-K lines")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also launch a plain 1 GiB device copy a few times (a kernel of known traffic that scales "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); --gpus %d is not supported" % args.gpus)
@@ -128,6 +135,15 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibration_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)      # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     B, H, D, S, t = 16, 32, 128, 4096, args.ctx
     ms, (qkv, bias, (kc, vc), out) = bench_attention(capi, dev, args.steps, args.warmup, B, H, H, D, S, t, nsets=4)
@@ -143,10 +159,14 @@ def main():
                    "storage": "fp16", "arithmetic": "fp32"},
         "hbm_gbps": round(gbps, 1), "hbm_frac_of_8TBps": round(gbps / HBM_PEAK_GBPS, 4),
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(t),
                      "kernel": "decode_attn_split_kernel<__half,16,1,4,4>",
                      "algorithmic_bytes_per_launch": nbytes,
-                     "note": "duration = HIP-event time of the whole step (split kernel + merge kernel) / steps"},
+                     "note": "duration = HIP-event time per step on the launch stream; at this shape a step is exactly "
+                             "one launch of the kernel (single sequence split, no merge pass). traffic = FETCH_SIZE + "
+                             "WRITE_SIZE of a separate rocprofv3 --pmc run, scaled by a 1 GiB copy "
+                             "(profiles/decode_attn_split_kernel_llama7b_ctx4096.md)"},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_attention(qkv, bias, kc, vc, H, t, D)
