@@ -453,19 +453,24 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     a.qscale = (1.0f / sqrtf((float)D)) * 1.4426950408889634f;
     a.slab = (size_t)layer * B * Hkv * (size_t)S * D;
 
-    // Sequence split.  Equal lengths (t_dev == NULL): about two workgroups (eight waves) per compute
-    // unit measured best on MI355X — long contiguous streams per workgroup, and with a single split
-    // there is no merge pass at all.  Per-sequence lengths: finer chunks (about 16 workgroups per
-    // compute unit, chunks of at least 256 rows) so that the dispatcher can balance ragged work.
+    // Sequence split, from sweeps on MI355X.  Equal lengths (t_dev == NULL): about one workgroup per
+    // compute unit with chunks of at least 512 rows (more, smaller workgroups only add per-workgroup
+    // set-up and merge work); a shape that already has that many workgroups is not split at all and
+    // needs no merge pass.  Per-sequence lengths: finer chunks (about 16 workgroups per compute unit,
+    // at least 256 rows each) so that the dispatcher can balance ragged work.
     const int G = a.G;
     const int gt = G == 1 ? 1 : (G == 2 ? 2 : 4);
     const int ngt = (G + gt - 1) / gt;
     const long base_wgs = (long)B * Hkv * ngt;
-    int target = tune_get("attn_target_wgs");
-    if (target <= 0) target = t_dev ? 4096 : 512;
+    const int user_target = tune_get("attn_target_wgs");
+    const int target = user_target > 0 ? user_target : (t_dev ? 4096 : 256);
     int nsplit = (int)((target + base_wgs - 1) / base_wgs);
     int cap = max_splits(max_t);
-    if (t_dev && tune_get("attn_target_wgs") <= 0) cap = (max_t + 255) / 256 < cap ? (max_t + 255) / 256 : cap;
+    if (user_target <= 0) {
+        const int min_rows = t_dev ? 256 : 512;
+        const int by_rows = max_t / min_rows;
+        cap = by_rows < cap ? by_rows : cap;
+    }
     if (nsplit > cap) nsplit = cap;
     if (nsplit < 1) nsplit = 1;
     const int forced = tune_get("attn_nsplit");
