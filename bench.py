@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the decode hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--calibration-copy]
 
 A step is one fused decode-attention call at the Llama-2-7B shape (batch 16, 32 heads x 128, fp16 KV
 cache, context 4096): bias + RoPE + cache write + softmax + V sum for one new token per sequence.
 Inputs are synthetic, resident in HBM before the timed region, and each step uses the next of several
-distinct cache sets so that the 256 MB Infinity Cache cannot serve the stream.  Prints ONE JSON line.
+distinct cache sets so that the 256 MB Infinity Cache cannot serve the stream.  Prints ONE JSON line;
+`extras` holds the other shapes of the path (context sweep, grouped-query config, KV concat/repeat,
+norms, beam top-K), each with the CPU oracle timed beside it.
 """
 import argparse
 import json
@@ -47,6 +49,33 @@ def time_steps(fn, steps, warmup):
     return start.elapsed_time(end) / steps
 
 
+def host_cores():
+    n = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
+    return min(n, os.cpu_count() or n)
+
+
+def time_cpu(fn, budget_s=6.0, max_runs=5):
+    """Median wall time (us) of fn() on the host, at most max_runs runs within a time budget."""
+    times = []
+    end = time.time() + budget_s
+    for _ in range(max_runs):
+        t0 = time.time()
+        fn()
+        times.append(time.time() - t0)
+        if time.time() + times[-1] > end:
+            break
+    times.sort()
+    return times[len(times) // 2] * 1e6, len(times)
+
+
+def entry(ms, nbytes, cpu_us=None):
+    e = {"us": round(ms * 1e3, 2), "gbps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
+         "bytes": int(nbytes)}
+    if cpu_us is not None:
+        e["cpu_us"] = round(cpu_us, 1)
+    return e
+
+
 def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=None):
     import torch
     torch.manual_seed(2)
@@ -69,11 +98,20 @@ def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=
     return ms, (qkv, bias, sets[0], out)
 
 
+def cpu_attention(qkv, bias, kc, vc, Hq, t, D, budget_s):
+    """The CPU oracle (a port of the reference semantics, OpenMP over (sequence, kv-head)) on the same inputs, on
+    this host's cores.  Checker used as a reported baseline only."""
+    from oracle import ref
+    h_qkv, h_bias = qkv.cpu().numpy(), bias.cpu().numpy()
+    h_kc, h_vc = kc.cpu().numpy(), vc.cpu().numpy()
+    return time_cpu(lambda: ref.decode_attn(h_qkv, h_bias, h_kc, h_vc, Hq, t, D, 10000.0), budget_s)
+
+
 def bench_norms(capi, dev, steps, warmup, N, H, fused):
     import torch
     torch.manual_seed(4)
-    nsets = max(3, int(1.2e9 // (N * H * 2 * (2 if fused else 1))) if N * H * 2 < 4e8 else 3)
-    nsets = min(nsets, 64)
+    per_set = N * H * 2 * (2 if fused else 1)
+    nsets = min(64, max(3, int(1.2e9 // per_set)))
     xs = [torch.randn(N, H, device=dev).half() for _ in range(nsets)]
     rs = [torch.randn(N, H, device=dev).half() for _ in range(nsets)] if fused else None
     g = torch.rand(H, device=dev).add_(0.5).half()
@@ -90,28 +128,85 @@ def bench_norms(capi, dev, steps, warmup, N, H, fused):
     return ms, nbytes
 
 
-def cpu_baseline_attention(qkv, bias, kc, vc, Hq, t, D):
-    """The CPU oracle (a port of the reference semantics, OpenMP over (sequence, kv-head)) on the same
-    inputs, on this host's cores.  Checker used as a reported baseline only."""
+def cpu_norm(N, H, fused, budget_s):
     import numpy as np
     from oracle import ref
-    ref.build()
-    h_qkv, h_bias = qkv.cpu().numpy(), bias.cpu().numpy()
-    h_kc, h_vc = kc.cpu().numpy(), vc.cpu().numpy()
-    cores = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
-    cores = min(cores, os.cpu_count() or cores)
-    times = []
-    budget = time.time() + 25.0
-    for _ in range(5):
-        t0 = time.time()
-        ref.decode_attn(h_qkv, h_bias, h_kc, h_vc, Hq, t, D, 10000.0)
-        times.append(time.time() - t0)
-        if time.time() + times[-1] > budget:
-            break
-    times.sort()
-    return {"value": round(times[len(times) // 2] * 1e6, 1), "unit": "us/step", "cores": cores, "kind": "port",
-            "sample": "the full batch-16 ctx-4096 step (1.07 GB of fp16 KV), median of %d runs, OpenMP over "
-                      "(sequence, kv-head)" % len(times)}
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((N, H), dtype=np.float32).astype(np.float16)
+    r = rng.standard_normal((N, H), dtype=np.float32).astype(np.float16)
+    b = rng.standard_normal(H, dtype=np.float32).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, H).astype(np.float16)
+    if fused:
+        return time_cpu(lambda: ref.fused_add_bias_residual_rmsnorm(r, x, b, g, 1e-5), budget_s)
+    return time_cpu(lambda: ref.rmsnorm(x, g, 1e-5), budget_s)
+
+
+def extras_section(capi, dev, args, with_cpu):
+    import numpy as np
+    import torch
+    ex = {}
+    B, H, D, S = 16, 32, 128, 4096
+    for c in (512, 1024, 2048):
+        ms, (qkv, bias, (kc, vc), _) = bench_attention(capi, dev, args.steps, args.warmup, B, H, H, D, S, c, nsets=4)
+        cpu = cpu_attention(qkv, bias, kc, vc, H, c, D, 3.0)[0] if with_cpu else None
+        ex["decode_attn_ctx%d" % c] = entry(ms, attn_bytes(B, H, H, D, [c] * B, 2), cpu)
+        del qkv, bias, kc, vc
+        torch.cuda.empty_cache()
+
+    # BASELINE configs[2]: batch 32, 32 query heads over 8 KV heads, lengths U[1024, 8192], S = 8192
+    B3, Hq3, Hkv3, S3 = 32, 32, 8, 8192
+    G = Hq3 // Hkv3
+    tl = np.random.default_rng(3).integers(1024, 8193, size=B3).astype(np.int32)
+    t_dev = torch.from_numpy(tl).to(dev)
+    nb_fused = attn_bytes(B3, Hq3, Hkv3, D, tl.tolist(), 2)
+    steps3 = max(args.steps // 3, 10)
+    ms, (qkv, bias, (kc, vc), _) = bench_attention(capi, dev, steps3, args.warmup, B3, Hq3, Hkv3, D, S3, S3, nsets=3, t_dev=t_dev)
+    cpu = cpu_attention(qkv, bias, kc, vc, Hq3, tl, D, 6.0)[0] if with_cpu else None
+    ex["decode_attn_gqa_fused_b32_q32_kv8_len1024-8192"] = entry(ms, nb_fused, cpu)
+    # the reference-style path on the same data: concat the new row, repeat KV to 32 heads, attend over 32 heads
+    hist = (t_dev - 1).contiguous()
+    ones = torch.ones(B3, dtype=torch.int32, device=dev)
+    ksrc = torch.randn(B3, Hkv3, 1, D, device=dev).mul_(0.5).half()
+    vsrc = torch.randn(B3, Hkv3, 1, D, device=dev).mul_(0.5).half()
+    ms_app = time_steps(lambda i: capi.kv_append(ksrc, vsrc, kc, vc, ones, hist), args.steps, args.warmup)
+    ex["kv_append_decode_b32_kv8"] = entry(ms_app, 2 * 2 * B3 * Hkv3 * D * 2)
+    rk = torch.empty(1, B3, Hq3, S3, D, dtype=torch.float16, device=dev)
+    rv = torch.empty(1, B3, Hq3, S3, D, dtype=torch.float16, device=dev)
+    ms_rep = time_steps(lambda i: capi.kv_repeat(kc, vc, rk[0], rv[0], t_dev), steps3, 3)
+    nb_rep = (1 + G) * 2 * int(tl.sum()) * Hkv3 * D * 2
+    ex["kv_repeat_b32_q32_kv8_len1024-8192"] = entry(ms_rep, nb_rep)
+    qkv_r = torch.cat([qkv[:, :Hq3], qkv[:, Hq3:Hq3 + Hkv3].repeat_interleave(G, 1),
+                       qkv[:, Hq3 + Hkv3:].repeat_interleave(G, 1)], 1).contiguous()
+    b3 = bias.view(Hq3 + 2 * Hkv3, D)
+    bias_r = torch.cat([b3[:Hq3], b3[Hq3:Hq3 + Hkv3].repeat_interleave(G, 0), b3[Hq3 + Hkv3:].repeat_interleave(G, 0)], 0).contiguous().view(-1)
+    out_r = torch.zeros(B3, Hq3 * D, dtype=torch.float16, device=dev)
+    ws = torch.empty(capi.decode_attn_workspace_bytes(B3, Hq3, Hq3, D, S3), dtype=torch.uint8, device=dev)
+    ms_mha = time_steps(lambda i: capi.decode_attn(qkv_r, bias_r, rk, rv, out_r, Hq3, S3, D, 10000.0, t_dev=t_dev, max_t=S3,
+                                                   workspace=ws), steps3, 3)
+    e = entry(ms_app + ms_rep + ms_mha, nb_fused)
+    e["parts_us"] = {"append": round(ms_app * 1e3, 2), "repeat": round(ms_rep * 1e3, 2), "mha_over_32_heads": round(ms_mha * 1e3, 2)}
+    e["note"] = "concat -> repeat -> attend on the same data; gbps/frac are against the FUSED path's algorithmic bytes"
+    ex["decode_attn_gqa_repeat_path_total"] = e
+    del rk, rv, kc, vc, qkv, bias, qkv_r, ws
+    torch.cuda.empty_cache()
+
+    for (N, Hd) in ((16, 4096), (512, 4096), (8192, 4096), (8192, 8192)):
+        for fused in (False, True):
+            ms, nb = bench_norms(capi, dev, args.steps, args.warmup, N, Hd, fused)
+            cpu = cpu_norm(N, Hd, fused, 2.0)[0] if with_cpu else None
+            ex["%s_%dx%d" % ("fused_norm" if fused else "rmsnorm", N, Hd)] = entry(ms, nb, cpu)
+        torch.cuda.empty_cache()
+
+    logits = torch.randn(32, 32000, device=dev).mul_(2.0)
+    wsk = torch.empty(capi.beam_topk_workspace_bytes(8, 4, 4) // 4, dtype=torch.float32, device=dev)
+    ms = time_steps(lambda i: capi.beam_topk(logits, 8, 4, 4, workspace=wsk), args.steps, args.warmup)
+    cpu = None
+    if with_cpu:
+        from oracle import ref
+        h = logits.cpu().numpy()
+        cpu = time_cpu(lambda: ref.beam_topk(h, 8, 4, 4), 2.0)[0]
+    ex["beam_topk_b8_beam4_v32000_k4"] = entry(ms, 32 * 32000 * 4, cpu)
+    return ex
 
 
 def main():
@@ -120,8 +215,8 @@ def main():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--ctx", type=int, default=4096)
-    ap.add_argument("--no-extras", action="store_true", help="skip the context sweep, GQA, norm and top-K lines")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-extras", action="store_true", help="skip the context sweep, GQA, KV, norm and top-K lines")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also launch a plain 1 GiB device copy a few times (a kernel of known traffic that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -135,6 +230,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if not args.no_cpu:
+        from oracle import ref
+        ref.build()
 
     if args.calibration_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)      # 1 GiB read + 1 GiB written per copy
@@ -169,37 +267,14 @@ def main():
                              "(profiles/decode_attn_split_kernel_llama7b_ctx4096.md)"},
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline_attention(qkv, bias, kc, vc, H, t, D)
-
+        cpu_us, runs = cpu_attention(qkv, bias, kc, vc, H, t, D, 20.0)
+        line["cpu_baseline"] = {"value": round(cpu_us, 1), "unit": "us/step", "cores": host_cores(), "kind": "port",
+                                "sample": "the full batch-16 ctx-%d step (%.2f GB of fp16 KV), median of %d runs, OpenMP "
+                                          "over (sequence, kv-head)" % (t, nbytes / 1e9, runs)}
+    del qkv, bias, kc, vc, out
+    torch.cuda.empty_cache()
     if not args.no_extras:
-        extras = {}
-        for c in (512, 1024, 2048):
-            m, _ = bench_attention(capi, dev, args.steps, args.warmup, B, H, H, D, S, c, nsets=4)
-            nb = attn_bytes(B, H, H, D, [c] * B, 2)
-            extras["decode_attn_ctx%d" % c] = {"us": round(m * 1e3, 2), "gbps": round(nb / m / 1e6, 1),
-                                               "frac": round(nb / m / 1e6 / HBM_PEAK_GBPS, 4)}
-        del kc, vc
-        torch.cuda.empty_cache()
-        # BASELINE configs[2]: fused grouped-query read, ragged lengths
-        import numpy as np
-        tl = np.random.default_rng(3).integers(1024, 8193, size=32).astype(np.int32)
-        m, _ = bench_attention(capi, dev, max(args.steps // 3, 10), args.warmup, 32, 32, 8, 128, 8192, 8192, nsets=3,
-                               t_dev=torch.from_numpy(tl).to(dev))
-        nb = attn_bytes(32, 32, 8, 128, tl.tolist(), 2)
-        extras["decode_attn_gqa_b32_q32_kv8_len1024-8192"] = {"us": round(m * 1e3, 2), "gbps": round(nb / m / 1e6, 1),
-                                                             "frac": round(nb / m / 1e6 / HBM_PEAK_GBPS, 4)}
-        torch.cuda.empty_cache()
-        for (N, Hd) in ((16, 4096), (512, 4096), (8192, 4096), (8192, 8192)):
-            for fused in (False, True):
-                m, nb = bench_norms(capi, dev, args.steps, args.warmup, N, Hd, fused)
-                extras["%s_%dx%d" % ("fused_norm" if fused else "rmsnorm", N, Hd)] = {
-                    "us": round(m * 1e3, 2), "gbps": round(nb / m / 1e6, 1), "frac": round(nb / m / 1e6 / HBM_PEAK_GBPS, 4)}
-            torch.cuda.empty_cache()
-        logits = torch.randn(32, 32000, device=dev).mul_(2.0)
-        wsk = torch.empty(capi.beam_topk_workspace_bytes(8, 4, 4) // 4, dtype=torch.float32, device=dev)
-        m = time_steps(lambda i: capi.beam_topk(logits, 8, 4, 4, workspace=wsk), args.steps, args.warmup)
-        extras["beam_topk_b8_beam4_v32000_k4"] = {"us": round(m * 1e3, 2), "gbps": round(4096000 / m / 1e6, 1)}
-        line["extras"] = extras
+        line["extras"] = extras_section(capi, dev, args, not args.no_cpu)
     print(json.dumps(line), flush=True)
 
 

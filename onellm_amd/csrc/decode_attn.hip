@@ -337,26 +337,38 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     }
 }
 
-// Merge the per-split partial states of one (sequence, query head) and normalise.
+// Merge the per-split partial states of one (sequence, query head) and normalise: one wave per
+// (sequence, head).  Lane s holds split s's (m, l), so the maximum, the weights and the denominator
+// are two wave reductions instead of loops of dependent loads; the weighted sum over splits then
+// runs with the loads of several splits in flight.
 template <typename T>
-__global__ __launch_bounds__(128)
+__global__ __launch_bounds__(kWave)
 void decode_attn_merge_kernel(const AttnArgs a, int D)
 {
-    const int bh = blockIdx.x;
+    __shared__ float w_s[kWave];
+    const int bh = blockIdx.x, lane = threadIdx.x;
     const int b = bh / a.Hq;
     const int t = a.t_dev ? a.t_dev[b] : a.t_host;
     if (t < 1 || t > a.S) return;
     const int nvalid = min((t - 1) / a.chunk + 1, a.nsplit);   // t above max_t is out of contract: stay in bounds
     const float* ml = a.part_ml + (size_t)bh * a.nsplit * 2;
     const float* po = a.part_o + (size_t)bh * a.nsplit * D;
-    float M = -INFINITY;
-    for (int s = 0; s < nvalid; ++s) M = fmaxf(M, ml[s * 2]);
-    float L = 0.f;
-    for (int s = 0; s < nvalid; ++s) L = fmaf(ml[s * 2 + 1], __builtin_amdgcn_exp2f(ml[s * 2] - M), L);
-    const float invL = 1.0f / L;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float m = -INFINITY, l = 0.f;
+    if (lane < nvalid) {
+        m = ml[lane * 2];
+        l = ml[lane * 2 + 1];
+    }
+    float M = m;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, kWave));
+    const float w = __builtin_amdgcn_exp2f(m - M);          // 0 for the lanes without a split
+    const float invL = 1.0f / wave_sum(l * w);
+    w_s[lane] = w;
+    __syncthreads();
+    for (int d = lane; d < D; d += kWave) {
         float O = 0.f;
-        for (int s = 0; s < nvalid; ++s) O = fmaf(po[(size_t)s * D + d], __builtin_amdgcn_exp2f(ml[s * 2] - M), O);
+#pragma unroll 8
+        for (int s = 0; s < nvalid; ++s) O = fmaf(po[(size_t)s * D + d], w_s[s], O);
         static_cast<T*>(a.out)[(size_t)bh * D + d] = from_f32<T>(O * invL);
     }
 }
@@ -496,9 +508,9 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     if (rc != 0) return rc;
     if (nsplit > 1) {
         if (dtype == ONELLM_FP16)
-            hipLaunchKernelGGL((decode_attn_merge_kernel<__half>), dim3(B * Hq), dim3(128), 0, st, a, D);
+            hipLaunchKernelGGL((decode_attn_merge_kernel<__half>), dim3(B * Hq), dim3(kWave), 0, st, a, D);
         else
-            hipLaunchKernelGGL((decode_attn_merge_kernel<float>), dim3(B * Hq), dim3(128), 0, st, a, D);
+            hipLaunchKernelGGL((decode_attn_merge_kernel<float>), dim3(B * Hq), dim3(kWave), 0, st, a, D);
         rc = launch_status();
     }
     return rc;

@@ -8,7 +8,9 @@
 namespace onellm {
 namespace {
 
-// COPY is the access type: uint4 (16 B) on the normal path, the element itself otherwise.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// COPY is the access type: 16 bytes on the normal path, the element itself otherwise.
 template <typename COPY>
 __global__ __launch_bounds__(256)
 void kv_append_kernel(const COPY* __restrict__ k_src, const COPY* __restrict__ v_src,
@@ -26,7 +28,9 @@ void kv_append_kernel(const COPY* __restrict__ k_src, const COPY* __restrict__ v
     if (drow < 0 || drow >= S) return;
     const COPY* src = blockIdx.z ? v_src : k_src;
     COPY* dst = blockIdx.z ? v_cache : k_cache;
-    dst[slab + ((size_t)bh * S + (size_t)drow) * rowv + c] = src[((size_t)bh * max_q_len + tau) * rowv + c];
+    // streamed once in, once out: keep it out of the way of reusable cache lines
+    __builtin_nontemporal_store(__builtin_nontemporal_load(&src[((size_t)bh * max_q_len + tau) * rowv + c]),
+                                &dst[slab + ((size_t)bh * S + (size_t)drow) * rowv + c]);
 }
 
 template <typename COPY>
@@ -47,10 +51,10 @@ void kv_repeat_kernel(const COPY* __restrict__ k_cache, const COPY* __restrict__
     if (s >= len) return;
     const COPY* src = blockIdx.z ? v_cache : k_cache;
     COPY* dst = blockIdx.z ? v_dst : k_dst;
-    const COPY val = src[slab + ((size_t)bh * S + s) * rowv + c];
+    const COPY val = __builtin_nontemporal_load(&src[slab + ((size_t)bh * S + s) * rowv + c]);
     const size_t Hq = (size_t)Hkv * G;
     size_t o = (((size_t)b * Hq + (size_t)kvh * G) * max_k_len + s) * rowv + c;
-    for (int g = 0; g < G; ++g, o += (size_t)max_k_len * rowv) dst[o] = val;
+    for (int g = 0; g < G; ++g, o += (size_t)max_k_len * rowv) __builtin_nontemporal_store(val, &dst[o]);
 }
 
 struct CopyPlan {
@@ -88,7 +92,7 @@ extern "C" int onellm_kv_append(int dtype, const void* k_src, const void* v_src,
 #define ONELLM_APPEND(CT)                                                                                            \
     hipLaunchKernelGGL((kv_append_kernel<CT>), grid, block, 0, st, (const CT*)k_src, (const CT*)v_src, (CT*)k_cache, \
                        (CT*)v_cache, cur_len, history_len, Hkv, max_q_len, S, p.rowv, slab)
-    if (p.access == 16) ONELLM_APPEND(uint4);
+    if (p.access == 16) ONELLM_APPEND(u32x4);
     else if (p.access == 4) ONELLM_APPEND(uint32_t);
     else ONELLM_APPEND(uint16_t);
 #undef ONELLM_APPEND
@@ -115,7 +119,7 @@ extern "C" int onellm_kv_repeat(int dtype, const void* k_cache, const void* v_ca
 #define ONELLM_REPEAT(CT)                                                                                         \
     hipLaunchKernelGGL((kv_repeat_kernel<CT>), grid, block, 0, st, (const CT*)k_cache, (const CT*)v_cache,        \
                        (CT*)k_dst, (CT*)v_dst, context_len, Hkv, Hq / Hkv, S, max_k_len, p.rowv, slab)
-    if (p.access == 16) ONELLM_REPEAT(uint4);
+    if (p.access == 16) ONELLM_REPEAT(u32x4);
     else if (p.access == 4) ONELLM_REPEAT(uint32_t);
     else ONELLM_REPEAT(uint16_t);
 #undef ONELLM_REPEAT
