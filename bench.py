@@ -197,6 +197,37 @@ def extras_section(capi, dev, args, with_cpu):
             ex["%s_%dx%d" % ("fused_norm" if fused else "rmsnorm", N, Hd)] = entry(ms, nb, cpu)
         torch.cuda.empty_cache()
 
+    # the callers either side of the path: prefill QKV bias + RoPE + transpose (4 x 2048 tokens, 32 heads x 128)
+    # and the SwiGLU gate (8192 x 11008)
+    Bp, Sp, Hp = 4, 2048, 32
+    qkvs = [torch.randn(Bp * Sp, 3 * Hp, D, device=dev).mul_(0.5).half() for _ in range(3)]
+    biasp = torch.randn(3 * Hp * D, device=dev).mul_(0.5).half()
+    qb = torch.empty(Bp, Hp, Sp, D, dtype=torch.float16, device=dev)
+    kb, vb = torch.empty_like(qb), torch.empty_like(qb)
+    po = torch.zeros(Bp * Sp, dtype=torch.int32, device=dev)
+    hl = torch.zeros(Bp, dtype=torch.int32, device=dev)
+    ms = time_steps(lambda i: capi.qkv_bias_rope_transpose(qb, kb, vb, qkvs[i % 3], biasp, po, hl, D, 10000.0), steps3, 5)
+    cpu = None
+    if with_cpu:
+        from oracle import ref
+        hq, hk, hv = qb.cpu().numpy(), kb.cpu().numpy(), vb.cpu().numpy()
+        h_in, h_b, h_po, h_hl = qkvs[0].cpu().numpy(), biasp.cpu().numpy(), po.cpu().numpy(), hl.cpu().numpy()
+        cpu = time_cpu(lambda: ref.qkv_bias_rope_transpose(hq, hk, hv, h_in, h_b, h_po, h_hl, D, 10000.0), 4.0)[0]
+    ex["prefill_qkv_bias_rope_4x2048_tokens_32x128"] = entry(ms, 2 * Bp * Sp * 3 * Hp * D * 2 + 3 * Hp * D * 2, cpu)
+    del qkvs, qb, kb, vb
+    torch.cuda.empty_cache()
+    ins = [torch.randn(8192, 2, 11008, device=dev).half() for _ in range(3)]
+    oa = torch.empty(8192, 11008, dtype=torch.float16, device=dev)
+    ms = time_steps(lambda i: capi.silu_and_mul(ins[i % 3], oa), steps3, 5)
+    cpu = None
+    if with_cpu:
+        from oracle import ref
+        h_in, h_out = ins[0].cpu().numpy(), oa.cpu().numpy()
+        cpu = time_cpu(lambda: ref.silu_and_mul(h_in, h_out), 3.0)[0]
+    ex["swiglu_8192x11008"] = entry(ms, 3 * 8192 * 11008 * 2, cpu)
+    del ins, oa
+    torch.cuda.empty_cache()
+
     logits = torch.randn(32, 32000, device=dev).mul_(2.0)
     wsk = torch.empty(capi.beam_topk_workspace_bytes(8, 4, 4) // 4, dtype=torch.float32, device=dev)
     ms = time_steps(lambda i: capi.beam_topk(logits, 8, 4, 4, workspace=wsk), args.steps, args.warmup)

@@ -52,3 +52,18 @@ void launchTopKforBeamSearch(const float* probs,
                              const int batch_size,
                              const int vocab_size,
                              float* topk_workspace);
+
+// src/kernels/qkv_bias_and_RoPE.h (context phase; produces the K/V the decode step reads)
+void launchAddFusedQKVBiasTransposeAndRoPE(Tensor* q_buf,
+                                           Tensor* k_buf,
+                                           Tensor* v_buf,
+                                           Tensor* QKV,
+                                           BaseWeight& qkv,
+                                           Tensor* padding_offset,
+                                           Tensor* history_length,
+                                           Tensor* input_length,
+                                           LLaMAAttentionStaticParams& params);
+
+// src/kernels/activation_kernel.h (float as in the reference, half added)
+template<typename T>
+void launchAct(const T* input, T* out, const int batch_size, const int intermedia_size);

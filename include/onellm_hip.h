@@ -150,6 +150,35 @@ int onellm_beam_topk(const float* logits, int B, int beam, int V, int K,
                      float* workspace, onellm_stream_t stream);
 size_t onellm_beam_topk_workspace_bytes(int B, int beam, int K);
 
+/* ------------------------------------------------------------------------------------------------
+ * The callers either side of the decode path (built after the six entry points above).
+ * ---------------------------------------------------------------------------------------------- */
+
+/*
+ * Context-phase fused QKV bias + RoPE + un-pad transpose: produces the K/V rows the decode step
+ * streams.  Replaces launchAddFusedQKVBiasTransposeAndRoPE (src/kernels/qkv_bias_and_RoPE.h,
+ * src/kernels/qkv_bias_and_RoPE.cu:74-207).  For each packed token tok:
+ *   dst = tok + padding_offset[tok]; b = dst / seq_len; s = dst % seq_len; pos = history_length[b] + s
+ *   q_buf[b, h, s, :] = RoPE(qkv[tok, h] + bias, pos);  k_buf[b, kvh, s, :] likewise;
+ *   v_buf[b, kvh, s, :] = qkv[tok, Hq+Hkv+kvh] + bias
+ * qkv [token_num, Hq+2*Hkv, D]; q_buf [B, Hq, seq_len, D]; k_buf, v_buf [B, Hkv, seq_len, D];
+ * padding_offset device int32[token_num]; history_length device int32[B]; qkv_bias may be NULL.
+ * Bias layout, RoPE arithmetic and rotary parameters are those of onellm_decode_attn; a decode step
+ * with rope_pos_offset = -1 continues the positions this function writes.  D even, D <= 512.
+ */
+int onellm_qkv_bias_rope_transpose(int dtype, void* q_buf, void* k_buf, void* v_buf,
+                                   const void* qkv, const void* qkv_bias,
+                                   const int* padding_offset, const int* history_length,
+                                   int B, int seq_len, int token_num, int Hq, int Hkv, int D,
+                                   int rotary_dim, float rope_base, onellm_stream_t stream);
+
+/*
+ * SwiGLU gate.  Replaces launchAct<T> (src/kernels/activation_kernel.h, src/kernels/activation_kernel.cu:5-32):
+ *   out[b, i] = silu(input[b, 0, i]) * input[b, 1, i],  silu(x) = x / (1 + exp(-x)) in fp32.
+ * input [B, 2, I], out [B, I].
+ */
+int onellm_silu_and_mul(int dtype, const void* input, void* out, int B, int I, onellm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

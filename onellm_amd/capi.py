@@ -30,6 +30,9 @@ SYMBOLS = {
     "onellm_kv_repeat": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp]),
     "onellm_beam_topk": (_ci, [_vp, _ci, _ci, _ci, _ci, _vp, _vp]),
     "onellm_beam_topk_workspace_bytes": (_sz, [_ci, _ci, _ci]),
+    "onellm_qkv_bias_rope_transpose": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci,
+                                             _cf, _vp]),
+    "onellm_silu_and_mul": (_ci, [_ci, _vp, _vp, _ci, _ci, _vp]),
 }
 
 _lib = None
@@ -163,3 +166,22 @@ def beam_topk(logits, B, beam, K, workspace=None):
     fv = workspace[2 * n1:2 * n1 + B * K].view(B, K)
     fi = workspace[2 * n1 + B * K:2 * n1 + 2 * B * K].view(torch.int32).view(B, K)
     return workspace, vals, ids, fv, fi
+
+
+def qkv_bias_rope_transpose(q_buf, k_buf, v_buf, qkv, bias, padding_offset, history_length, rotary_dim, rope_base):
+    """qkv [token_num, Hq+2Hkv, D]; q_buf [B, Hq, seq_len, D]; k_buf / v_buf [B, Hkv, seq_len, D]."""
+    token_num, QKVH, D = qkv.shape
+    B, Hq, seq_len, _ = q_buf.shape
+    Hkv = k_buf.shape[1]
+    assert QKVH == Hq + 2 * Hkv
+    _check(lib().onellm_qkv_bias_rope_transpose(_dt(qkv), _ptr(q_buf), _ptr(k_buf), _ptr(v_buf), _ptr(qkv), _ptr(bias),
+                                                _ptr(padding_offset), _ptr(history_length), B, seq_len, token_num, Hq,
+                                                Hkv, D, rotary_dim, rope_base, _stream()),
+           "onellm_qkv_bias_rope_transpose")
+
+
+def silu_and_mul(inp, out):
+    B, two, I = inp.shape
+    assert two == 2
+    _check(lib().onellm_silu_and_mul(_dt(inp), _ptr(inp), _ptr(out), B, I, _stream()), "onellm_silu_and_mul")
+    return out

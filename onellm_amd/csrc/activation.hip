@@ -1,0 +1,62 @@
+// SwiGLU gate for gfx950: out[b, i] = silu(in[b, 0, i]) * in[b, 1, i], silu(x) = x / (1 + exp(-x)) in
+// fp32.  One 16-byte piece of the output per thread, non-temporal streams; HBM-bound: 3*B*I*e bytes.
+#include "common.hpp"
+
+namespace onellm {
+namespace {
+
+__device__ __forceinline__ float silu_mul(float x, float y) { return (x / (1.0f + __expf(-x))) * y; }
+
+template <typename T>
+__global__ __launch_bounds__(256)
+void silu_and_mul_kernel(T* __restrict__ out, const T* __restrict__ in, int I)
+{
+    constexpr int VEC = Elt<T>::kVec;
+    const int b = blockIdx.y;
+    const int v = blockIdx.x * 256 + threadIdx.x;
+    if (v >= I / VEC) return;
+    const T* row = in + (size_t)b * 2 * I;
+    const Vec16<T> x = load16_stream(row + v * VEC), y = load16_stream(row + I + v * VEC);
+    Vec16<T> o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o.set(e, silu_mul(x.get(e), y.get(e)));
+    store16_stream(out + (size_t)b * I + v * VEC, o);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256)
+void silu_and_mul_scalar_kernel(T* __restrict__ out, const T* __restrict__ in, int I)
+{
+    const int b = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= I) return;
+    const T* row = in + (size_t)b * 2 * I;
+    out[(size_t)b * I + i] = from_f32<T>(silu_mul(to_f32(row[i]), to_f32(row[I + i])));
+}
+
+template <typename T>
+int launch_act(const T* in, T* out, int B, int I, hipStream_t st)
+{
+    constexpr int VEC = Elt<T>::kVec;
+    if (B > 65535) return ONELLM_EUNSUPPORTED;
+    if (I % VEC == 0 && aligned16(in) && aligned16(out)) {
+        hipLaunchKernelGGL((silu_and_mul_kernel<T>), dim3((I / VEC + 255) / 256, B), dim3(256), 0, st, out, in, I);
+    } else {
+        hipLaunchKernelGGL((silu_and_mul_scalar_kernel<T>), dim3((I + 255) / 256, B), dim3(256), 0, st, out, in, I);
+    }
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace onellm
+
+extern "C" int onellm_silu_and_mul(int dtype, const void* input, void* out, int B, int I, onellm_stream_t stream)
+{
+    using namespace onellm;
+    if (B == 0 && I > 0) return 0;
+    if (!input || !out || B < 0 || I <= 0) return ONELLM_EINVAL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == ONELLM_FP32) return launch_act<float>((const float*)input, (float*)out, B, I, st);
+    if (dtype == ONELLM_FP16) return launch_act<__half>((const __half*)input, (__half*)out, B, I, st);
+    return ONELLM_EINVAL;
+}

@@ -180,3 +180,36 @@ void launchTopKforBeamSearch(const float* probs, const int batch_size, const int
     const int rc = onellm_beam_topk(probs, batch_size, beamwidth, vocab_size, beamwidth, topk_workspace, nullptr);
     throw_on_error(rc, "launchTopKforBeamSearch");
 }
+
+// src/kernels/qkv_bias_and_RoPE.cu:167-207
+void launchAddFusedQKVBiasTransposeAndRoPE(Tensor* q_buf, Tensor* k_buf, Tensor* v_buf, Tensor* QKV, BaseWeight& qkv,
+                                           Tensor* padding_offset, Tensor* history_length, Tensor* input_length,
+                                           LLaMAAttentionStaticParams& params)
+{
+    (void)input_length;   // the reference only forms an unused value from it (:139)
+    ONELLM_CHECK_WITH_INFO(q_buf && k_buf && v_buf && QKV && padding_offset && history_length, "null tensor");
+    ONELLM_CHECK_WITH_INFO(QKV->shape.size() == 3 && q_buf->shape.size() == 4, "QKV must be [tokens, heads, D], q_buf [B, Hq, S, D]");
+    const int token_num = QKV->shape[0];               // :177
+    const int qkv_head_num = QKV->shape[1];            // :178
+    const int head_size = QKV->shape[2];               // :179
+    const int batch_size = q_buf->shape[0];            // :180
+    const int head_num = q_buf->shape[1];              // :181
+    const int seq_len = q_buf->shape[2];               // :182
+    const int kv_head_num = (qkv_head_num - head_num) / 2;   // :183
+    const int rc = onellm_qkv_bias_rope_transpose(abi_dtype(QKV, "launchAddFusedQKVBiasTransposeAndRoPE"), q_buf->data,
+                                                  k_buf->data, v_buf->data, QKV->data, qkv.bias,
+                                                  (const int*)padding_offset->data, (const int*)history_length->data,
+                                                  batch_size, seq_len, token_num, head_num, kv_head_num, head_size,
+                                                  params.rotary_embedding_dim, params.rotary_embedding_base, nullptr);
+    throw_on_error(rc, "launchAddFusedQKVBiasTransposeAndRoPE");
+}
+
+// src/kernels/activation_kernel.cu:24-34
+template <typename T>
+void launchAct(const T* input, T* out, const int batch_size, const int intermedia_size)
+{
+    const int dtype = std::is_same<T, half>::value ? ONELLM_FP16 : ONELLM_FP32;
+    throw_on_error(onellm_silu_and_mul(dtype, input, out, batch_size, intermedia_size, nullptr), "launchAct");
+}
+template void launchAct(const float*, float*, const int, const int);
+template void launchAct(const half*, half*, const int, const int);

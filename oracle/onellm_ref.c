@@ -458,3 +458,86 @@ int onellm_ref_beam_topk(const float* logits, int B, int beam, int V, int K, int
     }
     return 0;
 }
+
+/* ---------------------------------------------------------------- prefill: fused QKV bias + RoPE + un-pad transpose */
+
+/*
+ * Context-phase companion of the decode kernel (src/kernels/qkv_bias_and_RoPE.cu:74-161 kernel,
+ * :167-207 launcher).  For every packed token `tok` (no padding between sequences):
+ *   dst = tok + padding_offset[tok];  b = dst / seq_len;  s = dst % seq_len          (:97-104)
+ *   q[h]   = QKV[tok, h]          + bias[h*D..]                                      (:115-119)
+ *   k[kvh] = QKV[tok, Hq+kvh]     + bias[Hq*D + kvh*D..]                             (:123-128)
+ *   v[kvh] = QKV[tok, Hq+Hkv+kvh] + bias[(Hq+Hkv)*D + kvh*D..]                       (:130-134)
+ *   RoPE(q), RoPE(k) at the 0-based position history_length[b] + s                   (:138-143)
+ *   q_buf[b, h, s, :] = q;  k_buf[b, kvh, s, :] = k;  v_buf[b, kvh, s, :] = v        (:147-159)
+ * q_buf is [B, Hq, seq_len, D], k_buf/v_buf [B, Hkv, seq_len, D]; padded positions are not written.
+ * input_length is read by the reference only to form an unused value (:139) and is not needed.
+ * Same bias/RoPE arithmetic as the decode step above, so prefill and decode agree bit for bit.
+ */
+int onellm_ref_qkv_bias_rope_transpose(int dtype, void* q_buf, void* k_buf, void* v_buf, const void* qkv,
+                                       const void* qkv_bias, const int* padding_offset, const int* history_length,
+                                       int B, int seq_len, int token_num, int Hq, int Hkv, int D,
+                                       int rotary_dim, float rope_base)
+{
+    if (!q_buf || !k_buf || !v_buf || !qkv || !padding_offset || !history_length) return -1;
+    if (B <= 0 || seq_len <= 0 || token_num < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return -1;
+    const int QKVH = Hq + 2 * Hkv;
+    float* freq = (float*)malloc(sizeof(float) * (size_t)(D / 2 + 1));
+    onellm_ref_rope_freqs(freq, D, rotary_dim, rope_base);
+    int bad = 0;
+#pragma omp parallel for schedule(static)
+    for (int tok = 0; tok < token_num; ++tok) {
+        const long dst = (long)tok + padding_offset[tok];
+        const long b = dst / seq_len, s = dst % seq_len;
+        if (dst < 0 || b >= B) {
+#pragma omp atomic write
+            bad = 1;
+            continue;
+        }
+        const int pos = history_length[b] + (int)s;
+        float* row = (float*)malloc(sizeof(float) * (size_t)D);
+        for (int h = 0; h < QKVH; ++h) {
+            for (int d = 0; d < D; ++d) {
+                row[d] = ld(qkv, ((size_t)tok * QKVH + h) * D + d, dtype);
+                if (qkv_bias) row[d] += ld(qkv_bias, (size_t)h * D + d, dtype);
+            }
+            void* out;
+            size_t o;
+            if (h < Hq) {
+                onellm_ref_rope_row(row, D, rotary_dim, freq, pos);
+                out = q_buf;
+                o = (((size_t)b * Hq + h) * seq_len + (size_t)s) * D;
+            } else if (h < Hq + Hkv) {
+                onellm_ref_rope_row(row, D, rotary_dim, freq, pos);
+                out = k_buf;
+                o = (((size_t)b * Hkv + (h - Hq)) * seq_len + (size_t)s) * D;
+            } else {
+                out = v_buf;
+                o = (((size_t)b * Hkv + (h - Hq - Hkv)) * seq_len + (size_t)s) * D;
+            }
+            for (int d = 0; d < D; ++d) st(out, o + d, dtype, row[d]);
+        }
+        free(row);
+    }
+    free(freq);
+    return bad ? -1 : 0;
+}
+
+/* ---------------------------------------------------------------- SwiGLU */
+
+/*
+ * silu(x) * y over [B, 2, I] -> [B, I]  (src/kernels/activation_kernel.cu:5-22; CPU checker
+ * tests/unittests/test_activation.cu:12-22): silu(x) = x / (1 + expf(-x)) in fp32.
+ */
+int onellm_ref_silu_and_mul(int dtype, const void* input, void* out, int B, int I)
+{
+    if (!input || !out || B < 0 || I <= 0) return -1;
+#pragma omp parallel for schedule(static)
+    for (int b = 0; b < B; ++b)
+        for (int i = 0; i < I; ++i) {
+            const float x = ld(input, (size_t)b * 2 * I + i, dtype);
+            const float y = ld(input, (size_t)b * 2 * I + I + i, dtype);
+            st(out, (size_t)b * I + i, dtype, (x / (1.0f + expf(-x))) * y);
+        }
+    return 0;
+}

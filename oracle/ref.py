@@ -48,6 +48,8 @@ def lib():
         L.onellm_ref_kv_append.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci]
         L.onellm_ref_kv_repeat.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci]
         L.onellm_ref_beam_topk.argtypes = [vp, ci, ci, ci, ci, ci, vp]
+        L.onellm_ref_qkv_bias_rope_transpose.argtypes = [ci, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, cf]
+        L.onellm_ref_silu_and_mul.argtypes = [ci, vp, vp, ci, ci]
         _lib = L
     return _lib
 
@@ -172,3 +174,23 @@ def beam_topk(logits, B, beam, K, nblk=8):
     fv = ws[2 * n1:2 * n1 + B * K].reshape(B, K).copy()
     fi = ws[2 * n1 + B * K:].view(np.int32).reshape(B, K).copy()
     return vals, ids, fv, fi
+
+
+def qkv_bias_rope_transpose(q_buf, k_buf, v_buf, qkv, bias, padding_offset, history_length, rotary_dim, rope_base):
+    """qkv [token_num, Hq+2Hkv, D]; q_buf [B, Hq, seq_len, D]; k_buf/v_buf [B, Hkv, seq_len, D] (written in place)."""
+    token_num, QKVH, D = qkv.shape
+    B, Hq, seq_len, _ = q_buf.shape
+    Hkv = k_buf.shape[1]
+    assert QKVH == Hq + 2 * Hkv
+    po = np.ascontiguousarray(padding_offset, dtype=np.int32)
+    hl = np.ascontiguousarray(history_length, dtype=np.int32)
+    _chk(lib().onellm_ref_qkv_bias_rope_transpose(_dt(qkv), _p(q_buf), _p(k_buf), _p(v_buf), _p(qkv), _p(bias), _p(po),
+                                                  _p(hl), B, seq_len, token_num, Hq, Hkv, D, rotary_dim, rope_base),
+         "qkv_bias_rope_transpose")
+
+
+def silu_and_mul(inp, out):
+    B, two, I = inp.shape
+    assert two == 2 and out.shape == (B, I) and out.dtype == inp.dtype
+    _chk(lib().onellm_ref_silu_and_mul(_dt(inp), _p(inp), _p(out), B, I), "silu_and_mul")
+    return out

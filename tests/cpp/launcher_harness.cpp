@@ -111,6 +111,30 @@ int h_topk(const float* probs, int B, int V, float* ws)
     return guarded([&] { launchTopKforBeamSearch(probs, B, V, ws); });
 }
 
+int h_prefill_rope(int dtype, void* q, void* k, void* v, void* qkv, void* bias, void* padding_offset, void* history, void* input_len,
+                   int B, int S, int tokens, int Hq, int Hkv, int D, int rotary_dim, float base)
+{
+    return guarded([&] {
+        Tensor q_buf(GPU, dt(dtype), {B, Hq, S, D}, q), k_buf(GPU, dt(dtype), {B, Hkv, S, D}, k), v_buf(GPU, dt(dtype), {B, Hkv, S, D}, v);
+        Tensor QKV(GPU, dt(dtype), {tokens, Hq + 2 * Hkv, D}, qkv);
+        BaseWeight w;
+        w.data = nullptr;
+        w.type = dtype == 1 ? WeightType::FP16_W : WeightType::FP32_W;
+        w.bias = bias;
+        Tensor po(GPU, INT32, {B, S}, padding_offset), hist(GPU, INT32, {B}, history), in_len(GPU, INT32, {B}, input_len);
+        LLaMAAttentionStaticParams params{rotary_dim, base, 2048, false};
+        launchAddFusedQKVBiasTransposeAndRoPE(&q_buf, &k_buf, &v_buf, &QKV, w, &po, &hist, &in_len, params);
+    });
+}
+
+int h_act(int dtype, const void* input, void* out, int B, int I)
+{
+    return guarded([&] {
+        if (dtype == 1) launchAct<half>((const half*)input, (half*)out, B, I);
+        else launchAct<float>((const float*)input, (float*)out, B, I);
+    });
+}
+
 // the callers' pattern after every launch (src/layers/attention/masked_self_attention.cpp:73 in oneLLM)
 int h_sync_and_check()
 {

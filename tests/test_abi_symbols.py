@@ -19,7 +19,8 @@ def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ["onellm_decode_attn", "onellm_decode_attn_workspace_bytes", "onellm_rmsnorm",
                  "onellm_fused_add_bias_residual_rmsnorm", "onellm_kv_append", "onellm_kv_repeat",
-                 "onellm_beam_topk", "onellm_beam_topk_workspace_bytes", "onellm_error_string", "onellm_hip_version"]:
+                 "onellm_beam_topk", "onellm_beam_topk_workspace_bytes", "onellm_error_string", "onellm_hip_version",
+                 "onellm_qkv_bias_rope_transpose", "onellm_silu_and_mul"]:
         assert must in names
 
 
@@ -39,7 +40,10 @@ def test_launcher_library_exports_reference_signatures(capi):
                 "void launchFusedAddBiasResidualRMSNorm<__half>(__half*, __half*, __half const*, __half const*, float, int, int)",
                 "launchAppendKVCache(Tensor*, Tensor*, Tensor*, Tensor*, Tensor*, Tensor*, Tensor*)",
                 "launchTransposeKVCache(Tensor*, Tensor*, Tensor*, Tensor*, Tensor*, Tensor*)",
-                "launchTopKforBeamSearch(float const*, int, int, float*)"]:
+                "launchTopKforBeamSearch(float const*, int, int, float*)",
+                "launchAddFusedQKVBiasTransposeAndRoPE(Tensor*, Tensor*, Tensor*, Tensor*, BaseWeight&, Tensor*, Tensor*, Tensor*, LLaMAAttentionStaticParams&)",
+                "void launchAct<float>(float const*, float*, int, int)",
+                "void launchAct<__half>(__half const*, __half*, int, int)"]:
         assert sig in out, sig
 
 

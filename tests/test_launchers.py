@@ -27,6 +27,8 @@ def H():
     L.h_append.argtypes = [ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci]
     L.h_repeat.argtypes = [ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci]
     L.h_topk.argtypes = [vp, ci, ci, vp]
+    L.h_prefill_rope.argtypes = [ci, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, cf]
+    L.h_act.argtypes = [ci, vp, vp, ci, ci]
     return L
 
 
@@ -160,3 +162,31 @@ def test_launchTopKforBeamSearch_reference_layout(H, ref, dev):
     _, _, wfv, wfi = ref.beam_topk(logits, B, 2, 2)
     np.testing.assert_array_equal(w[off:off + B * 2].reshape(B, 2), wfv)
     np.testing.assert_array_equal(w.view(np.int32)[off + B * 2:off + 2 * B * 2].reshape(B, 2), wfi)
+
+
+@pytest.mark.gpu
+def test_launchAddFusedQKVBiasTransposeAndRoPE_and_launchAct(H, ref, dev):
+    import torch
+    announce("launchAddFusedQKVBiasTransposeAndRoPE / launchAct")
+    rng = np.random.default_rng(6)
+    B, S, Hq, Hkv, D = 2, 16, 4, 2, 64
+    lens = [16, 9]
+    T = sum(lens)
+    po = np.array([0] * 16 + [16 + s - (16 + s) + 0 for s in range(9)], np.int32)    # packed: second sequence starts at token 16 = slot 16
+    hist = np.array([3, 100], np.int32)
+    qkv = rng.standard_normal((T, Hq + 2 * Hkv, D)).astype(np.float32)
+    bias = rng.standard_normal((Hq + 2 * Hkv) * D).astype(np.float32)
+    q = np.zeros((B, Hq, S, D), np.float32); k = np.zeros((B, Hkv, S, D), np.float32); v = np.zeros_like(k)
+    d = [_dev(a, dev) for a in (q, k, v, qkv, bias, po, hist, np.array(lens, np.int32))]
+    assert H.h_prefill_rope(0, *[t.data_ptr() for t in d], B, S, T, Hq, Hkv, D, D, 10000.0) == 0, H.h_last_error()
+    ref.qkv_bias_rope_transpose(q, k, v, qkv, bias, po, hist, D, 10000.0)
+    for got, want in zip(d[:3], (q, k, v)):
+        np.testing.assert_array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    for dtype, code in ((np.float32, 0), (np.float16, 1)):
+        inp = (rng.standard_normal((5, 2, 11008)) * 2).astype(dtype)
+        out = torch.zeros(5, 11008, dtype=torch.float32 if code == 0 else torch.float16, device=dev)
+        assert H.h_act(code, _dev(inp, dev).data_ptr(), out.data_ptr(), 5, 11008) == 0, H.h_last_error()
+        want = ref.silu_and_mul(inp, np.zeros((5, 11008), dtype))
+        tol = dict(rtol=1e-5, atol=1e-6) if code == 0 else dict(rtol=1e-2, atol=2e-3)
+        np.testing.assert_allclose(out.cpu().numpy().astype(np.float64), want.astype(np.float64), **tol)
+    assert H.h_sync_and_check() == 0
