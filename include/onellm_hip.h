@@ -73,8 +73,9 @@ const char* onellm_error_string(int code);
  *
  * Arithmetic is fp32 throughout; with ONELLM_FP16 the cache, qkv, bias and out are fp16 and the
  * new k/v rows are rounded to fp16 before they take part in this step's scores.
- * Supported shapes: D*sizeof(elt) a power of two in [16, 1024] bytes, Hq % Hkv == 0, 1 <= t <= S,
- * caches 16-byte aligned.
+ * Shapes: Hq % Hkv == 0, 1 <= t <= S, D <= 512, B <= 65535.  Head sizes whose rows are a power of
+ * two number of bytes (16..1024) in 16-byte aligned caches run the tiled kernels; anything else
+ * (D = 96, 80, ..., odd D, unaligned caches) runs a slower scalar kernel with the same results.
  */
 int onellm_decode_attn(int dtype,
                        const void* qkv, const void* qkv_bias,

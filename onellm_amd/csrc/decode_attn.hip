@@ -333,6 +333,137 @@ void decode_attn_merge_kernel(const AttnArgs a, int D)
     }
 }
 
+// Any head size up to 512 and any alignment: one workgroup per (sequence, query head), scalar
+// accesses, no sequence split, grouped-query heads each re-read their kv-head's rows.  Same
+// arithmetic and the same cache write as the tiled kernel; a correctness path for head sizes
+// whose rows are not a power-of-two number of bytes (96, 80, ...), not a performance path.
+template <typename T>
+__global__ __launch_bounds__(256)
+void decode_attn_generic_kernel(const AttnArgs a, const RopeFreqs fr, int D)
+{
+    constexpr int NW = 4, MAXJ = 2 * kMaxPairs / kWave;       // elements of a row per lane
+    extern __shared__ float lds[];
+    float* sq = lds;                  // [D]
+    float* sk = sq + D;               // [D]
+    float* sv = sk + D;               // [D]
+    float* st_ml = sv + D;            // [NW][2]
+    float* st_acc = st_ml + NW * 2;   // [NW][D]
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int kvh = h / a.G;
+    const int t = a.t_dev ? a.t_dev[b] : a.t_host;
+    if (t < 1 || t > a.S) return;
+    const int pos = t + a.pos_offset;
+    const T* qkv = static_cast<const T*>(a.qkv) + (size_t)b * (a.Hq + 2 * a.Hkv) * D;
+    const T* bias = static_cast<const T*>(a.bias);
+    const size_t head_off = a.slab + ((size_t)b * a.Hkv + kvh) * (size_t)a.S * D;
+    T* kc = static_cast<T*>(a.k_cache) + head_off;
+    T* vc = static_cast<T*>(a.v_cache) + head_off;
+    const bool store = (h % a.G) == 0 && !(a.flags & ONELLM_ATTN_NO_CACHE_WRITE);
+
+    // q, new k, new v: bias, RoPE on the pairs that exist, staging in LDS (an odd last element is not rotated)
+    for (int p = tid; 2 * p < D; p += 256) {
+        const bool pair = 2 * p + 1 < D;
+        const int oq = h * D + 2 * p, ok = (a.Hq + kvh) * D + 2 * p;
+        float q0 = to_f32(qkv[oq]), q1 = pair ? to_f32(qkv[oq + 1]) : 0.f;
+        float k0 = to_f32(qkv[ok]), k1 = pair ? to_f32(qkv[ok + 1]) : 0.f;
+        if (bias) {
+            q0 += to_f32(bias[oq]);
+            k0 += to_f32(bias[ok]);
+            if (pair) {
+                q1 += to_f32(bias[oq + 1]);
+                k1 += to_f32(bias[ok + 1]);
+            }
+        }
+        if (pair && 2 * p < a.rotary_dim) {
+            rope_pair(q0, q1, p, pos, fr);
+            rope_pair(k0, k1, p, pos, fr);
+        }
+        sq[2 * p] = q0 * a.qscale;
+        const T ks0 = from_f32<T>(k0);
+        sk[2 * p] = to_f32(ks0);
+        if (store) kc[(size_t)(t - 1) * D + 2 * p] = ks0;
+        if (pair) {
+            sq[2 * p + 1] = q1 * a.qscale;
+            const T ks1 = from_f32<T>(k1);
+            sk[2 * p + 1] = to_f32(ks1);
+            if (store) kc[(size_t)(t - 1) * D + 2 * p + 1] = ks1;
+        }
+    }
+    for (int d = tid; d < D; d += 256) {
+        const int o = (a.Hq + a.Hkv + kvh) * D + d;
+        float x = to_f32(qkv[o]);
+        if (bias && !(a.flags & ONELLM_ATTN_NO_V_BIAS)) x += to_f32(bias[o]);
+        const T v = from_f32<T>(x);
+        sv[d] = to_f32(v);
+        if (store) vc[(size_t)(t - 1) * D + d] = v;
+    }
+    __syncthreads();
+
+    float qr[MAXJ], acc[MAXJ];
+#pragma unroll
+    for (int j = 0; j < MAXJ; ++j) {
+        const int d = lane + j * kWave;
+        qr[j] = d < D ? sq[d] : 0.f;
+        acc[j] = 0.f;
+    }
+    float m = -INFINITY, l = 0.f;
+    auto row_step = [&](auto&& kget, auto&& vget) {
+        float part = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+            const int d = lane + j * kWave;
+            if (d < D) part = fmaf(qr[j], kget(d), part);
+        }
+        const float sc = wave_sum(part);
+        const float mx = fmaxf(m, sc);
+        const float alpha = __builtin_amdgcn_exp2f(m - mx), pr = __builtin_amdgcn_exp2f(sc - mx);
+        l = fmaf(l, alpha, pr);
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+            const int d = lane + j * kWave;
+            if (d < D) acc[j] = fmaf(pr, vget(d), acc[j] * alpha);
+        }
+        m = mx;
+    };
+    for (int r = wave; r < t - 1; r += NW) {
+        const T* kr = kc + (size_t)r * D;
+        const T* vr = vc + (size_t)r * D;
+        row_step([&](int d) { return to_f32(kr[d]); }, [&](int d) { return to_f32(vr[d]); });
+    }
+    if (wave == 0) row_step([&](int d) { return sk[d]; }, [&](int d) { return sv[d]; });   // the new token's row
+
+    if (lane == 0) {
+        st_ml[wave * 2] = m;
+        st_ml[wave * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int j = 0; j < MAXJ; ++j) {
+        const int d = lane + j * kWave;
+        if (d < D) st_acc[wave * D + d] = acc[j];
+    }
+    __syncthreads();
+    for (int d = tid; d < D; d += 256) {
+        float M = -INFINITY;
+        for (int w = 0; w < NW; ++w) M = fmaxf(M, st_ml[w * 2]);      // wave 0 always holds the new row: M is finite
+        float L = 0.f, O = 0.f;
+        for (int w = 0; w < NW; ++w) {
+            const float wt = __builtin_amdgcn_exp2f(st_ml[w * 2] - M);
+            L = fmaf(st_ml[w * 2 + 1], wt, L);
+            O = fmaf(st_acc[w * D + d], wt, O);
+        }
+        static_cast<T*>(a.out)[((size_t)b * a.Hq + h) * D + d] = from_f32<T>(O / L);
+    }
+}
+
+template <typename T>
+int launch_generic(const AttnArgs& a, const RopeFreqs& fr, int D, hipStream_t st)
+{
+    const size_t lds_bytes = sizeof(float) * (size_t)(3 * D + 8 + 4 * D);
+    hipLaunchKernelGGL((decode_attn_generic_kernel<T>), dim3(a.Hq, a.B), dim3(256), lds_bytes, st, a, fr, D);
+    return launch_status();
+}
+
 constexpr int kMaxSplits = 64;      // upper bound of splits the workspace is sized for
 constexpr int kMinChunk = 64;       // never split finer than this many cache rows
 
@@ -413,8 +544,11 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     if (rotary_dim < 0 || (rotary_dim > 0 && !(rope_base > 0.f))) return ONELLM_EINVAL;
     const int esz = dtype == ONELLM_FP16 ? 2 : 4;
     const int row_bytes = D * esz;
-    if (row_bytes < 16 || row_bytes > 1024 || (row_bytes & (row_bytes - 1))) return ONELLM_EUNSUPPORTED;
-    if (!aligned16(k_cache) || !aligned16(v_cache)) return ONELLM_EUNSUPPORTED;
+    if (D > 2 * kMaxPairs || B > 65535) return ONELLM_EUNSUPPORTED;
+    // rows of a power-of-two number of bytes in 16-byte aligned caches take the tiled kernels; any
+    // other head size or alignment takes the scalar kernel
+    const bool tiled = row_bytes >= 16 && row_bytes <= 1024 && !(row_bytes & (row_bytes - 1)) && aligned16(k_cache)
+                       && aligned16(v_cache);
     const int lpr = row_bytes / 16;
 
     AttnArgs a{};
@@ -424,6 +558,13 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     a.rotary_dim = rotary_dim; a.pos_offset = rope_pos_offset; a.flags = flags;
     a.qscale = (1.0f / sqrtf((float)D)) * 1.4426950408889634f;
     a.slab = (size_t)layer * B * Hkv * (size_t)S * D;
+
+    if (!tiled) {
+        RopeFreqs frg;
+        fill_rope_freqs(frg, D, rotary_dim, rope_base);
+        hipStream_t stg = static_cast<hipStream_t>(stream);
+        return dtype == ONELLM_FP16 ? launch_generic<__half>(a, frg, D, stg) : launch_generic<float>(a, frg, D, stg);
+    }
 
     // Sequence split, from sweeps on MI355X.  Equal lengths (t_dev == NULL): about one workgroup per
     // compute unit with chunks of at least 512 rows (more, smaller workgroups only add per-workgroup

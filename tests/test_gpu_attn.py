@@ -99,6 +99,40 @@ def test_shapes_and_lengths(capi, ref, dev, dtype, Hq, Hkv, D, t):
     _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), dtype)
 
 
+@pytest.mark.parametrize("dtype,Hq,Hkv,D", [(np.float16, 4, 2, 96), (np.float16, 8, 8, 80), (np.float32, 2, 1, 7),
+                                            (np.float32, 3, 3, 100), (np.float16, 2, 1, 2), (np.float32, 2, 2, 1),
+                                            (np.float16, 2, 1, 500)])
+@pytest.mark.parametrize("t", [1, 2, 70])
+def test_head_sizes_outside_the_tiled_kernels(capi, ref, dev, dtype, Hq, Hkv, D, t):
+    # rows that are not a power-of-two number of bytes run the scalar kernel: same parity bars
+    announce("attn generic", dtype.__name__, Hq, Hkv, D, "t", t)
+    qkv, bias, kc, vc = _case(dtype, 2, Hq, Hkv, D, 72, 2, seed=D * 7 + t, std=0.5)
+    _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D, layer=1), dtype)
+    lens = np.array([t, max(1, t // 2)])
+    _assert_parity(_run_both(capi, ref, dev, qkv, None, kc, vc, Hq, lens, D - D % 2), dtype)
+
+
+def test_unaligned_cache_takes_the_scalar_kernel(capi, ref, dev):
+    announce("attn unaligned cache")
+    qkv, bias, kc, vc = _case(np.float16, 2, 4, 2, 64, 40, 1, seed=77, std=0.5)
+    d_qkv, d_bias = torch.from_numpy(qkv).to(dev), torch.from_numpy(bias).to(dev)
+    n = kc.size
+    kbuf = torch.zeros(n + 8, dtype=torch.float16, device=dev)
+    vbuf = torch.zeros(n + 8, dtype=torch.float16, device=dev)
+    d_kc, d_vc = kbuf[1:1 + n].view(kc.shape), vbuf[1:1 + n].view(vc.shape)      # 2 bytes off a 16-byte boundary
+    d_kc.copy_(torch.from_numpy(kc)); d_vc.copy_(torch.from_numpy(vc))
+    out = torch.zeros(2, 4 * 64, dtype=torch.float16, device=dev)
+    rc = capi.lib().onellm_decode_attn(capi.FP16, d_qkv.data_ptr(), d_bias.data_ptr(), d_kc.data_ptr(), d_vc.data_ptr(),
+                                       out.data_ptr(), 2, 4, 2, 64, 40, 0, 1, 33, None, 33, 64, 10000.0, 0, 0, None, 0,
+                                       torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    want = ref.decode_attn(qkv, bias, kc, vc, 4, 33, 64, 10000.0)
+    np.testing.assert_allclose(out.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[np.float16])
+    np.testing.assert_array_equal(_bits(d_kc.cpu().numpy()), _bits(kc))
+    np.testing.assert_array_equal(_bits(d_vc.cpu().numpy()), _bits(vc))
+    assert kbuf[0].item() == 0 and kbuf[n + 1].item() == 0
+
+
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 @pytest.mark.parametrize("nsplit", [1, 2, 5, 64])
 def test_sequence_split_counts_and_ragged_lengths(capi, ref, dev, dtype, nsplit):

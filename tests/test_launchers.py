@@ -53,7 +53,7 @@ def test_precondition_failures_throw_without_touching_the_gpu(H):
     assert H.h_decode_mha(0, fake, None, fake, fake, fake, 1, 2, 1, 16, 32, 1, 33, 0, 128, 10000.0) == 1
     assert b"step outside" in H.h_last_error()
     # a head size the kernels are not built for: rejected by the C ABI before any launch, surfaces as [TM][ERROR]
-    assert H.h_decode_mha(0, fake, None, fake, fake, fake, 1, 2, 1, 24, 32, 1, 4, 0, 128, 10000.0) == 1
+    assert H.h_decode_mha(0, fake, None, fake, fake, fake, 1, 2, 1, 600, 32, 1, 4, 0, 128, 10000.0) == 1
     assert b"[TM][ERROR] launchDecoderMaskedMHA" in H.h_last_error()
     assert H.h_topk(None, 1, 100, fake) == 1
     assert b"launchTopKforBeamSearch" in H.h_last_error()
