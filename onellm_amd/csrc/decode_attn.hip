@@ -92,6 +92,26 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     T* kc = static_cast<T*>(a.k_cache) + head_off;
     T* vc = static_cast<T*>(a.v_cache) + head_off;
 
+    // ---- the first rows of the chunk are requested before anything else: they do not depend on q,
+    // and their latency then hides the q / new-row set-up below
+    const int col = (lane % LPR) * VEC;         // first of this lane's VEC columns
+    const int rg = wave * RPW + lane / LPR;     // row group of this lane
+    constexpr int RPI = U * NRG;                // rows per workgroup iteration
+    const T* kp = kc + col;
+    const T* vp = vc + col;
+    // loads of one iteration: U cache rows of K and of V per row group
+    auto issue = [&](Vec16<T> (&kv)[U], Vec16<T> (&vv)[U], int rbase) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int row = rbase + u * NRG + rg;
+            kv[u] = load16_stream(kp + (size_t)row * D);
+            vv[u] = load16_stream(vp + (size_t)row * D);
+        }
+    };
+    const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
+    Vec16<T> ka[U], va[U], kb[U], vb[U];
+    if (nfull > 0) issue(ka, va, r0);
+
     // ---- q (and, in the last split, the new k/v row): bias, RoPE, staging in LDS
     for (int i = tid; i < GT * (D / 2); i += NTHR) {
         const int g = i / (D / 2), p = i % (D / 2);
@@ -138,7 +158,6 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     }
     __syncthreads();
 
-    const int col = (lane % LPR) * VEC;         // first of this lane's VEC columns
     float qr[GT][VEC];
 #pragma unroll
     for (int g = 0; g < GT; ++g)
@@ -165,20 +184,6 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
         for (int e = 0; e < VEC; ++e) acc[g][e] = 0.f;
     }
 
-    const int rg = wave * RPW + lane / LPR;     // row group of this lane
-    constexpr int RPI = U * NRG;                // rows per workgroup iteration
-    const T* kp = kc + col;
-    const T* vp = vc + col;
-
-    // loads of one iteration: U cache rows of K and of V per row group
-    auto issue = [&](Vec16<T> (&kv)[U], Vec16<T> (&vv)[U], int rbase) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int row = rbase + u * NRG + rg;
-            kv[u] = load16_stream(kp + (size_t)row * D);
-            vv[u] = load16_stream(vp + (size_t)row * D);
-        }
-    };
     // scores, online softmax and weighted V sum for the rows held in (kv, vv); `valid` masks rows
     // past the end of the chunk in the tail iteration
     auto consume = [&](const Vec16<T> (&kv)[U], const Vec16<T> (&vv)[U], const bool (&valid)[U], auto masked_tag) {
@@ -226,11 +231,8 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
         // Full iterations are software-pipelined over two register buffers: the loads of the next
         // iteration are in flight while the current one is consumed, so a wave never sits with an
         // empty memory queue.  The (at most one) partial iteration at the end is masked.
-        const int nfull = (r1 - r0) / RPI;
         const bool none[U] = {};
-        Vec16<T> ka[U], va[U], kb[U], vb[U];
         int rbase = r0;
-        if (nfull > 0) issue(ka, va, rbase);
         for (int it = 0; it < nfull; it += 2) {
             if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
             consume(ka, va, none, std::false_type{});
