@@ -6,6 +6,7 @@
 #include "onellm/base_weights.h"
 #include "onellm/norm_weights.h"
 #include "onellm/llama_params.h"
+#include "onellm/params.h"
 
 // src/kernels/decoder_masked_attn.h:7-14
 void launchDecoderMaskedMHA(Tensor* qkv_buf,
@@ -67,3 +68,11 @@ void launchAddFusedQKVBiasTransposeAndRoPE(Tensor* q_buf,
 // src/kernels/activation_kernel.h (float as in the reference, half added)
 template<typename T>
 void launchAct(const T* input, T* out, const int batch_size, const int intermedia_size);
+
+// src/kernels/topK_sampling.h
+void launchSampling(Tensor* topk_id,
+                    Tensor* topk_val,
+                    Tensor* seqlen,
+                    Tensor* is_finished,
+                    Tensor* output_id,
+                    IntDict& params);

@@ -180,6 +180,21 @@ int onellm_qkv_bias_rope_transpose(int dtype, void* q_buf, void* k_buf, void* v_
  */
 int onellm_silu_and_mul(int dtype, const void* input, void* out, int B, int I, onellm_stream_t stream);
 
+/*
+ * Top-K sampling: the consumer of the beam top-K output.  Replaces launchSampling
+ * (src/kernels/topK_sampling.h, src/kernels/topK_sampling.cu:6-70).  Per batch row, with the K
+ * (value, id) pairs sorted best-first:  w_i = exp(val_i - val_0);  thr = u * sum(w);  the first i whose
+ * running subtraction takes thr below 0 wins (the last one if rounding never does);
+ *   output_id = topk_id[i] % vocab_size;  seqlen += 1 unless is_finished;  is_finished = (output_id == end_id).
+ * topk_id int32 [B, K], topk_val fp32 [B, K] (not modified), output_id / seqlen int32 [B],
+ * is_finished one byte per row (C++ bool).  u comes from Philox4x32-10 with key = seed (the reference
+ * passes the step) and counter = (row, 0, 0, 0): reproducible on a CPU, but NOT the stream cuRAND's
+ * XORWOW would give the reference.
+ */
+int onellm_topk_sample(const int* topk_id, const float* topk_val, int* output_id, int* seqlen,
+                       unsigned char* is_finished, int B, int K, unsigned long long seed, int end_id,
+                       int vocab_size, onellm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

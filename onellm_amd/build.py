@@ -25,7 +25,7 @@ LIB_LAUNCH = os.path.join(HERE, "libonellm_launchers.so")
 HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "launcher_harness.cpp")
 LIB_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
 
-KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip",
+KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip", "sampling.hip",
                   "tuning.cpp"]
 LAUNCHER_SOURCES = ["launchers.cpp"]
 

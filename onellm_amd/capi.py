@@ -33,6 +33,7 @@ SYMBOLS = {
     "onellm_qkv_bias_rope_transpose": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci,
                                              _cf, _vp]),
     "onellm_silu_and_mul": (_ci, [_ci, _vp, _vp, _ci, _ci, _vp]),
+    "onellm_topk_sample": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, ctypes.c_ulonglong, _ci, _ci, _vp]),
 }
 
 _lib = None
@@ -185,3 +186,11 @@ def silu_and_mul(inp, out):
     assert two == 2
     _check(lib().onellm_silu_and_mul(_dt(inp), _ptr(inp), _ptr(out), B, I, _stream()), "onellm_silu_and_mul")
     return out
+
+
+def topk_sample(topk_id, topk_val, output_id, seqlen, is_finished, seed, end_id, vocab_size):
+    """topk_id int32 [B, K]; topk_val fp32 [B, K]; output_id, seqlen int32 [B]; is_finished bool/uint8 [B]."""
+    B, K = topk_id.shape
+    _check(lib().onellm_topk_sample(_ptr(topk_id), _ptr(topk_val), _ptr(output_id), _ptr(seqlen), _ptr(is_finished), B, K,
+                                    int(seed), end_id, vocab_size, _stream()), "onellm_topk_sample")
+    return output_id

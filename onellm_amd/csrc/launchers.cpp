@@ -213,3 +213,19 @@ void launchAct(const T* input, T* out, const int batch_size, const int intermedi
 }
 template void launchAct(const float*, float*, const int, const int);
 template void launchAct(const half*, half*, const int, const int);
+
+// src/kernels/topK_sampling.cu:43-70
+void launchSampling(Tensor* topk_id, Tensor* topk_val, Tensor* seqlen, Tensor* is_finished, Tensor* output_id, IntDict& params)
+{
+    ONELLM_CHECK_WITH_INFO(topk_id && topk_val && seqlen && is_finished && output_id, "null tensor");
+    ONELLM_CHECK_WITH_INFO(topk_id->shape.size() == 2, "topk_id must be [batch, K]");
+    ONELLM_CHECK_WITH_INFO(params.count("vocab_size") && params.count("step") && params.count("end_id"),
+                           "params need vocab_size, step and end_id");
+    const int batch_size = topk_id->shape[0];          // :49
+    const int K = topk_id->shape[1];                   // :50
+    const int rc = onellm_topk_sample((const int*)topk_id->data, (const float*)topk_val->data, (int*)output_id->data,
+                                      (int*)seqlen->data, (unsigned char*)is_finished->data, batch_size, K,
+                                      (unsigned long long)(unsigned)params["step"], params["end_id"], params["vocab_size"],
+                                      nullptr);
+    throw_on_error(rc, "launchSampling");
+}

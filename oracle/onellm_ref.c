@@ -21,9 +21,13 @@
  * sin/cos in the test-suite.
  *
  * Parity status: every function below is pinned by known-answer tests taken from the reference's
- * own unit tests and by independent float64 formulations (tests/test_oracle_*.py); none is
- * "parity unpinned".  Tie order of the beam top-K is fixed by the task statement (lower index
- * wins), not by a reference test.
+ * own unit tests and by independent float64 formulations (tests/test_oracle_*.py), with one
+ * exception.  onellm_ref_topk_sample: the random draw is "parity unpinned" against the reference,
+ * whose uniform comes from cuRAND's XORWOW generator (a CUDA-toolkit library, not vendored, no
+ * version pinned, absent here); everything around the draw (weights, threshold walk, id % vocab,
+ * seqlen / finished bookkeeping) and the Philox generator used instead are pinned.
+ * Tie order of the beam top-K is fixed by the task statement (lower index wins), not by a
+ * reference test.
  */
 #include <math.h>
 #include <stdint.h>
@@ -539,5 +543,94 @@ int onellm_ref_silu_and_mul(int dtype, const void* input, void* out, int B, int 
             const float y = ld(input, (size_t)b * 2 * I + I + i, dtype);
             st(out, (size_t)b * I + i, dtype, (x / (1.0f + expf(-x))) * y);
         }
+    return 0;
+}
+
+/* ---------------------------------------------------------------- top-K sampling */
+
+/*
+ * Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11): counter-based,
+ * so a CPU and a GPU produce the same stream from (key, counter) alone.  The reference draws its
+ * uniform from cuRAND's XORWOW generator (src/kernels/topK_sampling.cu:28-30, `curand_init(step,
+ * batch_id, 0)` + `curand_uniform`); cuRAND is a CUDA-toolkit library that is neither vendored in
+ * the reference tree nor available here, so THAT stream is not reproduced: the random draw is
+ * "parity unpinned" against the reference, and pinned only against this restatement (itself
+ * checked on the published Philox known-answer vectors).
+ */
+void onellm_ref_philox4x32_10(const uint32_t ctr_in[4], const uint32_t key_in[2], uint32_t out[4])
+{
+    uint32_t c0 = ctr_in[0], c1 = ctr_in[1], c2 = ctr_in[2], c3 = ctr_in[3];
+    uint32_t k0 = key_in[0], k1 = key_in[1];
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* uniform in (0, 1]: (x + 1) * 2^-32 evaluated as x * 2^-32 + 2^-32 in fp32 (one fma) */
+float onellm_ref_uniform_from_u32(uint32_t x) { return fmaf((float)x, 0x1.0p-32f, 0x1.0p-32f); }
+
+/* e^x for x <= 0 as a fixed fp32 sequence (same idea as the sin/cos above): n = rint(x*log2 e),
+ * r = x - n*ln2 in two fma steps, degree-6 polynomial by Horner with fma, scale by 2^n through the
+ * exponent field; below 2^-126 the result is 0. */
+float onellm_ref_exp_fixed(float x)
+{
+    const float n = rintf(x * 0x1.715476p+0f);
+    float r = fmaf(-n, 0x1.62e400p-1f, x);
+    r = fmaf(-n, 0x1.7f7d1cp-20f, r);
+    float p = fmaf(0x1.6c16c2p-10f, r, 0x1.111112p-7f);    /* 1/720, 1/120 */
+    p = fmaf(p, r, 0x1.555556p-5f);                         /* 1/24 */
+    p = fmaf(p, r, 0x1.555556p-3f);                         /* 1/6 */
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    const int e = (int)n;
+    if (e < -126) return 0.0f;
+    union { uint32_t u; float f; } s;
+    s.u = (uint32_t)(e + 127) << 23;
+    return p * s.f;
+}
+
+/*
+ * Top-K sampling (src/kernels/topK_sampling.cu:6-41 kernel, :43-70 launcher).  Per batch row:
+ *   w_i = exp(val_i - val_0)                      (:20-21; val_0 is the maximum, the row is sorted)
+ *   sum = w_0 + ... + w_{K-1}, added in that order (:24-27)
+ *   thr = u * sum, u uniform in (0, 1]            (:28-30)
+ *   walk i = 0..K-1: thr -= w_i; first i with thr < 0 wins (:31-37).  The snapshot subtracts the
+ *     same element every time (`topk_val[offset]` with thread 0's offset, :32); the walk over w_i is
+ *     what the loop is for and is what is restated.  If rounding leaves thr >= 0 after the last
+ *     element, the last element wins (the snapshot would leave the output unwritten).
+ *   output_id = topk_id[i] % vocab_size           (:34)
+ *   seqlen += 1 unless already finished (:38);  is_finished = (output_id == end_id) (:39)
+ * The snapshot also overwrites topk_val with the w_i (:21); this restatement leaves the inputs alone.
+ * RNG: Philox4x32-10, key = (seed low word, seed high word) with seed = the reference's `rand_num`
+ * (the step), counter = (batch row, 0, 0, 0), first output word.
+ */
+int onellm_ref_topk_sample(const int* topk_id, const float* topk_val, int* output_id, int* seqlen,
+                           unsigned char* is_finished, int B, int K, unsigned long long seed, int end_id, int vocab_size)
+{
+    if (!topk_id || !topk_val || !output_id || !seqlen || !is_finished || B < 0 || K <= 0 || vocab_size <= 0) return -1;
+    for (int b = 0; b < B; ++b) {
+        const float* v = topk_val + (size_t)b * K;
+        float sum = 0.0f;
+        for (int i = 0; i < K; ++i) sum += onellm_ref_exp_fixed(v[i] - v[0]);
+        const uint32_t ctr[4] = {(uint32_t)b, 0, 0, 0}, key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+        uint32_t rnd[4];
+        onellm_ref_philox4x32_10(ctr, key, rnd);
+        float thr = onellm_ref_uniform_from_u32(rnd[0]) * sum;
+        int pick = K - 1;
+        for (int i = 0; i < K; ++i) {
+            thr -= onellm_ref_exp_fixed(v[i] - v[0]);
+            if (thr < 0) { pick = i; break; }
+        }
+        output_id[b] = topk_id[(size_t)b * K + pick] % vocab_size;
+        seqlen[b] = is_finished[b] ? seqlen[b] : seqlen[b] + 1;
+        is_finished[b] = output_id[b] == end_id ? 1 : 0;
+    }
     return 0;
 }

@@ -50,6 +50,13 @@ def lib():
         L.onellm_ref_beam_topk.argtypes = [vp, ci, ci, ci, ci, ci, vp]
         L.onellm_ref_qkv_bias_rope_transpose.argtypes = [ci, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, cf]
         L.onellm_ref_silu_and_mul.argtypes = [ci, vp, vp, ci, ci]
+        L.onellm_ref_philox4x32_10.argtypes = [vp, vp, vp]
+        L.onellm_ref_philox4x32_10.restype = None
+        L.onellm_ref_uniform_from_u32.argtypes = [ctypes.c_uint32]
+        L.onellm_ref_uniform_from_u32.restype = cf
+        L.onellm_ref_exp_fixed.argtypes = [cf]
+        L.onellm_ref_exp_fixed.restype = cf
+        L.onellm_ref_topk_sample.argtypes = [vp, vp, vp, vp, vp, ci, ci, ctypes.c_ulonglong, ci, ci]
         _lib = L
     return _lib
 
@@ -193,4 +200,32 @@ def silu_and_mul(inp, out):
     B, two, I = inp.shape
     assert two == 2 and out.shape == (B, I) and out.dtype == inp.dtype
     _chk(lib().onellm_ref_silu_and_mul(_dt(inp), _p(inp), _p(out), B, I), "silu_and_mul")
+    return out
+
+
+def philox4x32_10(ctr, key):
+    c = np.asarray(ctr, dtype=np.uint32).copy()
+    k = np.asarray(key, dtype=np.uint32).copy()
+    out = np.zeros(4, np.uint32)
+    lib().onellm_ref_philox4x32_10(_p(c), _p(k), _p(out))
+    return out
+
+
+def uniform_from_u32(x):
+    return lib().onellm_ref_uniform_from_u32(int(x))
+
+
+def exp_fixed(x):
+    return lib().onellm_ref_exp_fixed(float(x))
+
+
+def topk_sample(topk_id, topk_val, seqlen, is_finished, seed, end_id, vocab_size):
+    """topk_id int32 [B, K], topk_val fp32 [B, K] sorted best-first; seqlen int32 [B] and is_finished uint8 [B]
+    are updated in place.  Returns output_id int32 [B]."""
+    B, K = topk_id.shape
+    assert topk_id.dtype == np.int32 and topk_val.dtype == np.float32 and seqlen.dtype == np.int32
+    assert is_finished.dtype == np.uint8
+    out = np.zeros(B, np.int32)
+    _chk(lib().onellm_ref_topk_sample(_p(topk_id), _p(topk_val), _p(out), _p(seqlen), _p(is_finished), B, K,
+                                      int(seed), end_id, vocab_size), "topk_sample")
     return out

@@ -135,6 +135,19 @@ int h_act(int dtype, const void* input, void* out, int B, int I)
     });
 }
 
+int h_sampling(void* topk_id, void* topk_val, void* seqlen, void* finished, void* out, int B, int K, int step, int end_id, int vocab)
+{
+    return guarded([&] {
+        Tensor id(GPU, INT32, {B, K}, topk_id), val(GPU, FP32, {B, K}, topk_val), sl(GPU, INT32, {B}, seqlen);
+        Tensor fin(GPU, BOOL, {B}, finished), o(GPU, INT32, {B}, out);
+        IntDict params;
+        params.insert({"step", step});
+        params.insert({"vocab_size", vocab});
+        params.insert({"end_id", end_id});
+        launchSampling(&id, &val, &sl, &fin, &o, params);
+    });
+}
+
 // the callers' pattern after every launch (src/layers/attention/masked_self_attention.cpp:73 in oneLLM)
 int h_sync_and_check()
 {

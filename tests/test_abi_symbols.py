@@ -20,7 +20,7 @@ def test_header_declares_the_expected_entry_points():
     for must in ["onellm_decode_attn", "onellm_decode_attn_workspace_bytes", "onellm_rmsnorm",
                  "onellm_fused_add_bias_residual_rmsnorm", "onellm_kv_append", "onellm_kv_repeat",
                  "onellm_beam_topk", "onellm_beam_topk_workspace_bytes", "onellm_error_string", "onellm_hip_version",
-                 "onellm_qkv_bias_rope_transpose", "onellm_silu_and_mul"]:
+                 "onellm_qkv_bias_rope_transpose", "onellm_silu_and_mul", "onellm_topk_sample"]:
         assert must in names
 
 
@@ -43,7 +43,8 @@ def test_launcher_library_exports_reference_signatures(capi):
                 "launchTopKforBeamSearch(float const*, int, int, float*)",
                 "launchAddFusedQKVBiasTransposeAndRoPE(Tensor*, Tensor*, Tensor*, Tensor*, BaseWeight&, Tensor*, Tensor*, Tensor*, LLaMAAttentionStaticParams&)",
                 "void launchAct<float>(float const*, float*, int, int)",
-                "void launchAct<__half>(__half const*, __half*, int, int)"]:
+                "void launchAct<__half>(__half const*, __half*, int, int)",
+                "launchSampling(Tensor*, Tensor*, Tensor*, Tensor*, Tensor*, std::unordered_map<"]:
         assert sig in out, sig
 
 

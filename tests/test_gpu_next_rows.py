@@ -120,3 +120,38 @@ def test_swiglu_reference_unit_vector(capi, dev):
     x, y = inp[:, 0].double(), inp[:, 1].double()
     want = x / (1 + torch.exp(-x)) * y
     assert ((out.double() - want).abs() <= 1e-6 * want.abs() + 1e-6).all()
+
+
+def test_sampling_matches_oracle_bit_for_bit(capi, ref, dev):
+    announce("topk sampling")
+    rng = np.random.default_rng(13)
+    for (B, K, vocab, seed) in ((3, 3, 1000, 5), (1000, 4, 32000, 987654321098), (65, 8, 50, 0), (1, 1, 7, 42)):
+        vals = np.sort(rng.standard_normal((B, K)).astype(np.float32) * 3, axis=1)[:, ::-1].copy()
+        ids = rng.integers(0, 4 * vocab, size=(B, K)).astype(np.int32)
+        seqlen = rng.integers(0, 100, B).astype(np.int32)
+        fin = rng.integers(0, 2, B).astype(np.uint8)
+        end_id = int(ids[0, 0] % vocab)
+        d_out = torch.zeros(B, dtype=torch.int32, device=dev)
+        d_seq, d_fin = torch.from_numpy(seqlen).to(dev), torch.from_numpy(fin).to(dev)
+        capi.topk_sample(torch.from_numpy(ids).to(dev), torch.from_numpy(vals).to(dev), d_out, d_seq, d_fin, seed, end_id, vocab)
+        want = ref.topk_sample(ids, vals, seqlen, fin, seed, end_id, vocab)
+        np.testing.assert_array_equal(d_out.cpu().numpy(), want)
+        np.testing.assert_array_equal(d_seq.cpu().numpy(), seqlen)
+        np.testing.assert_array_equal(d_fin.cpu().numpy(), fin)
+
+
+def test_topk_then_sampling_pipeline(capi, ref, dev):
+    # beam top-K feeds sampling: final (val, id) pairs of each batch entry -> one token per entry
+    announce("topk -> sampling")
+    rng = np.random.default_rng(14)
+    B, beam, V, K = 8, 4, 32000, 4
+    logits = (rng.standard_normal((B * beam, V)) * 2).astype(np.float32)
+    _, _, _, fv, fi = capi.beam_topk(torch.from_numpy(logits).to(dev), B, beam, K)
+    out = torch.zeros(B, dtype=torch.int32, device=dev)
+    seq = torch.zeros(B, dtype=torch.int32, device=dev)
+    fin = torch.zeros(B, dtype=torch.uint8, device=dev)
+    capi.topk_sample(fi.contiguous(), fv.contiguous(), out, seq, fin, 77, 2, V)
+    _, _, wfv, wfi = ref.beam_topk(logits, B, beam, K)
+    want = ref.topk_sample(wfi, wfv, np.zeros(B, np.int32), np.zeros(B, np.uint8), 77, 2, V)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+    assert (out.cpu().numpy() < V).all() and (seq.cpu().numpy() == 1).all()

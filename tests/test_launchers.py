@@ -29,6 +29,7 @@ def H():
     L.h_topk.argtypes = [vp, ci, ci, vp]
     L.h_prefill_rope.argtypes = [ci, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, cf]
     L.h_act.argtypes = [ci, vp, vp, ci, ci]
+    L.h_sampling.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
     return L
 
 
@@ -190,3 +191,23 @@ def test_launchAddFusedQKVBiasTransposeAndRoPE_and_launchAct(H, ref, dev):
         tol = dict(rtol=1e-5, atol=1e-6) if code == 0 else dict(rtol=1e-2, atol=2e-3)
         np.testing.assert_allclose(out.cpu().numpy().astype(np.float64), want.astype(np.float64), **tol)
     assert H.h_sync_and_check() == 0
+
+
+@pytest.mark.gpu
+def test_launchSampling(H, ref, dev):
+    import torch
+    announce("launchSampling")
+    # the reference unit test's inputs: B3, K3, ids 0..8, vals 2,1,0, seqlen 4, step 5, end_id 10, vocab 1000
+    B, K = 3, 3
+    ids = np.arange(B * K, dtype=np.int32).reshape(B, K)
+    vals = np.tile(np.array([2.0, 1.0, 0.0], np.float32), (B, 1))
+    seqlen = np.full(B, 4, np.int32)
+    fin = np.zeros(B, np.uint8)
+    d = [_dev(a, dev) for a in (ids, vals, seqlen, fin)]
+    out = torch.zeros(B, dtype=torch.int32, device=dev)
+    assert H.h_sampling(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), out.data_ptr(), B, K, 5, 10, 1000) == 0, H.h_last_error()
+    assert H.h_sync_and_check() == 0
+    want = ref.topk_sample(ids, vals, seqlen, fin, 5, 10, 1000)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+    np.testing.assert_array_equal(d[2].cpu().numpy(), seqlen)
+    np.testing.assert_array_equal(d[3].cpu().numpy(), fin)

@@ -116,3 +116,83 @@ def test_swiglu_matches_torch_silu(ref, dtype):
     t = torch.from_numpy(inp).double()
     want = (torch.nn.functional.silu(t[:, 0]) * t[:, 1]).numpy()
     np.testing.assert_allclose(out.astype(np.float64), want, rtol=2e-6 if dtype == np.float32 else 2 ** -10, atol=1e-7)
+
+
+# ---------------------------------------------------------------- top-K sampling
+
+def test_philox_published_known_answers(ref):
+    # Random123's kat_vectors for philox4x32-10
+    assert [hex(x) for x in ref.philox4x32_10([0, 0, 0, 0], [0, 0])] == ['0x6627e8d5', '0xe169c58d', '0xbc57ac4c', '0x9b00dbd8']
+    assert [hex(x) for x in ref.philox4x32_10([0xffffffff] * 4, [0xffffffff] * 2)] == \
+        ['0x408f276d', '0x41c83b0e', '0xa20bc7c6', '0x6d5451fd']
+    assert [hex(x) for x in ref.philox4x32_10([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0])] == \
+        ['0xd16cfe09', '0x94fdcceb', '0x5001e420', '0x24126ea1']
+
+
+def test_fixed_exp_and_uniform(ref):
+    xs = np.linspace(-100, 0, 4001).astype(np.float32)
+    got = np.array([ref.exp_fixed(x) for x in xs])
+    want = np.exp(xs.astype(np.float64))
+    ok = want > 1e-37
+    assert (np.abs(got[ok] - want[ok]) / want[ok]).max() < 4e-7
+    assert ref.exp_fixed(0.0) == 1.0 and ref.exp_fixed(-200.0) == 0.0
+    assert ref.uniform_from_u32(0) == 2.0 ** -32 and ref.uniform_from_u32(0xffffffff) == 1.0      # (0, 1]
+
+
+def _sample_model(ids, vals, seed, vocab):
+    """Independent float64 statement: inverse-CDF sampling of softmax(vals) with the oracle's uniform."""
+    from oracle import ref as r
+    out = []
+    for b in range(ids.shape[0]):
+        u = r.uniform_from_u32(r.philox4x32_10([b, 0, 0, 0], [seed & 0xffffffff, seed >> 32])[0])
+        p = np.exp(vals[b].astype(np.float64) - vals[b, 0])
+        cdf = np.cumsum(p)
+        i = int(np.searchsorted(cdf, u * cdf[-1], side="right"))
+        out.append(ids[b, min(i, ids.shape[1] - 1)] % vocab)
+    return np.array(out, np.int32)
+
+
+def test_sampling_reference_unit_vector_shapes(ref):
+    # tests/unittests/test_topK_sampling.cu:8-47: B3, K3, vocab 1000, step 5, end_id 10, ids 0..8, vals 2,1,0 per row
+    B, K = 3, 3
+    ids = np.arange(B * K, dtype=np.int32).reshape(B, K)
+    vals = np.tile(np.array([2.0, 1.0, 0.0], np.float32), (B, 1))
+    seqlen = np.full(B, 4, np.int32)
+    fin = np.zeros(B, np.uint8)
+    out = ref.topk_sample(ids, vals, seqlen, fin, 5, 10, 1000)
+    np.testing.assert_array_equal(out, _sample_model(ids, vals, 5, 1000))
+    assert all(out[b] in ids[b] for b in range(B))
+    np.testing.assert_array_equal(seqlen, 5)
+    np.testing.assert_array_equal(fin, 0)
+
+
+def test_sampling_distribution_bookkeeping_and_determinism(ref):
+    rng = np.random.default_rng(3)
+    B, K, vocab = 4000, 4, 32000
+    vals = np.sort(rng.standard_normal((B, K)).astype(np.float32) * 2, axis=1)[:, ::-1].copy()
+    vals[:] = vals[0]                                       # same distribution in every row
+    ids = np.tile(np.array([5, 32000 + 7, 9, 11], np.int32), (B, 1))     # a global flat id: % vocab -> 7
+    seqlen = np.arange(B, dtype=np.int32)
+    fin = (np.arange(B) % 2).astype(np.uint8)
+    out = ref.topk_sample(ids, vals, seqlen, fin, 123456789012, 7, vocab)
+    np.testing.assert_array_equal(out, _sample_model(ids, vals, 123456789012, vocab))
+    # frequencies follow softmax(vals) (4000 draws: 4 sigma of a binomial)
+    p = np.exp(vals[0].astype(np.float64) - vals[0, 0]); p /= p.sum()
+    for k, tok in enumerate([5, 7, 9, 11]):
+        f = (out == tok).mean()
+        assert abs(f - p[k]) < 4 * np.sqrt(p[k] * (1 - p[k]) / B) + 1e-3
+    np.testing.assert_array_equal(seqlen, np.arange(B) + (np.arange(B) % 2 == 0))      # finished rows do not grow
+    np.testing.assert_array_equal(fin, (out == 7).astype(np.uint8))
+    out2 = ref.topk_sample(ids, vals, np.zeros(B, np.int32), np.zeros(B, np.uint8), 123456789012, 7, vocab)
+    np.testing.assert_array_equal(out, out2)
+    out3 = ref.topk_sample(ids, vals, np.zeros(B, np.int32), np.zeros(B, np.uint8), 123456789013, 7, vocab)
+    assert (out != out3).any()
+
+
+def test_sampling_degenerate_rows(ref):
+    ids = np.array([[3, 4, 5]], np.int32)
+    vals = np.array([[0.0, -np.inf, -np.inf]], np.float32)              # all the mass on the first
+    out = ref.topk_sample(ids, vals, np.zeros(1, np.int32), np.zeros(1, np.uint8), 1, -1, 100)
+    assert out[0] == 3
+    out = ref.topk_sample(ids[:, :1].copy(), vals[:, :1].copy(), np.zeros(1, np.int32), np.zeros(1, np.uint8), 9, -1, 100)
+    assert out[0] == 3
