@@ -3,9 +3,7 @@
 // way the reference launcher does and throws std::runtime_error on a non-zero return code.
 #pragma once
 #include "onellm/tensor.h"
-#include "onellm/base_weights.h"
-#include "onellm/norm_weights.h"
-#include "onellm/llama_params.h"
+#include "onellm/weights.h"
 #include "onellm/params.h"
 
 // src/kernels/decoder_masked_attn.h:7-14
