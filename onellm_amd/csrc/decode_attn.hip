@@ -46,6 +46,141 @@ struct AttnArgs {
     size_t slab;          // element offset of the layer slab inside the cache
 };
 
+// What one workgroup works on: a chunk of the history of one (sequence, kv-head) for up to GT query heads.
+struct Unit {
+    int b, kvh, g0;        // sequence, kv head, first query head of the tile inside the group
+    int t, pos;            // attended positions of the sequence; RoPE position of the new token
+    int split, last;       // this workgroup's split and the sequence's last split
+    int r0, r1;            // history rows [r0, r1) of this split
+    bool is_last;          // the last split also owns the new token's row
+};
+
+// Workgroups are dealt to the 8 XCDs round-robin in linear block order.  The kv-head index is the
+// fastest grid dimension so that every XCD sees the same mix of sequences and splits, and the split
+// index is rotated by the sequence index so that, with ragged lengths, the splits every sequence has
+// (the low ones) do not all land on the same XCDs.  Returns false when there is nothing to do.
+template <int GT>
+__device__ __forceinline__ bool locate_unit(const AttnArgs& a, Unit& u)
+{
+    const int ngt = (a.G + GT - 1) / GT;
+    u.kvh = blockIdx.x / ngt;
+    u.g0 = (blockIdx.x % ngt) * GT;
+    u.b = blockIdx.z;
+    u.split = (blockIdx.y + u.b) % a.nsplit;
+    u.t = a.t_dev ? a.t_dev[u.b] : a.t_host;
+    if (u.t < 1 || u.t > a.S) return false;      // out-of-contract length: touch nothing
+    u.last = (u.t - 1) / a.chunk;
+    if (u.split > u.last) return false;
+    u.is_last = u.split == u.last;
+    u.r0 = u.split * a.chunk;
+    u.r1 = min(u.r0 + a.chunk, u.t - 1);
+    u.pos = u.t + a.pos_offset;
+    return true;
+}
+
+// q of the tile's heads (and, in the last split, the new k/v row): bias, RoPE, staging in LDS; the
+// last split also stores the new row to the cache and leaves its scores in snew.  Ends with the
+// whole workgroup synchronised on sq / sk / sv (snew is ready after the caller's next barrier).
+template <typename T, int D, int GT, int NTHR>
+__device__ __forceinline__ void stage_q_and_new_row(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, T* kc, T* vc,
+                                                    float* sq, float* sk, float* sv, float* snew)
+{
+    const int tid = threadIdx.x;
+    const T* qkv = static_cast<const T*>(a.qkv) + (size_t)u.b * (a.Hq + 2 * a.Hkv) * D;
+    const T* bias = static_cast<const T*>(a.bias);
+    for (int i = tid; i < GT * (D / 2); i += NTHR) {
+        const int g = i / (D / 2), p = i % (D / 2);
+        float x0 = 0.f, x1 = 0.f;
+        if (u.g0 + g < a.G) {
+            const int h = u.kvh * a.G + u.g0 + g;
+            x0 = to_f32(qkv[h * D + 2 * p]);
+            x1 = to_f32(qkv[h * D + 2 * p + 1]);
+            if (bias) {
+                x0 += to_f32(bias[h * D + 2 * p]);
+                x1 += to_f32(bias[h * D + 2 * p + 1]);
+            }
+            if (2 * p < a.rotary_dim) rope_pair(x0, x1, p, u.pos, fr);
+        }
+        sq[g * D + 2 * p] = x0 * a.qscale;
+        sq[g * D + 2 * p + 1] = x1 * a.qscale;
+    }
+    if (u.is_last) {
+        const bool store = u.g0 == 0 && !(a.flags & ONELLM_ATTN_NO_CACHE_WRITE);
+        for (int p = tid; p < D / 2; p += NTHR) {
+            const int o = (a.Hq + u.kvh) * D + 2 * p;
+            float x0 = to_f32(qkv[o]), x1 = to_f32(qkv[o + 1]);
+            if (bias) {
+                x0 += to_f32(bias[o]);
+                x1 += to_f32(bias[o + 1]);
+            }
+            if (2 * p < a.rotary_dim) rope_pair(x0, x1, p, u.pos, fr);
+            const T k0 = from_f32<T>(x0), k1 = from_f32<T>(x1);
+            sk[2 * p] = to_f32(k0);
+            sk[2 * p + 1] = to_f32(k1);
+            if (store) {
+                kc[(size_t)(u.t - 1) * D + 2 * p] = k0;
+                kc[(size_t)(u.t - 1) * D + 2 * p + 1] = k1;
+            }
+        }
+        for (int d = tid; d < D; d += NTHR) {
+            const int o = (a.Hq + a.Hkv + u.kvh) * D + d;
+            float x = to_f32(qkv[o]);
+            if (bias && !(a.flags & ONELLM_ATTN_NO_V_BIAS)) x += to_f32(bias[o]);
+            const T v = from_f32<T>(x);
+            sv[d] = to_f32(v);
+            if (store) vc[(size_t)(u.t - 1) * D + d] = v;
+        }
+    }
+    __syncthreads();
+    if (u.is_last && tid < kWave) {
+        const int lane = tid;
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+            float part = 0.f;
+            for (int d = lane; d < D; d += kWave) part = fmaf(sq[g * D + d], sk[d], part);
+            part = wave_sum(part);
+            if (lane == 0) snew[g] = part;
+        }
+    }
+}
+
+// Merge the NST softmax states the workgroup left in LDS (plus the new token's row in the last
+// split) and write either the output (single split) or this split's partial state.  The caller has
+// synchronised the workgroup on st_ml / st_acc / snew.
+template <typename T, int D, int GT, int NST, int NTHR>
+__device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, const float* st_ml, const float* st_acc,
+                                            const float* snew, const float* sv)
+{
+    for (int i = threadIdx.x; i < GT * D; i += NTHR) {
+        const int g = i / D, d = i % D;
+        if (u.g0 + g >= a.G) continue;
+        float M = u.is_last ? snew[g] : -INFINITY;
+        for (int r = 0; r < NST; ++r) M = fmaxf(M, st_ml[(r * GT + g) * 2]);
+        float L = 0.f, O = 0.f;
+        for (int r = 0; r < NST; ++r) {
+            const float w = __builtin_amdgcn_exp2f(st_ml[(r * GT + g) * 2] - M);
+            L = fmaf(st_ml[(r * GT + g) * 2 + 1], w, L);
+            O = fmaf(st_acc[(size_t)(r * GT + g) * D + d], w, O);
+        }
+        if (u.is_last) {
+            const float w = __builtin_amdgcn_exp2f(snew[g] - M);
+            L += w;
+            O = fmaf(sv[d], w, O);
+        }
+        const int h = u.kvh * a.G + u.g0 + g;
+        if (a.nsplit == 1) {
+            static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + d] = from_f32<T>(O / L);
+        } else {
+            const size_t pi = ((size_t)u.b * a.Hq + h) * a.nsplit + u.split;
+            a.part_o[pi * D + d] = O;
+            if (d == 0) {
+                a.part_ml[pi * 2] = M;
+                a.part_ml[pi * 2 + 1] = L;
+            }
+        }
+    }
+}
+
 template <typename T, int LPR, int GT, int U, int NW>
 __global__ __launch_bounds__(NW * kWave)
 void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
@@ -67,28 +202,10 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    // Workgroups are dealt to the 8 XCDs round-robin in linear block order.  The kv-head index is
-    // the fastest grid dimension so that every XCD sees the same mix of sequences and splits, and
-    // the split index is rotated by the sequence index so that, with ragged lengths, the splits
-    // every sequence has (the low ones) do not all land on the same XCDs.
-    const int ngt = (a.G + GT - 1) / GT;
-    const int kvh = blockIdx.x / ngt;
-    const int g0 = (blockIdx.x % ngt) * GT;
-    const int b = blockIdx.z;
-    const int split = (blockIdx.y + b) % a.nsplit;
-
-    const int t = a.t_dev ? a.t_dev[b] : a.t_host;
-    if (t < 1 || t > a.S) return;               // out-of-contract length: touch nothing
-    const int last = (t - 1) / a.chunk;
-    if (split > last) return;
-    const bool is_last = split == last;
-    const int r0 = split * a.chunk;
-    const int r1 = min(r0 + a.chunk, t - 1);    // history rows [r0, r1)
-    const int pos = t + a.pos_offset;
-
-    const T* qkv = static_cast<const T*>(a.qkv) + (size_t)b * (a.Hq + 2 * a.Hkv) * D;
-    const T* bias = static_cast<const T*>(a.bias);
-    const size_t head_off = a.slab + ((size_t)b * a.Hkv + kvh) * (size_t)a.S * D;
+    Unit u;
+    if (!locate_unit<GT>(a, u)) return;
+    const int r0 = u.r0, r1 = u.r1;
+    const size_t head_off = a.slab + ((size_t)u.b * a.Hkv + u.kvh) * (size_t)a.S * D;
     T* kc = static_cast<T*>(a.k_cache) + head_off;
     T* vc = static_cast<T*>(a.v_cache) + head_off;
 
@@ -102,77 +219,23 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     // loads of one iteration: U cache rows of K and of V per row group
     auto issue = [&](Vec16<T> (&kv)[U], Vec16<T> (&vv)[U], int rbase) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int row = rbase + u * NRG + rg;
-            kv[u] = load16_stream(kp + (size_t)row * D);
-            vv[u] = load16_stream(vp + (size_t)row * D);
+        for (int u_ = 0; u_ < U; ++u_) {
+            const int row = rbase + u_ * NRG + rg;
+            kv[u_] = load16_stream(kp + (size_t)row * D);
+            vv[u_] = load16_stream(vp + (size_t)row * D);
         }
     };
     const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
     Vec16<T> ka[U], va[U], kb[U], vb[U];
     if (nfull > 0) issue(ka, va, r0);
 
-    // ---- q (and, in the last split, the new k/v row): bias, RoPE, staging in LDS
-    for (int i = tid; i < GT * (D / 2); i += NTHR) {
-        const int g = i / (D / 2), p = i % (D / 2);
-        float x0 = 0.f, x1 = 0.f;
-        if (g0 + g < a.G) {
-            const int h = kvh * a.G + g0 + g;
-            x0 = to_f32(qkv[h * D + 2 * p]);
-            x1 = to_f32(qkv[h * D + 2 * p + 1]);
-            if (bias) {
-                x0 += to_f32(bias[h * D + 2 * p]);
-                x1 += to_f32(bias[h * D + 2 * p + 1]);
-            }
-            if (2 * p < a.rotary_dim) rope_pair(x0, x1, p, pos, fr);
-        }
-        sq[g * D + 2 * p] = x0 * a.qscale;
-        sq[g * D + 2 * p + 1] = x1 * a.qscale;
-    }
-    if (is_last) {
-        const bool store = g0 == 0 && !(a.flags & ONELLM_ATTN_NO_CACHE_WRITE);
-        for (int p = tid; p < D / 2; p += NTHR) {
-            const int o = (a.Hq + kvh) * D + 2 * p;
-            float x0 = to_f32(qkv[o]), x1 = to_f32(qkv[o + 1]);
-            if (bias) {
-                x0 += to_f32(bias[o]);
-                x1 += to_f32(bias[o + 1]);
-            }
-            if (2 * p < a.rotary_dim) rope_pair(x0, x1, p, pos, fr);
-            const T k0 = from_f32<T>(x0), k1 = from_f32<T>(x1);
-            sk[2 * p] = to_f32(k0);
-            sk[2 * p + 1] = to_f32(k1);
-            if (store) {
-                kc[(size_t)(t - 1) * D + 2 * p] = k0;
-                kc[(size_t)(t - 1) * D + 2 * p + 1] = k1;
-            }
-        }
-        for (int d = tid; d < D; d += NTHR) {
-            const int o = (a.Hq + a.Hkv + kvh) * D + d;
-            float x = to_f32(qkv[o]);
-            if (bias && !(a.flags & ONELLM_ATTN_NO_V_BIAS)) x += to_f32(bias[o]);
-            const T v = from_f32<T>(x);
-            sv[d] = to_f32(v);
-            if (store) vc[(size_t)(t - 1) * D + d] = v;
-        }
-    }
-    __syncthreads();
+    stage_q_and_new_row<T, D, GT, NTHR>(a, fr, u, kc, vc, sq, sk, sv, snew);
 
     float qr[GT][VEC];
 #pragma unroll
     for (int g = 0; g < GT; ++g)
 #pragma unroll
         for (int e = 0; e < VEC; ++e) qr[g][e] = sq[g * D + col + e];
-
-    if (is_last && wave == 0) {
-#pragma unroll
-        for (int g = 0; g < GT; ++g) {
-            float part = 0.f;
-            for (int d = lane; d < D; d += kWave) part = fmaf(sq[g * D + d], sk[d], part);
-            part = wave_sum(part);
-            if (lane == 0) snew[g] = part;
-        }
-    }
 
     // ---- stream the history rows of this chunk
     float m[GT], l[GT], acc[GT][VEC];
@@ -192,35 +255,35 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
 #pragma unroll
         for (int g = 0; g < GT; ++g)
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
+            for (int u_ = 0; u_ < U; ++u_) {
                 float part = 0.f;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) part = fmaf(qr[g][e], kv[u].get(e), part);
+                for (int e = 0; e < VEC; ++e) part = fmaf(qr[g][e], kv[u_].get(e), part);
                 part = group_sum<LPR>(part);
-                if constexpr (MASKED) part = valid[u] ? part : -INFINITY;
-                s[g][u] = part;
+                if constexpr (MASKED) part = valid[u_] ? part : -INFINITY;
+                s[g][u_] = part;
             }
 #pragma unroll
         for (int g = 0; g < GT; ++g) {
             float mx = m[g];
 #pragma unroll
-            for (int u = 0; u < U; ++u) mx = fmaxf(mx, s[g][u]);
+            for (int u_ = 0; u_ < U; ++u_) mx = fmaxf(mx, s[g][u_]);
             float mref = mx;
             if constexpr (MASKED) mref = (mx == -INFINITY) ? 0.f : mx;   // nothing seen yet: keep zeros
             const float alpha = __builtin_amdgcn_exp2f(m[g] - mref);
             float psum = 0.f;
             float p[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                p[u] = __builtin_amdgcn_exp2f(s[g][u] - mref);
-                psum += p[u];
+            for (int u_ = 0; u_ < U; ++u_) {
+                p[u_] = __builtin_amdgcn_exp2f(s[g][u_] - mref);
+                psum += p[u_];
             }
             l[g] = fmaf(l[g], alpha, psum);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 float v = acc[g][e] * alpha;
 #pragma unroll
-                for (int u = 0; u < U; ++u) v = fmaf(p[u], vv[u].get(e), v);
+                for (int u_ = 0; u_ < U; ++u_) v = fmaf(p[u_], vv[u_].get(e), v);
                 acc[g][e] = v;
             }
             m[g] = mx;
@@ -246,12 +309,12 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
         if (rbase < r1) {
             bool valid[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                int row = rbase + u * NRG + rg;
-                valid[u] = row < r1;
+            for (int u_ = 0; u_ < U; ++u_) {
+                int row = rbase + u_ * NRG + rg;
+                valid[u_] = row < r1;
                 row = min(row, r1 - 1);
-                ka[u] = load16_stream(kp + (size_t)row * D);
-                va[u] = load16_stream(vp + (size_t)row * D);
+                ka[u_] = load16_stream(kp + (size_t)row * D);
+                va[u_] = load16_stream(vp + (size_t)row * D);
             }
             consume(ka, va, valid, std::true_type{});
         }
@@ -268,35 +331,7 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
         for (int e = 0; e < VEC; ++e) st_acc[(size_t)(rg * GT + g) * D + col + e] = acc[g][e];
     }
     __syncthreads();
-
-    for (int i = tid; i < GT * D; i += NTHR) {
-        const int g = i / D, d = i % D;
-        if (g0 + g >= a.G) continue;
-        float M = is_last ? snew[g] : -INFINITY;
-        for (int r = 0; r < NRG; ++r) M = fmaxf(M, st_ml[(r * GT + g) * 2]);
-        float L = 0.f, O = 0.f;
-        for (int r = 0; r < NRG; ++r) {
-            const float w = __builtin_amdgcn_exp2f(st_ml[(r * GT + g) * 2] - M);
-            L = fmaf(st_ml[(r * GT + g) * 2 + 1], w, L);
-            O = fmaf(st_acc[(size_t)(r * GT + g) * D + d], w, O);
-        }
-        if (is_last) {
-            const float w = __builtin_amdgcn_exp2f(snew[g] - M);
-            L += w;
-            O = fmaf(sv[d], w, O);
-        }
-        const int h = kvh * a.G + g0 + g;
-        if (a.nsplit == 1) {
-            static_cast<T*>(a.out)[((size_t)b * a.Hq + h) * D + d] = from_f32<T>(O / L);
-        } else {
-            const size_t pi = ((size_t)b * a.Hq + h) * a.nsplit + split;
-            a.part_o[pi * D + d] = O;
-            if (d == 0) {
-                a.part_ml[pi * 2] = M;
-                a.part_ml[pi * 2 + 1] = L;
-            }
-        }
-    }
+    finish_unit<T, D, GT, NRG, NTHR>(a, u, st_ml, st_acc, snew, sv);
 }
 
 // Merge the per-split partial states of one (sequence, query head) and normalise: one wave per
