@@ -334,6 +334,219 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     finish_unit<T, D, GT, NRG, NTHR>(a, u, st_ml, st_acc, snew, sv);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Grouped-query form on the matrix cores (fp16 storage, D = 128; GT = 4, 8 or 16 query heads per
+// kv head and workgroup).
+//
+// With one query head the scores are a matrix-vector product and the vector ALU keeps up with the
+// memory stream (it is ~17 % busy).  With four query heads sharing every K/V row the same loop is
+// ~65 % VALU-busy and becomes the limiter, and more than four heads need a second pass over the
+// rows.  Here both products of a batch of 16 cache rows run on v_mfma_f32_16x16x16_f16 and the
+// vector ALU only does the softmax bookkeeping:
+//   scores  S[16 rows x 16] = K[16 x 128] . Qt[128 x 16]: A = K as loaded, B = q with the GT heads
+//           repeated across the 16 columns; lane L ends up with rows 4*(L/16) + {0..3} of head L % GT;
+//   output  O[16 x 128] += P[16 x 16 rows] . V[16 x 128]: A = P, exactly the registers the score tile
+//           left in each lane, B = V, again straight from the load registers (a lane loads 8 columns
+//           of rows 4*(L/16) + {0..3}; product c takes column c of each).
+// No lane exchange is needed between the two products, the accumulators are 8 result tiles (32
+// registers: 8 columns of up to 16 heads, spread over the four lane rows) instead of 128, and nothing
+// has to be summed across lanes at the end.  q and P are fp32 values: each is split into an fp16 high
+// part and an fp16 remainder and every product is issued for both, so they enter at ~2^-22 instead
+// of being rounded to fp16; K and V are fp16 in memory, the accumulation is fp32.  The running
+// maximum is per head and wave-wide; it moves rarely, so its update (two cross-row exchanges and
+// the rescale) sits behind a wave-uniform branch.
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+template <int GT, int NW>
+__global__ __launch_bounds__(NW * kWave)
+void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
+{
+    using T = __half;
+    static_assert(GT == 4 || GT == 8 || GT == 16, "heads per tile");
+    constexpr int D = 128, VEC = 8;
+    constexpr int NKB = D / 16;                 // k-blocks of the score product
+    constexpr int NTHR = NW * kWave;
+    constexpr int RPI = NW * 16;                // rows per workgroup iteration
+
+    extern __shared__ float lds[];
+    float* sq = lds;                            // [GT][D]
+    float* sk = sq + GT * D;                    // [D]
+    float* sv = sk + D;                         // [D]
+    float* snew = sv + D;                       // [GT]
+    float* st_ml = snew + GT;                   // [NW][GT][2]
+    float* st_acc = st_ml + NW * GT * 2;        // [NW][GT][D]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int slot = lane & 15;
+    const int grp = lane >> 4;
+    Unit u;
+    if (!locate_unit<GT>(a, u)) return;
+    const int r0 = u.r0, r1 = u.r1;
+    const size_t head_off = a.slab + ((size_t)u.b * a.Hkv + u.kvh) * (size_t)a.S * D;
+    T* kc = static_cast<T*>(a.k_cache) + head_off;
+    T* vc = static_cast<T*>(a.v_cache) + head_off;
+    // K: lane (slot, grp) holds row `slot` of the batch, 16-byte pieces grp + 4*jp (columns grp*8 + jp*32 ..)
+    // V: lane (slot, grp) holds rows 4*grp + e of the batch, columns 8*slot .. 8*slot + 7
+    const T* kp = kc + (size_t)(wave * 16 + slot) * D + grp * VEC;
+    const T* vp = vc + (size_t)(wave * 16 + 4 * grp) * D + slot * VEC;
+
+    auto issue = [&](Vec16<T> (&kv)[4], Vec16<T> (&vv)[4], int rbase) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            kv[j] = load16_stream(kp + (size_t)rbase * D + j * 32);
+            vv[j] = load16_stream(vp + (size_t)(rbase + j) * D);
+        }
+    };
+    const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
+    Vec16<T> ka[4], va[4], kb[4], vb[4];
+    if (nfull > 0) issue(ka, va, r0);
+
+    stage_q_and_new_row<T, D, GT, NTHR>(a, fr, u, kc, vc, sq, sk, sv, snew);
+
+    // B operand of the score product: column (lane % 16) is head (lane % GT); k slots 4*grp + e of
+    // k-block (jp, h) are the columns grp*8 + jp*32 + 4*h + e — the ones the K registers hold there
+    f16x4 qhi[NKB], qlo[NKB];
+    {
+        const float* qh = sq + (lane % GT) * D + grp * VEC;
+#pragma unroll
+        for (int jp = 0; jp < 4; ++jp)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float v = qh[jp * 32 + 4 * h + e];
+                    const _Float16 hi = (_Float16)v;
+                    qhi[jp * 2 + h][e] = hi;
+                    qlo[jp * 2 + h][e] = (_Float16)(v - (float)hi);
+                }
+    }
+
+    // per lane: head (lane % GT); m is the same in every lane of a head, l is this lane's share
+    float m = -INFINITY, l = 0.f;
+    f32x4 o[VEC];                               // o[c][r]: head (4*grp + r) % GT, column 8*slot + c
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto consume = [&](const Vec16<T> (&kv)[4], const Vec16<T> (&vv)[4], int rbase, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int jp = 0; jp < 4; ++jp) {
+            const f16x4 k0 = __builtin_shufflevector(kv[jp].raw, kv[jp].raw, 0, 1, 2, 3);
+            const f16x4 k1 = __builtin_shufflevector(kv[jp].raw, kv[jp].raw, 4, 5, 6, 7);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qhi[jp * 2], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qlo[jp * 2], s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qhi[jp * 2 + 1], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qlo[jp * 2 + 1], s1, 0, 0, 0);
+        }
+        float s[4];
+        float bm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s[r] = s0[r] + s1[r];               // score of row 4*grp + r of the batch, head lane % GT
+            if constexpr (MASKED) s[r] = (rbase + wave * 16 + 4 * grp + r < r1) ? s[r] : -INFINITY;
+            bm = fmaxf(bm, s[r]);
+        }
+        if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+            bm = fmaxf(bm, __shfl_xor(bm, 16, kWave));
+            bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
+            const float mnew = fmaxf(m, bm);    // finite: some row of the batch is valid
+            const float alpha = __builtin_amdgcn_exp2f(m - mnew);
+            l *= alpha;
+            // accumulator register r belongs to head (4*grp + r) % GT: fetch that head's factor from a
+            // lane that tracks it (lane % GT == head)
+            float al[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, (lane & 48) | ((4 * grp + r) % GT), kWave);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[c][r] *= al[r];
+            m = mnew;
+        }
+        f16x4 phi, plo;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float p = __builtin_amdgcn_exp2f(s[r] - m);
+            l += p;
+            const _Float16 hi = (_Float16)p;
+            phi[r] = hi;
+            plo[r] = (_Float16)(p - (float)hi);
+        }
+        u32x4 vw[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vw[e] = __builtin_bit_cast(u32x4, vv[e].raw);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+            // column c of the four rows: one byte-permute per pair of rows
+            constexpr unsigned kLow = 0x05040100u, kHigh = 0x07060302u;
+            const unsigned sel = (c & 1) ? kHigh : kLow;
+            const u32x2 packed = {__builtin_amdgcn_perm(vw[1][c / 2], vw[0][c / 2], sel),
+                                  __builtin_amdgcn_perm(vw[3][c / 2], vw[2][c / 2], sel)};
+            const f16x4 vcol = __builtin_bit_cast(f16x4, packed);
+            o[c] = __builtin_amdgcn_mfma_f32_16x16x16f16(phi, vcol, o[c], 0, 0, 0);
+            o[c] = __builtin_amdgcn_mfma_f32_16x16x16f16(plo, vcol, o[c], 0, 0, 0);
+        }
+    };
+
+    if (r1 > r0) {
+        int rbase = r0;
+        for (int it = 0; it < nfull; it += 2) {
+            if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
+            consume(ka, va, rbase, std::false_type{});
+            if (it + 1 < nfull) {
+                if (it + 2 < nfull) issue(ka, va, rbase + 2 * RPI);
+                consume(kb, vb, rbase + RPI, std::false_type{});
+            }
+            rbase += 2 * RPI;
+        }
+        rbase = r0 + nfull * RPI;
+        if (rbase < r1) {
+            // partial batch: rows past the end are read from the last valid row and masked
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int krow = min(rbase + wave * 16 + slot, r1 - 1);
+                const int vrow = min(rbase + wave * 16 + 4 * grp + j, r1 - 1);
+                ka[j] = load16_stream(kc + (size_t)krow * D + grp * VEC + j * 32);
+                va[j] = load16_stream(vc + (size_t)vrow * D + slot * VEC);
+            }
+            // a wave whose rows are all past the end must not touch its state (its scores are all -inf)
+            if (rbase + wave * 16 < r1) consume(ka, va, rbase, std::true_type{});
+        }
+    }
+
+    // ---- one state per wave: l is summed over the four row quarters, o is already complete
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (grp == 0 && slot < GT) {
+        st_ml[(wave * GT + slot) * 2] = m;
+        st_ml[(wave * GT + slot) * 2 + 1] = l;
+    }
+    if (4 * grp < GT) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) st_acc[(size_t)(wave * GT + 4 * grp + r) * D + slot * VEC + c] = o[c][r];
+    }
+    __syncthreads();
+    finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv);
+}
+
+template <int GT>
+int launch_gqa_mfma(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    constexpr int NW = 4, D = 128;
+    const size_t lds_bytes = sizeof(float) * (size_t)(GT * D + 2 * D + GT + NW * GT * 2 + NW * GT * D);
+    const int ngt = (a.G + GT - 1) / GT;
+    const dim3 grid(a.Hkv * ngt, a.nsplit, a.B), block(NW * kWave);
+    hipLaunchKernelGGL((decode_attn_gqa_mfma_kernel<GT, NW>), grid, block, lds_bytes, st, a, fr);
+    return launch_status();
+}
+
 // Merge the per-split partial states of one (sequence, query head) and normalise: one wave per
 // (sequence, head).  Lane s holds split s's (m, l), so the maximum, the weights and the denominator
 // are two wave reductions instead of loops of dependent loads; the weighted sum over splits then
@@ -525,11 +738,30 @@ int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     return launch_split<T, LPR, GT, 4, 4>(a, fr, st);
 }
 
+// query heads one workgroup serves (they share every K/V row it reads)
+int heads_per_tile(bool fp16, int D, int G)
+{
+    if (G <= 2) return G;
+    // three or more query heads per kv head, fp16, D = 128: both products on the matrix cores, where
+    // up to 16 heads cost the same as 4
+    if (fp16 && D == 128 && tune_get("attn_gqa_valu") != 1) return G <= 4 ? 4 : (G <= 8 ? 8 : 16);
+    return 4;
+}
+
 template <typename T, int LPR>
 int launch_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
-    if (a.G == 1) return launch_shape<T, LPR, 1>(a, fr, st);
-    if (a.G == 2) return launch_shape<T, LPR, 2>(a, fr, st);
+    constexpr bool kHalf = std::is_same<T, __half>::value;
+    switch (heads_per_tile(kHalf, LPR * Elt<T>::kVec, a.G)) {
+        case 1: return launch_shape<T, LPR, 1>(a, fr, st);
+        case 2: return launch_shape<T, LPR, 2>(a, fr, st);
+        case 8: return launch_gqa_mfma<8>(a, fr, st);
+        case 16: return launch_gqa_mfma<16>(a, fr, st);
+        default: break;
+    }
+    if constexpr (kHalf && LPR == 16) {
+        if (tune_get("attn_gqa_valu") != 1) return launch_gqa_mfma<4>(a, fr, st);
+    }
     return launch_shape<T, LPR, 4>(a, fr, st);
 }
 
@@ -609,7 +841,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // needs no merge pass.  Per-sequence lengths: finer chunks (about 16 workgroups per compute unit,
     // at least 256 rows each) so that the dispatcher can balance ragged work.
     const int G = a.G;
-    const int gt = G == 1 ? 1 : (G == 2 ? 2 : 4);
+    const int gt = heads_per_tile(dtype == ONELLM_FP16, D, G);
     const int ngt = (G + gt - 1) / gt;
     const long base_wgs = (long)B * Hkv * ngt;
     const int user_target = tune_get("attn_target_wgs");

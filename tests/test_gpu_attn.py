@@ -88,7 +88,8 @@ def test_example_driver_shape_two_layers(capi, ref, dev):
 
 @pytest.mark.parametrize("dtype,Hq,Hkv,D", [
     (np.float16, 4, 4, 128), (np.float16, 8, 2, 128), (np.float16, 8, 1, 64), (np.float16, 6, 3, 32),
-    (np.float16, 12, 2, 256), (np.float16, 2, 2, 8), (np.float16, 4, 2, 16), (np.float16, 2, 1, 512),
+    (np.float16, 16, 2, 128), (np.float16, 14, 2, 128), (np.float16, 16, 1, 128), (np.float16, 40, 2, 128),
+    (np.float16, 3, 1, 128), (np.float16, 12, 2, 256), (np.float16, 2, 2, 8), (np.float16, 4, 2, 16), (np.float16, 2, 1, 512),
     (np.float32, 4, 4, 128), (np.float32, 8, 2, 64), (np.float32, 3, 1, 32), (np.float32, 2, 2, 256),
     (np.float32, 4, 1, 4), (np.float32, 10, 2, 16),
 ])
@@ -143,6 +144,10 @@ def test_sequence_split_counts_and_ragged_lengths(capi, ref, dev, dtype, nsplit)
     capi.tune_set("attn_nsplit", nsplit)
     try:
         _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), dtype)
+        if dtype == np.float16:
+            # 7 query heads per kv head: the 8-head matrix-core tile with one head of padding
+            qkv7, bias7, kc7, vc7 = _case(dtype, B, 14, 2, D, S, 1, seed=31 + nsplit, std=0.5)
+            _assert_parity(_run_both(capi, ref, dev, qkv7, bias7, kc7, vc7, 14, t, D), dtype)
     finally:
         capi.tune_set("attn_nsplit", -1)
 
