@@ -163,6 +163,12 @@ def extras_section(capi, dev, args, with_cpu):
     ms, (qkv, bias, (kc, vc), _) = bench_attention(capi, dev, steps3, args.warmup, B3, Hq3, Hkv3, D, S3, S3, nsets=3, t_dev=t_dev)
     cpu = cpu_attention(qkv, bias, kc, vc, Hq3, tl, D, 6.0)[0] if with_cpu else None
     ex["decode_attn_gqa_fused_b32_q32_kv8_len1024-8192"] = entry(ms, nb_fused, cpu)
+    # same cache, every sequence at the full 8192 rows; then 64 query heads over the 8 KV heads (batch 16)
+    ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, B3, Hq3, Hkv3, D, S3, S3, nsets=3)
+    ex["decode_attn_gqa_fused_b32_q32_kv8_len8192"] = entry(ms_u, attn_bytes(B3, Hq3, Hkv3, D, [S3] * B3, 2))
+    ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, 16, 64, Hkv3, D, S3, S3, nsets=3)
+    ex["decode_attn_gqa_fused_b16_q64_kv8_len8192"] = entry(ms_u, attn_bytes(16, 64, Hkv3, D, [S3] * 16, 2))
+    torch.cuda.empty_cache()
     # the reference-style path on the same data: concat the new row, repeat KV to 32 heads, attend over 32 heads
     hist = (t_dev - 1).contiguous()
     ones = torch.ones(B3, dtype=torch.int32, device=dev)

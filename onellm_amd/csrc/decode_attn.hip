@@ -741,11 +741,11 @@ int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 // query heads one workgroup serves (they share every K/V row it reads)
 int heads_per_tile(bool fp16, int D, int G)
 {
-    if (G <= 2) return G;
-    // three or more query heads per kv head, fp16, D = 128: both products on the matrix cores, where
+    if (G == 1) return 1;       // one head: memory-bound on either kernel (measured equal), keep the lighter one
+    // two or more query heads per kv head, fp16, D = 128: both products on the matrix cores, where
     // up to 16 heads cost the same as 4
     if (fp16 && D == 128 && tune_get("attn_gqa_valu") != 1) return G <= 4 ? 4 : (G <= 8 ? 8 : 16);
-    return 4;
+    return G == 2 ? 2 : 4;
 }
 
 template <typename T, int LPR>
