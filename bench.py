@@ -141,6 +141,81 @@ def cpu_norm(N, H, fused, budget_s):
     return time_cpu(lambda: ref.rmsnorm(x, g, 1e-5), budget_s)
 
 
+def decoder_layer_section(capi, dev, args):
+    """One whole decoder layer of the Llama-2-7B shape at batch 16, ctx 4096, as LlamaSelfDecoder sequences it:
+    RMSNorm -> qkv projection -> fused masked attention -> output projection -> fused add-bias-residual-RMSNorm ->
+    gate / up projections -> SwiGLU -> down projection -> fused add-bias-residual-RMSNorm.  The projections are library
+    GEMMs (hipBLASLt through onellm_linear); everything else is this repository's kernels."""
+    import torch
+    B, H, D, S, I, t = 16, 32, 128, 4096, 11008, 4096
+    hid = H * D
+    g = torch.Generator(device=dev).manual_seed(7)
+    rnd = lambda *shape, scale=1.0: (torch.randn(*shape, device=dev, generator=g) * scale).half()
+    wqkv, wo = rnd(hid, 3 * hid, scale=hid ** -0.5), rnd(hid, hid, scale=hid ** -0.5)
+    wg, wu, wd = rnd(hid, I, scale=hid ** -0.5), rnd(hid, I, scale=hid ** -0.5), rnd(I, hid, scale=I ** -0.5)
+    bqkv, bo, bd = rnd(3 * hid, scale=0.1), rnd(hid, scale=0.1), rnd(hid, scale=0.1)
+    g1, g2, g3 = (torch.rand(hid, device=dev, generator=g) + 0.5).half(), (torch.rand(hid, device=dev, generator=g) + 0.5).half(), \
+        (torch.rand(hid, device=dev, generator=g) + 0.5).half()
+    sets = [(rnd(1, B, H, S, D, scale=0.5), rnd(1, B, H, S, D, scale=0.5)) for _ in range(3)]
+    x0 = rnd(B, hid)
+    x, y = x0.clone(), torch.empty_like(x0)
+    qkv, att = torch.empty(B, 3 * H, D, dtype=torch.float16, device=dev), torch.empty(B, hid, dtype=torch.float16, device=dev)
+    pair, act = torch.empty(B, 2, I, dtype=torch.float16, device=dev), torch.empty(B, I, dtype=torch.float16, device=dev)
+    ws_attn = torch.empty(capi.decode_attn_workspace_bytes(B, H, H, D, t), dtype=torch.uint8, device=dev)
+    ws_gemm = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dev)
+
+    def norm_in(i):
+        y.copy_(x)
+        capi.rmsnorm(y, g1, 1e-5)
+
+    def proj_qkv(i):
+        capi.linear(y, wqkv, qkv.view(B, 3 * hid), workspace=ws_gemm)
+
+    def attention(i):
+        kc, vc = sets[i % len(sets)]
+        capi.decode_attn(qkv, bqkv, kc, vc, att, H, t, D, 10000.0, rope_pos_offset=-1, workspace=ws_attn)
+
+    def proj_out(i):
+        capi.linear(att, wo, y, workspace=ws_gemm)
+
+    def norm_mid(i):
+        capi.fused_add_bias_residual_rmsnorm(x, y, bo, g2, 1e-5)
+
+    def proj_gate_up(i):
+        capi.linear(y, wg, pair, ldy=2 * I, workspace=ws_gemm)
+        capi.linear(y, wu, pair.view(-1)[I:], ldy=2 * I, workspace=ws_gemm)
+
+    def swiglu(i):
+        capi.silu_and_mul(pair, act)
+
+    def proj_down(i):
+        capi.linear(act, wd, y, workspace=ws_gemm)
+
+    def norm_out(i):
+        capi.fused_add_bias_residual_rmsnorm(x, y, bd, g3, 1e-5)
+
+    parts = [("rmsnorm", norm_in), ("qkv_proj", proj_qkv), ("attention", attention), ("out_proj", proj_out),
+             ("fused_norm_1", norm_mid), ("gate_up_proj", proj_gate_up), ("swiglu", swiglu), ("down_proj", proj_down),
+             ("fused_norm_2", norm_out)]
+
+    def layer(i):
+        if i % 8 == 0:
+            x.copy_(x0)            # keep the residual stream bounded over hundreds of repeated steps
+        for _, fn in parts:
+            fn(i)
+
+    steps = max(args.steps // 3, 10)
+    ms = time_steps(layer, steps, max(args.warmup // 3, 3))
+    weight_bytes = 2 * (wqkv.numel() + wo.numel() + wg.numel() + wu.numel() + wd.numel())
+    nb = weight_bytes + attn_bytes(B, H, H, D, [t] * B, 2)
+    e = entry(ms, nb)
+    e["parts_us"] = {name: round(time_steps(fn, steps, 3) * 1e3, 2) for name, fn in parts}
+    e["gemm_path"] = "hipBLASLt" if capi.gemm_lib().onellm_linear_last_path() == 1 else "plain kernel"
+    e["note"] = ("bytes = the five weight matrices (%d) + the attention step's algorithmic bytes; parts are timed "
+                 "one at a time, so their sum includes a launch gap per part" % weight_bytes)
+    return {"decoder_layer_llama7b_b16_ctx4096": e}
+
+
 def extras_section(capi, dev, args, with_cpu):
     import numpy as np
     import torch
@@ -194,6 +269,9 @@ def extras_section(capi, dev, args, with_cpu):
     e["note"] = "concat -> repeat -> attend on the same data; gbps/frac are against the FUSED path's algorithmic bytes"
     ex["decode_attn_gqa_repeat_path_total"] = e
     del rk, rv, kc, vc, qkv, bias, qkv_r, ws
+    torch.cuda.empty_cache()
+
+    ex.update(decoder_layer_section(capi, dev, args))
     torch.cuda.empty_cache()
 
     for (N, Hd) in ((16, 4096), (512, 4096), (8192, 4096), (8192, 8192)):

@@ -16,6 +16,20 @@ void launchDecoderMaskedMHA(Tensor* qkv_buf,
                             Tensor* mha_output,
                             LLaMAAttentionStaticParams& static_params);
 
+// The same with the RoPE position stated: the token at cache row step-1 is rotated as position
+// step + rope_pos_offset.  The 8-argument form is offset 0 (src/kernels/decoder_masked_attn.cu:186 rotates with
+// `step`); -1 is the 0-based position the context-phase kernel gives the same row
+// (src/kernels/qkv_bias_and_RoPE.cu:140), i.e. what a cache filled by prefill needs.
+void launchDecoderMaskedMHA(Tensor* qkv_buf,
+                            BaseWeight& qkv,
+                            Tensor* k_cache,
+                            Tensor* v_cache,
+                            Tensor* finished,
+                            Tensor* step,
+                            Tensor* mha_output,
+                            LLaMAAttentionStaticParams& static_params,
+                            int rope_pos_offset);
+
 // src/kernels/rmsnorm_kernel.h:6-9
 void launchRMSNorm(Tensor* decoder_out, LayerNormWeight& attn_norm_weight, float eps);
 

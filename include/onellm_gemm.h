@@ -1,0 +1,40 @@
+/* C ABI of the projection GEMMs around the decode path (exported by libonellm_gemm.so).
+ *
+ * Replaces launchLinearGemm (src/kernels/qkv_linear.cu:8-66, declared src/kernels/qkv_linear.h:9-14) and the
+ * cublasWrapper::Gemm call under it (src/kernels/cublas_wrapper.cc:33-85).  The multiplication itself is a library
+ * GEMM (hipBLASLt, fp32 accumulation); this entry point adds what the reference re-creates on every call: a handle
+ * per device and a cached plan per (dtype, M, K, N, layout).  Shapes the library has no kernel for fall back to a
+ * plain kernel in this library, so every shape returns a result.
+ *
+ * Kept out of libonellm_hip.so so that the decode-path kernels do not pull in the BLAS library.
+ */
+#ifndef ONELLM_GEMM_H
+#define ONELLM_GEMM_H
+#include <stddef.h>
+#include "onellm_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* y[M, N] = x[M, K] . W, row-major, fp32 accumulation, y rounded once to `dtype`.  x and W are contiguous; row m
+ * of y starts at y + m * ldy elements (ldy >= N; 0 means N), so two projections can write the two halves of one
+ * [M, 2, N] buffer — the layout the SwiGLU kernel reads (src/kernels/activation_kernel.cu:11-13).
+ *   w_is_nk == 0:  W is [K, N]  (the layout of every BaseWeight the oneLLM layers hold: shape = {in, out},
+ *                  src/weights/llama/layer_weights.cc:21-41)
+ *   w_is_nk != 0:  W is [N, K]  (y = x . W^T; launchLinearGemm's trans_b)
+ * workspace: device scratch for the library's split-K algorithms; may be NULL/0, then only algorithms that need
+ * none are considered.  Returns 0, an ONELLM_E* code, or a hipError_t. */
+int onellm_linear(int dtype, const void* x, const void* w, void* y, int M, int K, int N, int ldy, int w_is_nk,
+                  void* workspace, size_t workspace_bytes, onellm_stream_t stream);
+
+/* workspace size onellm_linear can make use of (a constant; any smaller size is valid too) */
+size_t onellm_linear_workspace_bytes(void);
+
+/* 1 if the last onellm_linear call on this thread ran the library GEMM, 0 if it ran the plain fallback kernel */
+int onellm_linear_last_path(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

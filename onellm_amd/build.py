@@ -3,8 +3,9 @@
     python -m onellm_amd.build            # build what is out of date
     python -m onellm_amd.build --force    # rebuild everything
 
-Outputs (next to this file): libonellm_hip.so (the C ABI of include/onellm_hip.h) and
-libonellm_launchers.so (the six launch* functions with oneLLM's own signatures).
+Outputs (next to this file): libonellm_hip.so (the C ABI of include/onellm_hip.h), libonellm_launchers.so (the
+launch* functions with oneLLM's own signatures), libonellm_gemm.so (the C ABI of include/onellm_gemm.h, over
+hipBLASLt) and libonellm_layers.so (the decode-side layers of include/onellm/layers.h).
 hipcc cross-compiles for gfx950 without a GPU.
 """
 import concurrent.futures
@@ -21,13 +22,19 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 LIB_HIP = os.path.join(HERE, "libonellm_hip.so")
 LIB_LAUNCH = os.path.join(HERE, "libonellm_launchers.so")
+LIB_GEMM = os.path.join(HERE, "libonellm_gemm.so")
+LIB_LAYERS = os.path.join(HERE, "libonellm_layers.so")
 # test-only: a C wrapper that drives the launcher shims with oneLLM-style Tensor objects
 HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "launcher_harness.cpp")
 LIB_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
+LAYERS_HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "layers_harness.cpp")
+LIB_LAYERS_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblayers_harness.so")
 
 KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip", "sampling.hip",
                   "tuning.cpp"]
 LAUNCHER_SOURCES = ["launchers.cpp"]
+GEMM_SOURCES = ["linear.hip"]
+LAYER_SOURCES = ["layers.cpp"]
 
 # packed fp32 VALU forms are switched off on purpose (code generation only; scalar fp32 code is
 # what the kernels are written in)
@@ -68,6 +75,8 @@ def build(force=False, verbose=False):
     with concurrent.futures.ThreadPoolExecutor(max_workers=6) as ex:
         kobjs = list(ex.map(lambda s: _compile(s, force), KERNEL_SOURCES))
         lobjs = list(ex.map(lambda s: _compile(s, force), LAUNCHER_SOURCES))
+        gobjs = list(ex.map(lambda s: _compile(s, force), GEMM_SOURCES))
+        yobjs = list(ex.map(lambda s: _compile(s, force), LAYER_SOURCES))
     if force or _newer(LIB_HIP, kobjs):
         cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_HIP] + kobjs
         subprocess.run(cmd, check=True, capture_output=not verbose)
@@ -81,7 +90,22 @@ def build(force=False, verbose=False):
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("hipcc failed for the launcher harness:\n" + r.stderr[-4000:])
-    return LIB_HIP, LIB_LAUNCH
+    if force or _newer(LIB_GEMM, gobjs + [LIB_HIP]):
+        cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_GEMM] + gobjs + \
+              ["-L" + HERE, "-lonellm_hip", "-L/opt/rocm/lib", "-lhipblaslt", "-Wl,-rpath,$ORIGIN"]
+        subprocess.run(cmd, check=True, capture_output=not verbose)
+    if force or _newer(LIB_LAYERS, yobjs + [LIB_GEMM, LIB_LAUNCH]):
+        cmd = [HIPCC, "-shared", "-fPIC", "-o", LIB_LAYERS] + yobjs + \
+              ["-L" + HERE, "-lonellm_gemm", "-lonellm_launchers", "-lonellm_hip", "-Wl,-rpath,$ORIGIN"]
+        subprocess.run(cmd, check=True, capture_output=not verbose)
+    if os.path.exists(LAYERS_HARNESS_SRC) and (force or _newer(LIB_LAYERS_HARNESS, [LAYERS_HARNESS_SRC, LIB_LAYERS] + _headers())):
+        cmd = [HIPCC, "-shared", "-fPIC", "-O2", "-std=c++17", "-I" + INCLUDE, LAYERS_HARNESS_SRC, "-o", LIB_LAYERS_HARNESS,
+               "-L" + HERE, "-lonellm_layers", "-lonellm_gemm", "-lonellm_launchers", "-lonellm_hip",
+               "-Wl,-rpath,$ORIGIN/../../onellm_amd"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for the layers harness:\n" + r.stderr[-4000:])
+    return LIB_HIP, LIB_LAUNCH, LIB_GEMM, LIB_LAYERS
 
 
 if __name__ == "__main__":

@@ -194,3 +194,47 @@ def topk_sample(topk_id, topk_val, output_id, seqlen, is_finished, seed, end_id,
     _check(lib().onellm_topk_sample(_ptr(topk_id), _ptr(topk_val), _ptr(output_id), _ptr(seqlen), _ptr(is_finished), B, K,
                                     int(seed), end_id, vocab_size, _stream()), "onellm_topk_sample")
     return output_id
+
+
+# ---------------------------------------------------------------- projection GEMMs (include/onellm_gemm.h)
+GEMM_PATH = os.path.join(_HERE, "libonellm_gemm.so")
+LAYERS_PATH = os.path.join(_HERE, "libonellm_layers.so")
+GEMM_SYMBOLS = {
+    "onellm_linear": (_ci, [_ci, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
+    "onellm_linear_workspace_bytes": (_sz, []),
+    "onellm_linear_last_path": (_ci, []),
+}
+_gemm = None
+
+
+def gemm_lib():
+    """Load the projection library (once); it brings in hipBLASLt, so it is separate from lib()."""
+    global _gemm
+    if _gemm is None:
+        if not os.path.exists(GEMM_PATH):
+            raise RuntimeError(f"{GEMM_PATH} is missing: build it with `python -m onellm_amd.build`")
+        import torch  # noqa: F401  first: the process must end up with one HIP runtime and one BLAS library
+        L = ctypes.CDLL(GEMM_PATH)
+        for name, (res, args) in GEMM_SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _gemm = L
+    return _gemm
+
+
+def linear_workspace_bytes():
+    return gemm_lib().onellm_linear_workspace_bytes()
+
+
+def linear(x, w, y, w_is_nk=False, ldy=0, workspace=None):
+    """y[M, N] = x[M, K] . W (W [K, N], or [N, K] with w_is_nk); y may be a strided view given by its first element
+    and `ldy`.  `workspace`: uint8 device tensor or None."""
+    M, K = x.shape
+    N = w.shape[0] if w_is_nk else w.shape[1]
+    assert (w.shape[1] if w_is_nk else w.shape[0]) == K and x.dtype == w.dtype == y.dtype
+    assert x.is_cuda and x.is_contiguous() and w.is_contiguous()
+    rc = gemm_lib().onellm_linear(_dt(x), x.data_ptr(), w.data_ptr(), y.data_ptr(), M, K, N, int(ldy), int(bool(w_is_nk)),
+                                  _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream())
+    _check(rc, "onellm_linear")
+    return y

@@ -78,6 +78,12 @@ int host_layer_id(const Tensor* layer_id)
 void launchDecoderMaskedMHA(Tensor* qkv_buf, BaseWeight& qkv, Tensor* k_cache, Tensor* v_cache, Tensor* finished,
                             Tensor* step, Tensor* mha_output, LLaMAAttentionStaticParams& static_params)
 {
+    launchDecoderMaskedMHA(qkv_buf, qkv, k_cache, v_cache, finished, step, mha_output, static_params, /*rope_pos_offset=*/0);
+}
+
+void launchDecoderMaskedMHA(Tensor* qkv_buf, BaseWeight& qkv, Tensor* k_cache, Tensor* v_cache, Tensor* finished,
+                            Tensor* step, Tensor* mha_output, LLaMAAttentionStaticParams& static_params, int rope_pos_offset)
+{
     (void)finished;   // unused by the reference as well (:284)
     ONELLM_CHECK_WITH_INFO(qkv_buf && k_cache && v_cache && step && mha_output, "null tensor");
     ONELLM_CHECK_WITH_INFO(qkv_buf->shape.size() == 3, "qkv_buf must be [B, Hq+2Hkv, D]");
@@ -99,7 +105,7 @@ void launchDecoderMaskedMHA(Tensor* qkv_buf, BaseWeight& qkv, Tensor* k_cache, T
                                   batch_size, head_num, kv_head_num, head_size, cs.S, /*layer=*/0, cs.layers,
                                   cur_step, nullptr, cur_step,
                                   static_params.rotary_embedding_dim, static_params.rotary_embedding_base,
-                                  /*rope_pos_offset=*/0, /*flags=*/0u, ws, ws_bytes, nullptr);
+                                  rope_pos_offset, /*flags=*/0u, ws, ws_bytes, nullptr);
     };
     int rc = call(nullptr, 0);
     if (rc == ONELLM_EWORKSPACE) {

@@ -229,3 +229,46 @@ def topk_sample(topk_id, topk_val, seqlen, is_finished, seed, end_id, vocab_size
     _chk(lib().onellm_ref_topk_sample(_p(topk_id), _p(topk_val), _p(out), _p(seqlen), _p(is_finished), B, K,
                                       int(seed), end_id, vocab_size), "topk_sample")
     return out
+
+
+def linear(x, w, w_is_nk=False):
+    """y[M, N] = x[M, K] . W with W [K, N] (or [N, K] when w_is_nk), accumulated in float64 and rounded once to
+    x.dtype — the projection of src/kernels/qkv_linear.cu:8-66 with the weight layout of
+    src/weights/llama/layer_weights.cc:21-41 (shape = {in, out}).  Pinned by the all-ones case of
+    tests/unittests/test_linear.cu:60-98 and by brute-force triple loops."""
+    assert x.dtype == w.dtype and x.ndim == 2 and w.ndim == 2
+    wm = w.astype(np.float64)
+    y = x.astype(np.float64) @ (wm.T if w_is_nk else wm)
+    return y.astype(x.dtype)
+
+
+def self_decoder_step(x, layers, output_norm, k_cache, v_cache, Hq, t, rotary_dim, rope_base, eps, rope_pos_offset=-1):
+    """One decode step of the LLaMA decoder stack (src/layers/decoder/self_decoder.cpp:15-78 with
+    src/layers/attention/masked_self_attention.cpp:51-82 and src/layers/ffn/ffn.cpp:53-73), built from the
+    per-kernel restatements above plus linear().  The data flow is the pre-norm decoder the reference is written
+    towards (x stays the residual stream; the snapshot normalises it in place, drops the FFN result and addresses
+    cache layer 0 for every layer).  The new token is rotated as position t + rope_pos_offset: -1 is the 0-based
+    position the context phase gives that row (src/kernels/qkv_bias_and_RoPE.cu:140), 0 what the decode kernel does
+    on its own (src/kernels/decoder_masked_attn.cu:186).
+
+    x [B, hidden] (updated in place: the residual stream); layers: list of dicts with attn_norm, ffn_norm, wqkv
+    [hidden, (Hq+2Hkv)D], bqkv, wo [hidden, hidden], bo, wgate/wup [hidden, I], wdown [I, hidden], bdown (biases
+    may be None); caches [L, B, Hkv, S, D] (row t-1 of every layer written).  Returns y [B, hidden]."""
+    B, hidden = x.shape
+    L, _, Hkv, S, D = k_cache.shape
+    assert len(layers) == L and hidden == Hq * D
+    zeros = np.zeros(hidden, dtype=x.dtype)
+    y = rmsnorm(x.copy(), layers[0]["attn_norm"], eps)
+    for l, w in enumerate(layers):
+        qkv = linear(y, w["wqkv"]).reshape(B, Hq + 2 * Hkv, D)
+        a = decode_attn(qkv, w["bqkv"], k_cache, v_cache, Hq, t, rotary_dim, rope_base, layer=l,
+                        rope_pos_offset=rope_pos_offset)
+        y = linear(a, w["wo"])
+        fused_add_bias_residual_rmsnorm(x, y, w["bo"] if w["bo"] is not None else zeros, w["ffn_norm"], eps)
+        gate, up = linear(y, w["wgate"]), linear(y, w["wup"])
+        pair = np.ascontiguousarray(np.stack([gate, up], axis=1))           # [B, 2, I]
+        act = silu_and_mul(pair, np.empty_like(gate))
+        y = linear(act, w["wdown"])
+        gamma = layers[l + 1]["attn_norm"] if l + 1 < L else output_norm
+        fused_add_bias_residual_rmsnorm(x, y, w["bdown"] if w["bdown"] is not None else zeros, gamma, eps)
+    return y

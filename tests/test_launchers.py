@@ -18,6 +18,7 @@ HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
 @pytest.fixture(scope="module")
 def H():
     assert os.path.exists(HARNESS), "build it with `python -m onellm_amd.build`"
+    import torch  # noqa: F401  first, so that the HIP runtime torch ships is the one this process uses
     L = ctypes.CDLL(HARNESS)
     vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
     L.h_last_error.restype = ctypes.c_char_p

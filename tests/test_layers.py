@@ -1,0 +1,263 @@
+"""The decode-side layers (include/onellm/layers.h: launchLinearGemm, LLaMASelfAttentionLayer, LLaMAFFNLayer,
+LlamaSelfDecoder) and the projection C ABI under them (include/onellm_gemm.h), driven through a small C harness that
+builds Tensor / TensorMap / LlamaLayerWeight objects the way examples/cpp/decoder/self_decoder_example.cpp does.
+Host-side behaviour runs without a GPU; parity against the CPU oracle (oracle/ref.py: linear, self_decoder_step — the
+latter pinned on an independent library implementation in tests/test_oracle_layers.py) is marked gpu."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import announce
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HARNESS = os.path.join(ROOT, "tests", "cpp", "liblayers_harness.so")
+LIB_GEMM = os.path.join(ROOT, "onellm_amd", "libonellm_gemm.so")
+LIB_LAYERS = os.path.join(ROOT, "onellm_amd", "libonellm_layers.so")
+
+
+@pytest.fixture(scope="module")
+def H():
+    assert os.path.exists(HARNESS), "build it with `python -m onellm_amd.build`"
+    import torch  # noqa: F401  first, so that the HIP runtime and BLAS library torch ships are the ones this process uses
+    L = ctypes.CDLL(HARNESS)
+    vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    pp = ctypes.POINTER(ctypes.c_void_p)
+    L.hl_last_error.restype = ctypes.c_char_p
+    L.hl_linear.argtypes = [ci, vp, vp, vp, ci, ci, ci, ci, ci, ci]
+    L.hl_decoder_create.restype = vp
+    L.hl_decoder_create.argtypes = [ci] * 9 + [cf, cf, ci] + [pp] * 10 + [vp]
+    L.hl_decoder_forward.argtypes = [vp, ci, vp, vp, vp, vp]
+    L.hl_decoder_destroy.argtypes = [vp]
+    return L
+
+
+@pytest.fixture(scope="module")
+def G():
+    import torch  # noqa: F401  (see H)
+    L = ctypes.CDLL(LIB_GEMM)
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    L.onellm_linear.argtypes = [ci, vp, vp, vp, ci, ci, ci, ci, ci, vp, ctypes.c_size_t, vp]
+    L.onellm_linear_workspace_bytes.restype = ctypes.c_size_t
+    return L
+
+
+# ---------------------------------------------------------------- host only
+
+def test_gemm_library_exports_what_its_header_declares(G):
+    text = open(os.path.join(ROOT, "include", "onellm_gemm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(onellm_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["onellm_linear", "onellm_linear_last_path", "onellm_linear_workspace_bytes"]
+    for n in names:
+        assert hasattr(G, n)
+    assert G.onellm_linear_workspace_bytes() > 0
+
+
+def test_linear_rejects_bad_arguments_before_any_launch(G):
+    fake = ctypes.c_void_p(0x1000)
+    assert G.onellm_linear(7, fake, fake, fake, 2, 4, 4, 0, 0, None, 0, None) == -1        # unknown dtype
+    assert G.onellm_linear(0, None, fake, fake, 2, 4, 4, 0, 0, None, 0, None) == -1        # null input
+    assert G.onellm_linear(0, fake, fake, fake, 2, 0, 4, 0, 0, None, 0, None) == -1        # empty inner size
+    assert G.onellm_linear(0, fake, fake, fake, 2, 4, 4, 3, 0, None, 0, None) == -1        # row stride below N
+    assert G.onellm_linear(0, fake, fake, fake, 0, 4, 4, 0, 0, None, 0, None) == 0         # no rows: nothing to do
+
+
+def test_layers_library_exports_reference_signatures():
+    out = subprocess.run(["nm", "-DC", LIB_LAYERS], capture_output=True, text=True, check=True).stdout
+    for sig in ["launchLinearGemm(Tensor*, BaseWeight&, Tensor*, bool, bool, bool)",
+                "LLaMASelfAttentionLayer::forward(TensorMap&, TensorMap&, LLaMAattentionWeights&, LLaMAAttentionDynParams&)",
+                "LLaMAFFNLayer::forward(TensorMap&, TensorMap&, LLaMAFFNWeights&, LLaMAAttentionDynParams&)",
+                "LlamaSelfDecoder::forward(TensorMap&, std::vector<LlamaLayerWeight*, std::allocator<LlamaLayerWeight*> > const&, TensorMap&, LLaMAAttentionDynParams&)",
+                "LlamaSelfDecoder::LlamaSelfDecoder(int, int, int, int, int, LLaMAAttentionStaticParams const&, float, ihipStream_t*, cublasWrapper*, BaseAllocator*, bool)"]:
+        assert sig in out, sig
+
+
+def test_linear_launcher_precondition_failures_throw(H):
+    fake = ctypes.c_void_p(0x1000)
+    assert H.hl_linear(0, None, fake, fake, 2, 4, 4, 0, 0, 0) == 1
+    assert b"null tensor or weight" in H.hl_last_error()
+    assert H.hl_linear(0, fake, fake, fake, 2, 4, 4, 0, 0, 1) == 1                          # second slot without a pair buffer
+    assert b"shared_out_buf" in H.hl_last_error()
+
+
+# ---------------------------------------------------------------- GPU parity
+
+TOL = {np.float32: dict(rtol=2e-5, atol=2e-5), np.float16: dict(rtol=1e-2, atol=2e-3)}
+
+
+def _dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("M,K,N", [(1, 16, 16), (2, 32, 64), (3, 7, 5), (16, 4096, 12288), (16, 4096, 4096), (16, 11008, 4096),
+                                   (5, 100, 36), (64, 256, 512)])
+def test_linear_matches_the_oracle(H, G, ref, dtype, M, K, N):
+    import torch
+    announce("linear", dtype.__name__, M, K, N)
+    rng = np.random.default_rng(M * 7 + N)
+    if (M, K, N) == (1, 16, 16):                       # tests/unittests/test_linear.cu:60-98
+        x, w = np.ones((M, K), dtype), np.ones((K, N), dtype)
+    else:
+        x = (rng.standard_normal((M, K)) * 0.5).astype(dtype)
+        w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(dtype)
+    want = ref.linear(x, w)
+    dx, dw = _dev(torch, x), _dev(torch, w)
+    y = torch.full((M, N), 7.0, dtype=dx.dtype, device=dx.device)
+    code = 1 if dtype == np.float16 else 0
+    assert H.hl_linear(code, dx.data_ptr(), dw.data_ptr(), y.data_ptr(), M, K, N, 0, 0, 0) == 0, H.hl_last_error()
+    np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[dtype])
+    if K >= 4096:
+        assert G.onellm_linear_last_path() == 1, "the projection shapes of a 7B layer must run the library GEMM"
+    # W given as [N, K]
+    dwt = _dev(torch, w.T)
+    y2 = torch.zeros_like(y)
+    assert H.hl_linear(code, dx.data_ptr(), dwt.data_ptr(), y2.data_ptr(), M, K, N, 1, 0, 0) == 0, H.hl_last_error()
+    np.testing.assert_allclose(y2.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[dtype])
+    # the gate/up pair buffer: two projections into the two slots of [M, 2, N]
+    w2 = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(dtype)
+    pair = torch.full((M, 2, N), -3.0, dtype=dx.dtype, device=dx.device)
+    assert H.hl_linear(code, dx.data_ptr(), dw.data_ptr(), pair.data_ptr(), M, K, N, 0, 1, 0) == 0, H.hl_last_error()
+    assert H.hl_linear(code, dx.data_ptr(), _dev(torch, w2).data_ptr(), pair.data_ptr(), M, K, N, 0, 1, 1) == 0, H.hl_last_error()
+    got = pair.cpu().numpy().astype(np.float64)
+    np.testing.assert_allclose(got[:, 0], want.astype(np.float64), **TOL[dtype])
+    np.testing.assert_allclose(got[:, 1], ref.linear(x, w2).astype(np.float64), **TOL[dtype])
+
+
+def _random_layers(rng, dtype, Hq, Hkv, D, I, L, bias=True):
+    hidden = Hq * D
+    out = []
+    for _ in range(L):
+        out.append({
+            "attn_norm": rng.uniform(0.5, 1.5, hidden).astype(dtype), "ffn_norm": rng.uniform(0.5, 1.5, hidden).astype(dtype),
+            "wqkv": (rng.standard_normal((hidden, (Hq + 2 * Hkv) * D)) / np.sqrt(hidden)).astype(dtype),
+            "bqkv": (rng.standard_normal((Hq + 2 * Hkv) * D) * 0.1).astype(dtype) if bias else None,
+            "wo": (rng.standard_normal((hidden, hidden)) / np.sqrt(hidden)).astype(dtype),
+            "bo": (rng.standard_normal(hidden) * 0.1).astype(dtype) if bias else None,
+            "wgate": (rng.standard_normal((hidden, I)) / np.sqrt(hidden)).astype(dtype),
+            "wup": (rng.standard_normal((hidden, I)) / np.sqrt(hidden)).astype(dtype),
+            "wdown": (rng.standard_normal((I, hidden)) / np.sqrt(I)).astype(dtype),
+            "bdown": (rng.standard_normal(hidden) * 0.1).astype(dtype) if bias else None,
+        })
+    return out
+
+
+class GpuDecoder:
+    """LlamaSelfDecoder over device copies of `layers`, created and driven through the C harness."""
+
+    ORDER = ["attn_norm", "ffn_norm", "wqkv", "bqkv", "wo", "bo", "wdown", "bdown", "wgate", "wup"]
+
+    def __init__(self, H, torch, dtype, B, Hq, Hkv, D, I, S, rotary_dim, base, eps, layers, output_norm, attn_bias=True):
+        self.H, self.torch = H, torch
+        self.keep = []
+        L = len(layers)
+        arrays = []
+        for name in self.ORDER:
+            arr = (ctypes.c_void_p * L)()
+            for l, w in enumerate(layers):
+                if w[name] is None:
+                    arr[l] = None
+                else:
+                    t = _dev(torch, w[name])
+                    self.keep.append(t)
+                    arr[l] = t.data_ptr()
+            arrays.append(arr)
+        self.out_norm = _dev(torch, output_norm)
+        code = 1 if dtype == np.float16 else 0
+        self.handle = H.hl_decoder_create(code, B, Hq, Hkv, D, I, L, S, rotary_dim, base, eps, int(attn_bias), *arrays,
+                                          self.out_norm.data_ptr())
+        assert self.handle, H.hl_last_error()
+
+    def forward(self, step, x, y, kc, vc):
+        rc = self.H.hl_decoder_forward(self.handle, step, x.data_ptr(), y.data_ptr(), kc.data_ptr(), vc.data_ptr())
+        assert rc == 0, self.H.hl_last_error()
+        self.torch.cuda.synchronize()
+
+    def close(self):
+        self.H.hl_decoder_destroy(self.handle)
+        self.handle = None
+
+
+STEP_TOL = {np.float32: dict(rtol=2e-4, atol=2e-4), np.float16: dict(rtol=3e-2, atol=3e-2)}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,B,Hq,Hkv,D,I,L,S,t,rotary", [
+    (np.float32, 2, 4, 2, 8, 12, 2, 12, 3, 128),        # examples/cpp/decoder/self_decoder_example.cpp:10-27
+    (np.float32, 3, 8, 2, 64, 172, 2, 40, 33, 64),
+    (np.float16, 4, 8, 2, 128, 1024, 2, 300, 257, 128),
+    (np.float16, 2, 32, 32, 128, 1408, 1, 64, 64, 128),
+    (np.float16, 1, 4, 4, 64, 96, 3, 16, 1, 64),
+])
+def test_decoder_step_matches_the_oracle(H, ref, dtype, B, Hq, Hkv, D, I, L, S, t, rotary):
+    import torch
+    announce("decoder step", dtype.__name__, B, Hq, Hkv, D, I, L, S, "t", t)
+    rng = np.random.default_rng(B * 1000 + Hq * 10 + t)
+    hidden, eps = Hq * D, 1e-5
+    layers = _random_layers(rng, dtype, Hq, Hkv, D, I, L)
+    out_norm = rng.uniform(0.5, 1.5, hidden).astype(dtype)
+    x = rng.standard_normal((B, hidden)).astype(dtype)
+    kc = np.zeros((L, B, Hkv, S, D), dtype)
+    vc = np.zeros((L, B, Hkv, S, D), dtype)
+    kc[:, :, :, :t - 1] = (rng.standard_normal((L, B, Hkv, t - 1, D)) * 0.5).astype(dtype)
+    vc[:, :, :, :t - 1] = (rng.standard_normal((L, B, Hkv, t - 1, D)) * 0.5).astype(dtype)
+
+    r_x, r_kc, r_vc = x.copy(), kc.copy(), vc.copy()
+    want = ref.self_decoder_step(r_x, layers, out_norm, r_kc, r_vc, Hq, t, rotary, 10000.0, eps)
+
+    dec = GpuDecoder(H, torch, dtype, B, Hq, Hkv, D, I, S, rotary, 10000.0, eps, layers, out_norm)
+    try:
+        g_x, g_kc, g_vc = _dev(torch, x), _dev(torch, kc), _dev(torch, vc)
+        g_y = torch.zeros_like(g_x)
+        dec.forward(t, g_x, g_y, g_kc, g_vc)
+        f64 = lambda a: a.cpu().numpy().astype(np.float64)
+        np.testing.assert_allclose(f64(g_y), want.astype(np.float64), **STEP_TOL[dtype])
+        np.testing.assert_allclose(f64(g_x), r_x.astype(np.float64), **STEP_TOL[dtype])            # residual stream
+        np.testing.assert_allclose(f64(g_kc), r_kc.astype(np.float64), **STEP_TOL[dtype])          # row t-1 of every layer
+        np.testing.assert_allclose(f64(g_vc), r_vc.astype(np.float64), **STEP_TOL[dtype])
+        assert np.abs(f64(g_y) - want.astype(np.float64)).mean() < (2e-5 if dtype == np.float32 else 4e-3)
+        # history rows and rows past t are untouched, bit for bit
+        got_k = g_kc.cpu().numpy()
+        np.testing.assert_array_equal(got_k[:, :, :, :t - 1].view(np.uint8), kc[:, :, :, :t - 1].view(np.uint8))
+        assert not got_k[:, :, :, t:].any()
+        # a second step on the grown cache, buffers recycled by the allocator
+        x2 = rng.standard_normal((B, hidden)).astype(dtype)
+        if t < S:
+            r_x2 = x2.copy()
+            want2 = ref.self_decoder_step(r_x2, layers, out_norm, r_kc, r_vc, Hq, t + 1, rotary, 10000.0, eps)
+            g_x2 = _dev(torch, x2)
+            dec.forward(t + 1, g_x2, g_y, g_kc, g_vc)
+            np.testing.assert_allclose(f64(g_y), want2.astype(np.float64), **STEP_TOL[dtype])
+    finally:
+        dec.close()
+
+
+@pytest.mark.gpu
+def test_decoder_without_attention_bias_and_reference_rope_position(H, ref):
+    """attn_bias = false drops the qkv / output biases (src/weights/llama/layer_weights.cc:26-29)."""
+    import torch
+    announce("decoder step without biases")
+    rng = np.random.default_rng(5)
+    dtype, B, Hq, Hkv, D, I, L, S, t = np.float32, 2, 4, 2, 16, 24, 2, 10, 6
+    hidden = Hq * D
+    layers = _random_layers(rng, dtype, Hq, Hkv, D, I, L, bias=False)
+    out_norm = rng.uniform(0.5, 1.5, hidden).astype(dtype)
+    x = rng.standard_normal((B, hidden)).astype(dtype)
+    kc = (rng.standard_normal((L, B, Hkv, S, D)) * 0.5).astype(dtype)
+    vc = (rng.standard_normal((L, B, Hkv, S, D)) * 0.5).astype(dtype)
+    r_x, r_kc, r_vc = x.copy(), kc.copy(), vc.copy()
+    want = ref.self_decoder_step(r_x, layers, out_norm, r_kc, r_vc, Hq, t, D, 10000.0, 1e-5)
+    dec = GpuDecoder(H, torch, dtype, B, Hq, Hkv, D, I, S, D, 10000.0, 1e-5, layers, out_norm, attn_bias=False)
+    try:
+        g_x, g_kc, g_vc = _dev(torch, x), _dev(torch, kc), _dev(torch, vc)
+        g_y = torch.zeros_like(g_x)
+        dec.forward(t, g_x, g_y, g_kc, g_vc)
+        np.testing.assert_allclose(g_y.cpu().numpy(), want, **STEP_TOL[dtype])
+        np.testing.assert_allclose(g_kc.cpu().numpy(), r_kc, **STEP_TOL[dtype])
+    finally:
+        dec.close()
