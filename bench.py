@@ -164,6 +164,9 @@ def decoder_layer_section(capi, dev, args):
     ws_attn = torch.empty(capi.decode_attn_workspace_bytes(B, H, H, D, t), dtype=torch.uint8, device=dev)
     ws_gemm = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dev)
 
+    for (K_, N_, ld_) in ((hid, 3 * hid, 0), (hid, hid, 0), (hid, I, 2 * I), (I, hid, 0)):
+        capi.linear_tune(capi.FP16, B, K_, N_, ldy=ld_, workspace=ws_gemm)
+
     def norm_in(i):
         y.copy_(x)
         capi.rmsnorm(y, g1, 1e-5)
@@ -205,11 +208,26 @@ def decoder_layer_section(capi, dev, args):
             fn(i)
 
     steps = max(args.steps // 3, 10)
-    ms = time_steps(layer, steps, max(args.warmup // 3, 3))
+    # the whole layer as the C++ LlamaSelfDecoder queues it (one call per step; its output-projection and down-projection
+    # biases are applied by the fused norms, as above)
+    dec = capi.SelfDecoder(capi.FP16, B, H, H, D, I, S, D, 10000.0, 1e-5,
+                           [dict(attn_norm=g1, ffn_norm=g2, wqkv=wqkv, bqkv=bqkv, wo=wo, bo=bo, wdown=wd, bdown=bd, wgate=wg, wup=wu)],
+                           g3)
+
+    def layer_cpp(i):
+        if i % 8 == 0:
+            x.copy_(x0)
+        kc, vc = sets[i % len(sets)]
+        dec.forward(t, x, y, kc, vc)
+
+    ms = time_steps(layer_cpp, steps, max(args.warmup // 3, 3))
+    dec.close()
+    ms_py = time_steps(layer, steps, 3)
     weight_bytes = 2 * (wqkv.numel() + wo.numel() + wg.numel() + wu.numel() + wd.numel())
     nb = weight_bytes + attn_bytes(B, H, H, D, [t] * B, 2)
     e = entry(ms, nb)
     e["parts_us"] = {name: round(time_steps(fn, steps, 3) * 1e3, 2) for name, fn in parts}
+    e["us_same_sequence_from_python"] = round(ms_py * 1e3, 2)
     e["gemm_path"] = "hipBLASLt" if capi.gemm_lib().onellm_linear_last_path() == 1 else "plain kernel"
     e["note"] = ("bytes = the five weight matrices (%d) + the attention step's algorithmic bytes; parts are timed "
                  "one at a time, so their sum includes a launch gap per part" % weight_bytes)

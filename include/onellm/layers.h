@@ -44,6 +44,11 @@ class cublasWrapper;   // carried for signature compatibility only; may be null,
 void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool trans_a = false, bool trans_b = false,
                       bool shared_out_buf = false);
 
+// launchLinearGemm times the GEMM library's candidate algorithms the first time it sees a shape and keeps the fastest;
+// that first call synchronises the null stream.  Switch it off to keep every call asynchronous (for example before
+// capturing a step into a graph; shapes tuned earlier stay tuned).
+void setLinearGemmAutotune(bool on);
+
 class LLaMASelfAttentionLayer {
 public:
     LLaMASelfAttentionLayer(int head_num, int kv_head_num, int head_size, LLaMAAttentionStaticParams attn_params,

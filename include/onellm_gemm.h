@@ -28,6 +28,14 @@ extern "C" {
 int onellm_linear(int dtype, const void* x, const void* w, void* y, int M, int K, int N, int ldy, int w_is_nk,
                   void* workspace, size_t workspace_bytes, onellm_stream_t stream);
 
+/* Optional, once per shape (for example when a model is loaded): times the library's candidate algorithms for this
+ * problem on stand-in operands it allocates and frees itself, and makes onellm_linear use the fastest one for this
+ * (dtype, M, K, N, ldy, w_is_nk, workspace or not) from then on instead of the library's first suggestion.
+ * Synchronises the stream.  best_us / first_us (either may be NULL) receive the time of the chosen algorithm and of
+ * the library's first suggestion.  ONELLM_EUNSUPPORTED if the library has no algorithm for the problem. */
+int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
+                       onellm_stream_t stream, float* best_us, float* first_us);
+
 /* workspace size onellm_linear can make use of (a constant; any smaller size is valid too) */
 size_t onellm_linear_workspace_bytes(void);
 

@@ -27,14 +27,12 @@ LIB_LAYERS = os.path.join(HERE, "libonellm_layers.so")
 # test-only: a C wrapper that drives the launcher shims with oneLLM-style Tensor objects
 HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "launcher_harness.cpp")
 LIB_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
-LAYERS_HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "layers_harness.cpp")
-LIB_LAYERS_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblayers_harness.so")
 
 KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip", "sampling.hip",
                   "tuning.cpp"]
 LAUNCHER_SOURCES = ["launchers.cpp"]
 GEMM_SOURCES = ["linear.hip"]
-LAYER_SOURCES = ["layers.cpp"]
+LAYER_SOURCES = ["layers.cpp", "layers_capi.cpp"]
 
 # packed fp32 VALU forms are switched off on purpose (code generation only; scalar fp32 code is
 # what the kernels are written in)
@@ -98,13 +96,6 @@ def build(force=False, verbose=False):
         cmd = [HIPCC, "-shared", "-fPIC", "-o", LIB_LAYERS] + yobjs + \
               ["-L" + HERE, "-lonellm_gemm", "-lonellm_launchers", "-lonellm_hip", "-Wl,-rpath,$ORIGIN"]
         subprocess.run(cmd, check=True, capture_output=not verbose)
-    if os.path.exists(LAYERS_HARNESS_SRC) and (force or _newer(LIB_LAYERS_HARNESS, [LAYERS_HARNESS_SRC, LIB_LAYERS] + _headers())):
-        cmd = [HIPCC, "-shared", "-fPIC", "-O2", "-std=c++17", "-I" + INCLUDE, LAYERS_HARNESS_SRC, "-o", LIB_LAYERS_HARNESS,
-               "-L" + HERE, "-lonellm_layers", "-lonellm_gemm", "-lonellm_launchers", "-lonellm_hip",
-               "-Wl,-rpath,$ORIGIN/../../onellm_amd"]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError("hipcc failed for the layers harness:\n" + r.stderr[-4000:])
     return LIB_HIP, LIB_LAUNCH, LIB_GEMM, LIB_LAYERS
 
 

@@ -201,6 +201,7 @@ GEMM_PATH = os.path.join(_HERE, "libonellm_gemm.so")
 LAYERS_PATH = os.path.join(_HERE, "libonellm_layers.so")
 GEMM_SYMBOLS = {
     "onellm_linear": (_ci, [_ci, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
+    "onellm_linear_tune": (_ci, [_ci, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp, ctypes.POINTER(_cf), ctypes.POINTER(_cf)]),
     "onellm_linear_workspace_bytes": (_sz, []),
     "onellm_linear_last_path": (_ci, []),
 }
@@ -227,6 +228,16 @@ def linear_workspace_bytes():
     return gemm_lib().onellm_linear_workspace_bytes()
 
 
+def linear_tune(dtype_code, M, K, N, ldy=0, w_is_nk=False, workspace=None):
+    """Time the library's candidates for this problem once and keep the fastest; returns (best_us, first_us)."""
+    best, first = _cf(0.0), _cf(0.0)
+    rc = gemm_lib().onellm_linear_tune(dtype_code, M, K, N, int(ldy), int(bool(w_is_nk)), _ptr(workspace),
+                                       workspace.numel() if workspace is not None else 0, _stream(), ctypes.byref(best),
+                                       ctypes.byref(first))
+    _check(rc, "onellm_linear_tune")
+    return best.value, first.value
+
+
 def linear(x, w, y, w_is_nk=False, ldy=0, workspace=None):
     """y[M, N] = x[M, K] . W (W [K, N], or [N, K] with w_is_nk); y may be a strided view given by its first element
     and `ldy`.  `workspace`: uint8 device tensor or None."""
@@ -238,3 +249,58 @@ def linear(x, w, y, w_is_nk=False, ldy=0, workspace=None):
                                   _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream())
     _check(rc, "onellm_linear")
     return y
+
+
+# ---------------------------------------------------------------- decode-side layers (include/onellm_layers.h)
+_layers = None
+
+
+def layers_lib():
+    global _layers
+    if _layers is None:
+        if not os.path.exists(LAYERS_PATH):
+            raise RuntimeError(f"{LAYERS_PATH} is missing: build it with `python -m onellm_amd.build`")
+        gemm_lib()
+        L = ctypes.CDLL(LAYERS_PATH)
+        pp = ctypes.POINTER(ctypes.c_void_p)
+        L.onellm_layers_last_error.restype = ctypes.c_char_p
+        L.onellm_layers_linear.argtypes = [_ci, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci]
+        L.onellm_decoder_create.restype = _vp
+        L.onellm_decoder_create.argtypes = [_ci] * 9 + [_cf, _cf, _ci] + [pp] * 10 + [_vp]
+        L.onellm_decoder_forward.argtypes = [_vp, _ci, _vp, _vp, _vp, _vp]
+        L.onellm_decoder_destroy.argtypes = [_vp]
+        _layers = L
+    return _layers
+
+
+class SelfDecoder:
+    """LlamaSelfDecoder over device tensors.  `layers`: list of dicts of torch device tensors with the keys attn_norm,
+    ffn_norm, wqkv, bqkv, wo, bo, wdown, bdown, wgate, wup (weights [in, out]; a bias may be None)."""
+
+    ORDER = ["attn_norm", "ffn_norm", "wqkv", "bqkv", "wo", "bo", "wdown", "bdown", "wgate", "wup"]
+
+    def __init__(self, dtype_code, B, Hq, Hkv, D, inter_size, S, rotary_dim, rope_base, eps, layers, output_norm, attn_bias=True):
+        self.L = layers_lib()
+        self._keep = (layers, output_norm)
+        n = len(layers)
+        arrays = []
+        for name in self.ORDER:
+            arr = (ctypes.c_void_p * n)()
+            for l, w in enumerate(layers):
+                arr[l] = None if w[name] is None else _ptr(w[name])
+            arrays.append(arr)
+        self.handle = self.L.onellm_decoder_create(dtype_code, B, Hq, Hkv, D, inter_size, n, S, rotary_dim, rope_base, eps,
+                                                   int(attn_bias), *arrays, _ptr(output_norm))
+        if not self.handle:
+            raise RuntimeError(self.L.onellm_layers_last_error().decode())
+
+    def forward(self, step, decoder_input, decoder_output, k_cache, v_cache):
+        rc = self.L.onellm_decoder_forward(self.handle, int(step), _ptr(decoder_input), _ptr(decoder_output), _ptr(k_cache),
+                                           _ptr(v_cache))
+        if rc != 0:
+            raise RuntimeError(self.L.onellm_layers_last_error().decode())
+
+    def close(self):
+        if self.handle:
+            self.L.onellm_decoder_destroy(self.handle)
+            self.handle = None

@@ -1,6 +1,8 @@
 // Decode-side layers of oneLLM over this backend (declared in onellm/layers.h): they sequence the launch*
 // functions and the projection GEMMs for one decode step and own no arithmetic of their own.
 #include <mutex>
+#include <set>
+#include <tuple>
 #include <stdexcept>
 #include <string>
 #include <hip/hip_runtime_api.h>
@@ -47,6 +49,22 @@ struct GemmWorkspace {
 };
 GemmWorkspace g_gemm_ws;
 
+// The first time a projection shape is seen, the library's candidate algorithms are timed once and the fastest is
+// kept (the first suggestion is up to 1.7x slower on the skinny decode shapes).  That one call synchronises the
+// stream; setLinearGemmAutotune(false) keeps every call asynchronous.
+std::mutex g_tuned_mu;
+std::set<std::tuple<int, int, int, int, int, int>> g_tuned;
+bool g_autotune = true;
+
+void tune_once(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* ws, size_t ws_bytes)
+{
+    {
+        std::lock_guard<std::mutex> g(g_tuned_mu);
+        if (!g_autotune || !g_tuned.insert(std::make_tuple(dtype, M, K, N, ldy, w_is_nk)).second) return;
+    }
+    (void)onellm_linear_tune(dtype, M, K, N, ldy, w_is_nk, ws, ws_bytes, nullptr, nullptr, nullptr);   // best effort
+}
+
 Tensor* new_buffer(BaseAllocator* a, DataType t, std::vector<int> shape)
 {
     size_t n = elt_bytes(t);
@@ -64,6 +82,12 @@ void drop_buffer(BaseAllocator* a, Tensor*& buf)
 }
 
 }  // namespace
+
+void setLinearGemmAutotune(bool on)
+{
+    std::lock_guard<std::mutex> g(g_tuned_mu);
+    g_autotune = on;
+}
 
 // src/kernels/qkv_linear.cu:8-66
 void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool trans_a, bool trans_b, bool shared_out_buf)
@@ -92,6 +116,8 @@ void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool tr
         require(rows_of(output) == M && cols_of(output) == N, "launchLinearGemm: output shape");
     }
     void* ws = g_gemm_ws.get();
+    const int dtype_code = input->dtype == FP32 ? ONELLM_FP32 : ONELLM_FP16;
+    tune_once(dtype_code, M, K, N, ldy, trans_b ? 1 : 0, ws, g_gemm_ws.bytes);
     const int rc = onellm_linear(input->dtype == FP32 ? ONELLM_FP32 : ONELLM_FP16, input->data, weight.data, y, M, K, N, ldy,
                                  trans_b ? 1 : 0, ws, g_gemm_ws.bytes, nullptr);
     if (rc != 0) throw std::runtime_error(std::string("[TM][ERROR] launchLinearGemm: ") + onellm_error_string(rc) + " \n");

@@ -1,14 +1,16 @@
-// Test harness for the decode-side layers: a C surface over LlamaSelfDecoder / launchLinearGemm that builds the
-// Tensor, TensorMap and LlamaLayerWeight objects the way examples/cpp/decoder/self_decoder_example.cpp does, from raw
-// device pointers handed in from Python.  C++ exceptions become return code 1 + a message.
+// C surface over LlamaSelfDecoder / launchLinearGemm (declared in onellm_layers.h) for callers that cannot build
+// C++ objects: it assembles the Tensor, TensorMap and LlamaLayerWeight objects the way
+// examples/cpp/decoder/self_decoder_example.cpp does, from raw device pointers.  C++ exceptions become return code 1 +
+// a message.
 #include <exception>
 #include <memory>
 #include <string>
 #include <vector>
 #include "onellm/layers.h"
+#include "onellm_layers.h"
 
 namespace {
-std::string g_last_error;
+thread_local std::string g_last_error;
 
 template <typename F>
 int guarded(F&& f)
@@ -37,10 +39,10 @@ struct Decoder {
 
 extern "C" {
 
-const char* hl_last_error() { return g_last_error.c_str(); }
+const char* onellm_layers_last_error() { return g_last_error.c_str(); }
 
 // pair: y is the {2, M, N} gate/up buffer; second: write its second slot (shared_out_buf)
-int hl_linear(int dtype, void* x, void* w, void* y, int M, int K, int N, int trans_b, int pair, int second)
+int onellm_layers_linear(int dtype, void* x, void* w, void* y, int M, int K, int N, int trans_b, int pair, int second)
 {
     return guarded([&] {
         Tensor in(GPU, dt(dtype), {M, K}, x);
@@ -55,7 +57,7 @@ int hl_linear(int dtype, void* x, void* w, void* y, int M, int K, int N, int tra
 }
 
 // per-layer pointer arrays of length L, in the argument order of LlamaLayerWeight::loadWeights
-void* hl_decoder_create(int dtype, int B, int Hq, int Hkv, int D, int I, int L, int S, int rotary_dim, float rope_base,
+void* onellm_decoder_create(int dtype, int B, int Hq, int Hkv, int D, int I, int L, int S, int rotary_dim, float rope_base,
                         float eps, int attn_bias, void** attn_norm, void** ffn_norm, void** wqkv, void** bqkv, void** wo,
                         void** bo, void** wdown, void** bdown, void** wgate, void** wup, void* output_norm)
 {
@@ -84,7 +86,7 @@ void* hl_decoder_create(int dtype, int B, int Hq, int Hkv, int D, int I, int L, 
     return d;
 }
 
-int hl_decoder_forward(void* handle, int step_value, void* decoder_input, void* decoder_output, void* k_cache, void* v_cache)
+int onellm_decoder_forward(void* handle, int step_value, void* decoder_input, void* decoder_output, void* k_cache, void* v_cache)
 {
     return guarded([&] {
         Decoder* d = static_cast<Decoder*>(handle);
@@ -105,6 +107,6 @@ int hl_decoder_forward(void* handle, int step_value, void* decoder_input, void* 
     });
 }
 
-void hl_decoder_destroy(void* handle) { delete static_cast<Decoder*>(handle); }
+void onellm_decoder_destroy(void* handle) { delete static_cast<Decoder*>(handle); }
 
 }  // extern "C"

@@ -59,7 +59,8 @@ thread_local int t_last_path = 0;
 
 // Row-major y[M,N] = x[M,K].W[K,N] is, read column-major, y^T[N,M] = W^T[N,K] . x^T[K,M]: the buffers are passed
 // as they are with A = W (leading dimension N, or K with a transpose when W is [N,K]) and B = x.
-Plan make_plan(hipblasLtHandle_t h, int dtype, int M, int K, int N, int ldy, int w_is_nk, size_t ws_bytes)
+// Descriptor and layouts of one problem; `heur` is filled by the callers below.
+Plan make_problem(int dtype, int M, int K, int N, int ldy, int w_is_nk)
 {
     Plan p;
     const hipDataType dt = dtype == ONELLM_FP16 ? HIP_R_16F : HIP_R_32F;
@@ -72,15 +73,33 @@ Plan make_plan(hipblasLtHandle_t h, int dtype, int M, int K, int N, int ldy, int
     else ok &= hipblasLtMatrixLayoutCreate(&p.la, dt, N, K, N) == HIPBLAS_STATUS_SUCCESS;
     ok &= hipblasLtMatrixLayoutCreate(&p.lb, dt, K, M, K) == HIPBLAS_STATUS_SUCCESS;
     ok &= hipblasLtMatrixLayoutCreate(&p.lc, dt, N, M, ldy) == HIPBLAS_STATUS_SUCCESS;
-    if (!ok) return p;
+    p.usable = ok;
+    return p;
+}
+
+// the library's ranked candidates for a problem (at most `want`), those that fit the workspace
+int candidates(hipblasLtHandle_t h, const Plan& p, size_t ws_bytes, hipblasLtMatmulHeuristicResult_t* out, int want)
+{
     hipblasLtMatmulPreference_t pref = nullptr;
-    if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
+    if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return 0;
     const uint64_t max_ws = ws_bytes;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
     int found = 0;
-    const hipblasStatus_t s = hipblasLtMatmulAlgoGetHeuristic(h, p.desc, p.la, p.lb, p.lc, p.lc, pref, 1, &p.heur, &found);
+    const hipblasStatus_t s = hipblasLtMatmulAlgoGetHeuristic(h, p.desc, p.la, p.lb, p.lc, p.lc, pref, want, out, &found);
     hipblasLtMatmulPreferenceDestroy(pref);
-    p.usable = s == HIPBLAS_STATUS_SUCCESS && found > 0 && p.heur.workspaceSize <= ws_bytes;
+    if (s != HIPBLAS_STATUS_SUCCESS) return 0;
+    int kept = 0;
+    for (int i = 0; i < found; ++i)
+        if (out[i].workspaceSize <= ws_bytes) out[kept++] = out[i];
+    return kept;
+}
+
+// the library's first suggestion for a problem
+Plan make_plan(hipblasLtHandle_t h, int dtype, int M, int K, int N, int ldy, int w_is_nk, size_t ws_bytes)
+{
+    Plan p = make_problem(dtype, M, K, N, ldy, w_is_nk);
+    if (!p.usable) return p;
+    p.usable = candidates(h, p, ws_bytes, &p.heur, 1) == 1;
     return p;
 }
 
@@ -96,6 +115,111 @@ int run_plain(const void* x, const void* w, void* y, int M, int K, int N, int ld
 
 }  // namespace
 }  // namespace onellm
+
+namespace onellm {
+namespace {
+// caller holds g_mu
+hipblasLtHandle_t device_handle(DeviceState& ds)
+{
+    if (!ds.handle && !ds.handle_failed) {
+        if (hipblasLtCreate(&ds.handle) != HIPBLAS_STATUS_SUCCESS) {
+            ds.handle = nullptr;
+            ds.handle_failed = true;
+        }
+    }
+    return ds.handle;
+}
+}  // namespace
+}  // namespace onellm
+
+extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
+                                  onellm_stream_t stream, float* best_us, float* first_us)
+{
+    using namespace onellm;
+    if (dtype != ONELLM_FP32 && dtype != ONELLM_FP16) return ONELLM_EINVAL;
+    if (M <= 0 || K <= 0 || N <= 0) return ONELLM_EINVAL;
+    if (ldy == 0) ldy = N;
+    if (ldy < N) return ONELLM_EINVAL;
+    if (!workspace) workspace_bytes = 0;
+    if (workspace_bytes > kWorkspaceBytes) workspace_bytes = kWorkspaceBytes;
+    w_is_nk = w_is_nk ? 1 : 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+
+    hipblasLtHandle_t handle = nullptr;
+    {
+        std::lock_guard<std::mutex> g(g_mu);
+        handle = device_handle(g_devices[dev]);
+    }
+    if (!handle) return ONELLM_EUNSUPPORTED;
+    Plan p = make_problem(dtype, M, K, N, ldy, w_is_nk);
+    if (!p.usable) return ONELLM_EUNSUPPORTED;
+    constexpr int kWant = 32;
+    hipblasLtMatmulHeuristicResult_t cand[kWant];
+    const int n = candidates(handle, p, workspace_bytes, cand, kWant);
+    if (n == 0) return ONELLM_EUNSUPPORTED;
+
+    // stand-in operands of the right size (values do not matter for the timing; 0x3c3c.. is ~1.06 in fp16 and a
+    // small normal number in fp32)
+    const size_t esz = dtype == ONELLM_FP16 ? 2 : 4;
+    void *x = nullptr, *w = nullptr, *y = nullptr;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    int rc = 0;
+    auto cleanup = [&] {
+        if (x) (void)hipFree(x);
+        if (w) (void)hipFree(w);
+        if (y) (void)hipFree(y);
+        if (t0) (void)hipEventDestroy(t0);
+        if (t1) (void)hipEventDestroy(t1);
+    };
+    if ((e = hipMalloc(&x, (size_t)M * K * esz)) != hipSuccess || (e = hipMalloc(&w, (size_t)K * N * esz)) != hipSuccess ||
+        (e = hipMalloc(&y, (size_t)M * ldy * esz)) != hipSuccess || (e = hipEventCreate(&t0)) != hipSuccess ||
+        (e = hipEventCreate(&t1)) != hipSuccess) {
+        cleanup();
+        return (int)e;
+    }
+    (void)hipMemsetAsync(x, 0x3c, (size_t)M * K * esz, st);
+    (void)hipMemsetAsync(w, 0x3c, (size_t)K * N * esz, st);
+    const float alpha = 1.f, beta = 0.f;
+    int best = -1;
+    float best_ms = 0.f, first_ms = 0.f;
+    constexpr int kWarm = 2, kRuns = 8;
+    for (int i = 0; i < n; ++i) {
+        bool ok = true;
+        for (int r = 0; r < kWarm + kRuns && ok; ++r) {
+            if (r == kWarm) (void)hipEventRecord(t0, st);
+            ok = hipblasLtMatmul(handle, p.desc, &alpha, w, p.la, x, p.lb, &beta, y, p.lc, y, p.lc, &cand[i].algo, workspace,
+                                 workspace_bytes, st) == HIPBLAS_STATUS_SUCCESS;
+        }
+        (void)hipEventRecord(t1, st);
+        if ((e = hipEventSynchronize(t1)) != hipSuccess) {
+            rc = (int)e;
+            break;
+        }
+        if (!ok) continue;
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, t0, t1);
+        ms /= kRuns;
+        if (i == 0) first_ms = ms;
+        if (best < 0 || ms < best_ms) {
+            best = i;
+            best_ms = ms;
+        }
+    }
+    cleanup();
+    if (rc != 0) return rc;
+    if (best < 0) return ONELLM_EUNSUPPORTED;
+    p.heur = cand[best];
+    {
+        std::lock_guard<std::mutex> g(g_mu);
+        g_devices[dev].plans[std::make_tuple(dtype, M, K, N, ldy, w_is_nk, workspace_bytes ? 1 : 0)] = p;
+    }
+    if (best_us) *best_us = best_ms * 1e3f;
+    if (first_us) *first_us = first_ms * 1e3f;
+    return 0;
+}
 
 extern "C" size_t onellm_linear_workspace_bytes(void) { return onellm::kWorkspaceBytes; }
 
@@ -126,12 +250,7 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
     {
         std::lock_guard<std::mutex> g(g_mu);
         DeviceState& ds = g_devices[dev];
-        if (!ds.handle && !ds.handle_failed) {
-            if (hipblasLtCreate(&ds.handle) != HIPBLAS_STATUS_SUCCESS) {
-                ds.handle = nullptr;
-                ds.handle_failed = true;
-            }
-        }
+        device_handle(ds);
         handle = ds.handle;
         if (handle) {
             const auto key = std::make_tuple(dtype, M, K, N, ldy, w_is_nk, workspace_bytes ? 1 : 0);

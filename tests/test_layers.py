@@ -1,6 +1,7 @@
 """The decode-side layers (include/onellm/layers.h: launchLinearGemm, LLaMASelfAttentionLayer, LLaMAFFNLayer,
-LlamaSelfDecoder) and the projection C ABI under them (include/onellm_gemm.h), driven through a small C harness that
-builds Tensor / TensorMap / LlamaLayerWeight objects the way examples/cpp/decoder/self_decoder_example.cpp does.
+LlamaSelfDecoder) and the projection C ABI under them (include/onellm_gemm.h), driven through the layers' C surface
+(include/onellm_layers.h), which builds Tensor / TensorMap / LlamaLayerWeight objects the way
+examples/cpp/decoder/self_decoder_example.cpp does.
 Host-side behaviour runs without a GPU; parity against the CPU oracle (oracle/ref.py: linear, self_decoder_step — the
 latter pinned on an independent library implementation in tests/test_oracle_layers.py) is marked gpu."""
 import ctypes
@@ -14,24 +15,23 @@ import pytest
 from conftest import announce
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HARNESS = os.path.join(ROOT, "tests", "cpp", "liblayers_harness.so")
 LIB_GEMM = os.path.join(ROOT, "onellm_amd", "libonellm_gemm.so")
 LIB_LAYERS = os.path.join(ROOT, "onellm_amd", "libonellm_layers.so")
 
 
 @pytest.fixture(scope="module")
 def H():
-    assert os.path.exists(HARNESS), "build it with `python -m onellm_amd.build`"
+    assert os.path.exists(LIB_LAYERS), "build it with `python -m onellm_amd.build`"
     import torch  # noqa: F401  first, so that the HIP runtime and BLAS library torch ships are the ones this process uses
-    L = ctypes.CDLL(HARNESS)
+    L = ctypes.CDLL(LIB_LAYERS)
     vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
     pp = ctypes.POINTER(ctypes.c_void_p)
-    L.hl_last_error.restype = ctypes.c_char_p
-    L.hl_linear.argtypes = [ci, vp, vp, vp, ci, ci, ci, ci, ci, ci]
-    L.hl_decoder_create.restype = vp
-    L.hl_decoder_create.argtypes = [ci] * 9 + [cf, cf, ci] + [pp] * 10 + [vp]
-    L.hl_decoder_forward.argtypes = [vp, ci, vp, vp, vp, vp]
-    L.hl_decoder_destroy.argtypes = [vp]
+    L.onellm_layers_last_error.restype = ctypes.c_char_p
+    L.onellm_layers_linear.argtypes = [ci, vp, vp, vp, ci, ci, ci, ci, ci, ci]
+    L.onellm_decoder_create.restype = vp
+    L.onellm_decoder_create.argtypes = [ci] * 9 + [cf, cf, ci] + [pp] * 10 + [vp]
+    L.onellm_decoder_forward.argtypes = [vp, ci, vp, vp, vp, vp]
+    L.onellm_decoder_destroy.argtypes = [vp]
     return L
 
 
@@ -51,7 +51,7 @@ def test_gemm_library_exports_what_its_header_declares(G):
     text = open(os.path.join(ROOT, "include", "onellm_gemm.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = sorted(set(re.findall(r"\b(onellm_[a-z0-9_]+)\s*\(", text)))
-    assert names == ["onellm_linear", "onellm_linear_last_path", "onellm_linear_workspace_bytes"]
+    assert names == ["onellm_linear", "onellm_linear_last_path", "onellm_linear_tune", "onellm_linear_workspace_bytes"]
     for n in names:
         assert hasattr(G, n)
     assert G.onellm_linear_workspace_bytes() > 0
@@ -66,6 +66,16 @@ def test_linear_rejects_bad_arguments_before_any_launch(G):
     assert G.onellm_linear(0, fake, fake, fake, 0, 4, 4, 0, 0, None, 0, None) == 0         # no rows: nothing to do
 
 
+def test_layers_library_exports_its_c_surface(H):
+    text = open(os.path.join(ROOT, "include", "onellm_layers.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(onellm_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["onellm_decoder_create", "onellm_decoder_destroy", "onellm_decoder_forward", "onellm_layers_last_error",
+                     "onellm_layers_linear"]
+    for n in names:
+        assert hasattr(H, n)
+
+
 def test_layers_library_exports_reference_signatures():
     out = subprocess.run(["nm", "-DC", LIB_LAYERS], capture_output=True, text=True, check=True).stdout
     for sig in ["launchLinearGemm(Tensor*, BaseWeight&, Tensor*, bool, bool, bool)",
@@ -78,10 +88,10 @@ def test_layers_library_exports_reference_signatures():
 
 def test_linear_launcher_precondition_failures_throw(H):
     fake = ctypes.c_void_p(0x1000)
-    assert H.hl_linear(0, None, fake, fake, 2, 4, 4, 0, 0, 0) == 1
-    assert b"null tensor or weight" in H.hl_last_error()
-    assert H.hl_linear(0, fake, fake, fake, 2, 4, 4, 0, 0, 1) == 1                          # second slot without a pair buffer
-    assert b"shared_out_buf" in H.hl_last_error()
+    assert H.onellm_layers_linear(0, None, fake, fake, 2, 4, 4, 0, 0, 0) == 1
+    assert b"null tensor or weight" in H.onellm_layers_last_error()
+    assert H.onellm_layers_linear(0, fake, fake, fake, 2, 4, 4, 0, 0, 1) == 1                          # second slot without a pair buffer
+    assert b"shared_out_buf" in H.onellm_layers_last_error()
 
 
 # ---------------------------------------------------------------- GPU parity
@@ -110,20 +120,20 @@ def test_linear_matches_the_oracle(H, G, ref, dtype, M, K, N):
     dx, dw = _dev(torch, x), _dev(torch, w)
     y = torch.full((M, N), 7.0, dtype=dx.dtype, device=dx.device)
     code = 1 if dtype == np.float16 else 0
-    assert H.hl_linear(code, dx.data_ptr(), dw.data_ptr(), y.data_ptr(), M, K, N, 0, 0, 0) == 0, H.hl_last_error()
+    assert H.onellm_layers_linear(code, dx.data_ptr(), dw.data_ptr(), y.data_ptr(), M, K, N, 0, 0, 0) == 0, H.onellm_layers_last_error()
     np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[dtype])
     if K >= 4096:
         assert G.onellm_linear_last_path() == 1, "the projection shapes of a 7B layer must run the library GEMM"
     # W given as [N, K]
     dwt = _dev(torch, w.T)
     y2 = torch.zeros_like(y)
-    assert H.hl_linear(code, dx.data_ptr(), dwt.data_ptr(), y2.data_ptr(), M, K, N, 1, 0, 0) == 0, H.hl_last_error()
+    assert H.onellm_layers_linear(code, dx.data_ptr(), dwt.data_ptr(), y2.data_ptr(), M, K, N, 1, 0, 0) == 0, H.onellm_layers_last_error()
     np.testing.assert_allclose(y2.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[dtype])
     # the gate/up pair buffer: two projections into the two slots of [M, 2, N]
     w2 = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(dtype)
     pair = torch.full((M, 2, N), -3.0, dtype=dx.dtype, device=dx.device)
-    assert H.hl_linear(code, dx.data_ptr(), dw.data_ptr(), pair.data_ptr(), M, K, N, 0, 1, 0) == 0, H.hl_last_error()
-    assert H.hl_linear(code, dx.data_ptr(), _dev(torch, w2).data_ptr(), pair.data_ptr(), M, K, N, 0, 1, 1) == 0, H.hl_last_error()
+    assert H.onellm_layers_linear(code, dx.data_ptr(), dw.data_ptr(), pair.data_ptr(), M, K, N, 0, 1, 0) == 0, H.onellm_layers_last_error()
+    assert H.onellm_layers_linear(code, dx.data_ptr(), _dev(torch, w2).data_ptr(), pair.data_ptr(), M, K, N, 0, 1, 1) == 0, H.onellm_layers_last_error()
     got = pair.cpu().numpy().astype(np.float64)
     np.testing.assert_allclose(got[:, 0], want.astype(np.float64), **TOL[dtype])
     np.testing.assert_allclose(got[:, 1], ref.linear(x, w2).astype(np.float64), **TOL[dtype])
@@ -148,39 +158,21 @@ def _random_layers(rng, dtype, Hq, Hkv, D, I, L, bias=True):
 
 
 class GpuDecoder:
-    """LlamaSelfDecoder over device copies of `layers`, created and driven through the C harness."""
-
-    ORDER = ["attn_norm", "ffn_norm", "wqkv", "bqkv", "wo", "bo", "wdown", "bdown", "wgate", "wup"]
+    """capi.SelfDecoder over device copies of numpy `layers`."""
 
     def __init__(self, H, torch, dtype, B, Hq, Hkv, D, I, S, rotary_dim, base, eps, layers, output_norm, attn_bias=True):
-        self.H, self.torch = H, torch
-        self.keep = []
-        L = len(layers)
-        arrays = []
-        for name in self.ORDER:
-            arr = (ctypes.c_void_p * L)()
-            for l, w in enumerate(layers):
-                if w[name] is None:
-                    arr[l] = None
-                else:
-                    t = _dev(torch, w[name])
-                    self.keep.append(t)
-                    arr[l] = t.data_ptr()
-            arrays.append(arr)
-        self.out_norm = _dev(torch, output_norm)
-        code = 1 if dtype == np.float16 else 0
-        self.handle = H.hl_decoder_create(code, B, Hq, Hkv, D, I, L, S, rotary_dim, base, eps, int(attn_bias), *arrays,
-                                          self.out_norm.data_ptr())
-        assert self.handle, H.hl_last_error()
+        from onellm_amd import capi
+        self.torch = torch
+        dl = [{k: (None if v is None else _dev(torch, v)) for k, v in w.items()} for w in layers]
+        self.dec = capi.SelfDecoder(1 if dtype == np.float16 else 0, B, Hq, Hkv, D, I, S, rotary_dim, base, eps, dl,
+                                    _dev(torch, output_norm), attn_bias=attn_bias)
 
     def forward(self, step, x, y, kc, vc):
-        rc = self.H.hl_decoder_forward(self.handle, step, x.data_ptr(), y.data_ptr(), kc.data_ptr(), vc.data_ptr())
-        assert rc == 0, self.H.hl_last_error()
+        self.dec.forward(step, x, y, kc, vc)
         self.torch.cuda.synchronize()
 
     def close(self):
-        self.H.hl_decoder_destroy(self.handle)
-        self.handle = None
+        self.dec.close()
 
 
 STEP_TOL = {np.float32: dict(rtol=2e-4, atol=2e-4), np.float16: dict(rtol=3e-2, atol=3e-2)}
