@@ -49,6 +49,22 @@ def time_steps(fn, steps, warmup):
     return start.elapsed_time(end) / steps
 
 
+def step_distribution(fn, steps):
+    """Per-step HIP-event durations (us) of `steps` further steps: median, 10th and 90th percentile.  A separate pass
+    from the timed region that gives `value`; an event pair per step adds a marker between launches."""
+    import torch
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    torch.cuda.synchronize()
+    ev[0].record()
+    for i in range(steps):
+        fn(i)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    d = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(steps))
+    pick = lambda q: round(d[min(len(d) - 1, int(q * len(d)))], 2)
+    return {"median": pick(0.5), "p10": pick(0.1), "p90": pick(0.9), "steps": steps}
+
+
 def host_cores():
     n = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
     return min(n, os.cpu_count() or n)
@@ -95,6 +111,7 @@ def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=
         capi.decode_attn(qkv, bias, kc, vc, out, Hq, max_t, D, 10000.0, t_dev=t_dev, max_t=max_t, workspace=ws)
 
     ms = time_steps(step, steps, warmup)
+    bench_attention.last_step = step
     return ms, (qkv, bias, sets[0], out)
 
 
@@ -378,6 +395,8 @@ def main():
 
     B, H, D, S, t = 16, 32, 128, 4096, args.ctx
     ms, (qkv, bias, (kc, vc), out) = bench_attention(capi, dev, args.steps, args.warmup, B, H, H, D, S, t, nsets=4)
+    dist = step_distribution(bench_attention.last_step, min(args.steps, 200))
+    bench_attention.last_step = None
     nbytes = attn_bytes(B, H, H, D, [t] * B, 2)
     gbps = nbytes / (ms * 1e-3) / 1e9
     line = {
@@ -388,7 +407,7 @@ def main():
         "config": {"workload": "BASELINE configs[1]: batch 16, 32 heads x 128, MHA, fp16 KV cache [1,16,32,4096,128], ctx %d, "
                                "RoPE base 10000; 4 cache sets rotated per step" % t,
                    "storage": "fp16", "arithmetic": "fp32"},
-        "hbm_gbps": round(gbps, 1), "hbm_frac_of_8TBps": round(gbps / HBM_PEAK_GBPS, 4),
+        "hbm_gbps": round(gbps, 1), "hbm_frac_of_8TBps": round(gbps / HBM_PEAK_GBPS, 4), "step_us": dist,
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(t),
@@ -404,6 +423,14 @@ def main():
         line["cpu_baseline"] = {"value": round(cpu_us, 1), "unit": "us/step", "cores": host_cores(), "kind": "port",
                                 "sample": "the full batch-16 ctx-%d step (%.2f GB of fp16 KV), median of %d runs, OpenMP "
                                           "over (sequence, kv-head)" % (t, nbytes / 1e9, runs)}
+        # one host thread, on one sequence of the batch (1/16 of the step's work), scaled to the whole step
+        from oracle import ref
+        before = ref.set_threads(1)
+        one_us, runs1 = cpu_attention(qkv[:1].contiguous(), bias, kc[:, :1].contiguous(), vc[:, :1].contiguous(), H, t, D, 8.0)
+        ref.set_threads(before)
+        line["cpu_baseline"]["one_thread"] = {"value": round(one_us * B, 1), "unit": "us/step", "cores": 1,
+                                              "sample": "sequence 0 of the batch only (%.1f ms, median of %d runs), "
+                                                        "multiplied by the batch size %d" % (one_us / 1e3, runs1, B)}
     del qkv, bias, kc, vc, out
     torch.cuda.empty_cache()
     if not args.no_extras:

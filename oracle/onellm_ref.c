@@ -34,6 +34,23 @@
 #include <stdlib.h>
 #include <string.h>
 #include <immintrin.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* Number of host threads the loops below may use; returns the previous setting (1 without OpenMP).  Only the
+ * benchmark's single-thread baseline changes it. */
+int onellm_ref_set_threads(int n)
+{
+#ifdef _OPENMP
+    const int before = omp_get_max_threads();
+    if (n > 0) omp_set_num_threads(n);
+    return before;
+#else
+    (void)n;
+    return 1;
+#endif
+}
 
 #define REF_FP32 0
 #define REF_FP16 1

@@ -272,3 +272,8 @@ def self_decoder_step(x, layers, output_norm, k_cache, v_cache, Hq, t, rotary_di
         gamma = layers[l + 1]["attn_norm"] if l + 1 < L else output_norm
         fused_add_bias_residual_rmsnorm(x, y, w["bdown"] if w["bdown"] is not None else zeros, gamma, eps)
     return y
+
+
+def set_threads(n):
+    """Host threads the oracle's OpenMP loops may use; returns the previous setting."""
+    return lib().onellm_ref_set_threads(int(n))
