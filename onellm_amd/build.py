@@ -27,6 +27,9 @@ LIB_LAYERS = os.path.join(HERE, "libonellm_layers.so")
 # test-only: a C wrapper that drives the launcher shims with oneLLM-style Tensor objects
 HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "launcher_harness.cpp")
 LIB_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
+# test-only: a stand-alone C++ program that runs one decode step through the layers, like the reference's example driver
+DRIVER_SRC = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver.cpp")
+DRIVER_BIN = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver")
 
 KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip", "sampling.hip",
                   "tuning.cpp"]
@@ -96,6 +99,12 @@ def build(force=False, verbose=False):
         cmd = [HIPCC, "-shared", "-fPIC", "-o", LIB_LAYERS] + yobjs + \
               ["-L" + HERE, "-lonellm_gemm", "-lonellm_launchers", "-lonellm_hip", "-Wl,-rpath,$ORIGIN"]
         subprocess.run(cmd, check=True, capture_output=not verbose)
+    if os.path.exists(DRIVER_SRC) and (force or _newer(DRIVER_BIN, [DRIVER_SRC, LIB_LAYERS] + _headers())):
+        cmd = [HIPCC, "-O2", "-std=c++17", "-I" + INCLUDE, DRIVER_SRC, "-o", DRIVER_BIN, "-L" + HERE, "-lonellm_layers",
+               "-lonellm_gemm", "-lonellm_launchers", "-lonellm_hip", "-Wl,-rpath,$ORIGIN/../../onellm_amd"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for the decoder driver:\n" + r.stderr[-4000:])
     return LIB_HIP, LIB_LAUNCH, LIB_GEMM, LIB_LAYERS
 
 

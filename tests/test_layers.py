@@ -253,3 +253,34 @@ def test_decoder_without_attention_bias_and_reference_rope_position(H, ref):
         np.testing.assert_allclose(g_kc.cpu().numpy(), r_kc, **STEP_TOL[dtype])
     finally:
         dec.close()
+
+
+@pytest.mark.gpu
+def test_standalone_cpp_driver_matches_the_oracle(ref):
+    """tests/cpp/self_decoder_driver.cpp is a C++ program written against onellm/layers.h with the shapes and constants
+    of examples/cpp/decoder/self_decoder_example.cpp; it runs in its own process (system HIP runtime and hipBLASLt, no
+    PyTorch) and prints its results."""
+    announce("stand-alone C++ decoder driver")
+    exe = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver")
+    assert os.path.exists(exe), "build it with `python -m onellm_amd.build`"
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert run.returncode == 0, run.stdout[-2000:] + run.stderr[-2000:]
+    rows = {}
+    for line in run.stdout.splitlines():
+        name, *vals = line.split()
+        rows.setdefault(name, []).append(np.array([float(v) for v in vals], np.float32))
+
+    B, Hq, Hkv, D, I, L, S, t = 2, 4, 2, 8, 12, 2, 12, 3
+    hidden, f = Hq * D, np.float32
+    layer = {"attn_norm": np.ones(hidden, f), "ffn_norm": np.ones(hidden, f), "wqkv": np.ones((hidden, (Hq + 2 * Hkv) * D), f),
+             "bqkv": np.full((Hq + 2 * Hkv) * D, 2, f), "wo": np.ones((hidden, hidden), f), "bo": np.full(hidden, 2, f),
+             "wgate": np.full((hidden, I), 2, f), "wup": np.ones((hidden, I), f), "wdown": np.full((I, hidden), 2, f),
+             "bdown": np.zeros(hidden, f)}
+    x = np.ones((B, hidden), f)
+    kc, vc = np.ones((L, B, Hkv, S, D), f), np.ones((L, B, Hkv, S, D), f)
+    want = ref.self_decoder_step(x, [layer] * L, np.full(hidden, 2, f), kc, vc, Hq, t, 128, 10000.0, 1e-16)
+    np.testing.assert_allclose(rows["decoder_output"][0], want.reshape(-1), rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(rows["residual"][0], x.reshape(-1), rtol=1e-4)
+    for l in range(L):
+        np.testing.assert_allclose(rows["k_row"][l], kc[l, 0, 0, t - 1], rtol=1e-4, atol=1e-4)
+        np.testing.assert_allclose(rows["v_row"][l], vc[l, 0, 0, t - 1], rtol=1e-4, atol=1e-4)
