@@ -5,6 +5,7 @@
 #include <exception>
 #include <string>
 #include "onellm/kernels.h"
+#include "onellm/tensor_map.h"
 
 namespace {
 std::string g_last_error;
@@ -176,6 +177,47 @@ int h_type_tags()
     return (getTensorType<float>() == FP32) + 2 * (getTensorType<half>() == FP16) + 4 * (getTensorType<int>() == INT32)
            + 8 * (getTensorType<const float>() == FP32) + 16 * (getWeightType<half>() == WeightType::FP16_W)
            + 32 * (getBitNum(WeightType::INT8_W) == 8);
+}
+
+// TensorMap as the layers use it (src/utils/tensor.h:160-296): returns a bit per check that holds
+int h_tensor_map_checks()
+{
+    int v = 5, w = 9;
+    Tensor good(CPU, INT32, {1}, &v), other(CPU, INT32, {1}, &w), no_data(CPU, INT32, {1}), no_shape(CPU, INT32, {}, &v);
+    TensorMap m{{"step", good}, {"dropped_a", no_data}, {"dropped_b", no_shape}};
+    int ok = 0;
+    ok |= (m.size() == 1) << 0;                                  // tensors without data or shape are not inserted
+    ok |= (m.isExist("step") && !m.isExist("dropped_a")) << 1;
+    ok |= (m["step"].getVal<int>() == 5 && m.getVal<int>("step") == 5) << 2;
+    m.insert("other", other);
+    m["step"] = other;                                           // entries are assignable views
+    ok |= (m.size() == 2 && m.at("step").getVal<int>() == 9 && m.getPtr<int>("other") == &w) << 3;
+    const int threw = guarded([&] { (void)m["missing"]; });
+    ok |= (threw == 1 && g_last_error.find("missing") != std::string::npos && g_last_error.find("other") != std::string::npos) << 4;
+    ok |= (m.keys().size() == 2) << 5;
+    return ok;
+}
+
+// LlamaLayerWeight records the shapes of src/weights/llama/layer_weights.cc:21-41 and only views the pointers
+int h_layer_weight_checks(int head_num, int kv_head_num, int head_size, int inter_size, int attn_bias)
+{
+    LlamaLayerWeight lw(head_num, kv_head_num, head_size, inter_size, WeightType::FP16_W, attn_bias != 0);
+    const int hidden = head_num * head_size;
+    float buf[10];
+    lw.loadWeights<float>(buf + 0, buf + 1, buf + 2, buf + 3, buf + 4, buf + 5, buf + 6, buf + 7, buf + 8, buf + 9);
+    int ok = 0;
+    ok |= (lw.self_attn_weight.qkv.shape == std::vector<int>{hidden, (head_num + 2 * kv_head_num) * head_size}) << 0;
+    ok |= (lw.self_attn_weight.output.shape == std::vector<int>{hidden, hidden}) << 1;
+    ok |= (lw.ffn_weight.gate.shape == std::vector<int>{hidden, inter_size} && lw.ffn_weight.up.shape == lw.ffn_weight.gate.shape) << 2;
+    ok |= (lw.ffn_weight.down.shape == std::vector<int>{inter_size, hidden}) << 3;
+    ok |= (lw.attn_norm_weight.gamma == buf + 0 && lw.ffn_norm_weight.gamma == buf + 1 && lw.self_attn_weight.qkv.data == buf + 2
+           && lw.self_attn_weight.output.data == buf + 4 && lw.ffn_weight.down.data == buf + 6 && lw.ffn_weight.down.bias == buf + 7
+           && lw.ffn_weight.gate.data == buf + 8 && lw.ffn_weight.up.data == buf + 9) << 4;
+    const bool biases = lw.self_attn_weight.qkv.bias == buf + 3 && lw.self_attn_weight.output.bias == buf + 5;
+    const bool none = lw.self_attn_weight.qkv.bias == nullptr && lw.self_attn_weight.output.bias == nullptr;
+    ok |= (attn_bias ? biases : none) << 5;
+    ok |= (lw.self_attn_weight.qkv.type == WeightType::FP16_W && lw.ffn_weight.down.type == WeightType::FP16_W) << 6;
+    return ok;
 }
 
 }  // extern "C"

@@ -43,6 +43,13 @@ def test_carrier_types(H):
     assert b"[oneLLM][ERROR]" in H.h_last_error()
 
 
+def test_tensor_map_and_layer_weight_views(H):
+    assert H.h_tensor_map_checks() == 63
+    assert b"missing" in H.h_last_error()
+    assert H.h_layer_weight_checks(4, 2, 8, 12, 1) == 127
+    assert H.h_layer_weight_checks(32, 8, 128, 11008, 0) == 127
+
+
 def test_precondition_failures_throw_without_touching_the_gpu(H):
     fake = ctypes.c_void_p(0x1000)
     # step tensor on the GPU: the launcher must refuse to dereference it on the host
