@@ -252,3 +252,53 @@ def test_constant_value_rows_at_full_size(capi, dev):
     out = torch.zeros(B, H * D, dtype=torch.float16, device=dev)
     capi.decode_attn(qkv, None, kc, vc, out, H, t, D, 10000.0)
     assert (out.float() - 0.375).abs().max().item() <= 1e-3
+
+
+def test_options_on_the_matrix_core_kernel(capi, ref, dev):
+    """The same option matrix as test_options on a shape that takes the MFMA grouped-query kernel (fp16, D = 128,
+    4 query heads per kv head), with one and with several sequence splits."""
+    announce("attn options, mfma kernel")
+    qkv, bias, kc, vc = _case(np.float16, 2, 8, 2, 128, 200, 2, seed=23, std=0.5)
+    for nsplit in (-1, 3):
+        capi.tune_set("attn_nsplit", nsplit)
+        try:
+            _assert_parity(_run_both(capi, ref, dev, qkv, None, kc, vc, 8, 177, 128, layer=1), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 0), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 64), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 128, pos_offset=-1, layer=1), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 128, base=500000.0), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 128, flags=capi.ATTN_NO_V_BIAS), np.float16)
+            res = _run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 128, flags=capi.ATTN_NO_CACHE_WRITE)
+            _assert_parity(res, np.float16)
+            np.testing.assert_array_equal(_bits(res[2]), _bits(kc))
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 200, 128), np.float16)       # t == S
+        finally:
+            capi.tune_set("attn_nsplit", -1)
+
+
+def test_random_shapes_sweep(capi, ref, dev):
+    """Forty seeded random (dtype, heads, group size, head size, lengths, split count) combinations, ragged lengths
+    included: every kernel variant and padded head tile gets shapes nobody picked by hand."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        dtype = [np.float16, np.float32][int(rng.integers(0, 2))]
+        D = int(rng.choice([16, 32, 64, 128, 128, 128, 256]))
+        Hkv = int(rng.integers(1, 4))
+        G = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 20]))
+        if D >= 256:
+            G = min(G, 4)
+        Hq = Hkv * G
+        B = int(rng.integers(1, 5))
+        S = int(rng.integers(8, 420))
+        lens = rng.integers(1, S + 1, size=B)
+        ragged = bool(rng.integers(0, 2))
+        t = lens if ragged else int(lens.max())
+        nsplit = int(rng.choice([-1, -1, 1, 2, 3, 7]))
+        rot = int(rng.choice([D, D, D // 2, 0]))
+        announce("attn sweep", case, dtype.__name__, "B", B, "Hq", Hq, "Hkv", Hkv, "D", D, "S", S, "t", t, "nsplit", nsplit, "rot", rot)
+        qkv, bias, kc, vc = _case(dtype, B, Hq, Hkv, D, S, 1, seed=5000 + case, std=0.5)
+        capi.tune_set("attn_nsplit", nsplit)
+        try:
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, rot), dtype)
+        finally:
+            capi.tune_set("attn_nsplit", -1)
