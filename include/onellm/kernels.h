@@ -2,9 +2,16 @@
 // unit tests call.  Each is a thin shim over the C ABI in onellm_hip.h: it unpacks shapes the
 // way the reference launcher does and throws std::runtime_error on a non-zero return code.
 #pragma once
+#include <hip/hip_runtime_api.h>
 #include "onellm/tensor.h"
 #include "onellm/weights.h"
 #include "onellm/params.h"
+
+// Stream the launch* functions below queue on, per calling thread; the default is the null stream, which is where
+// the reference launches everything.  No counterpart in the reference: it is for callers that own a stream, for
+// example to capture a decode step into a HIP graph (the null stream cannot be captured).
+void onellmSetLaunchStream(hipStream_t stream);
+hipStream_t onellmGetLaunchStream();
 
 // src/kernels/decoder_masked_attn.h:7-14
 void launchDecoderMaskedMHA(Tensor* qkv_buf,

@@ -14,7 +14,7 @@
 //     x <- x + y + bo ; y <- RMSNorm(x, ffn_norm[l])               (launchFusedAddBiasResidualRMSNorm)
 //     y <- (silu(y . Wgate) * (y . Wup)) . Wdown
 //     x <- x + y + bdown ; y <- RMSNorm(x, attn_norm[l+1] or output_norm_weight)
-// Element type (FP32 or FP16) follows "decoder_input".  Everything is queued on the null stream, like the launchers;
+// Element type (FP32 or FP16) follows "decoder_input".  Everything is queued on one stream (see below);
 // forward() returns without synchronising.
 //
 // Where this differs from the reference snapshot, on purpose (the snapshot cannot produce a decoder output):
@@ -36,8 +36,11 @@
 #include "onellm/tensor_map.h"
 #include "onellm/weights.h"
 
-class cublasWrapper;   // carried for signature compatibility only; may be null, never dereferenced.  The same holds
-                       // for the `stream` arguments: like the launchers, the layers queue on the null stream.
+class cublasWrapper;   // carried for signature compatibility only; may be null, never dereferenced
+// `stream` arguments: the attention and FFN layers queue where the launch* functions do (onellmSetLaunchStream, the
+// null stream by default, as in the reference).  A LlamaSelfDecoder constructed with a non-null stream queues its
+// whole step there, which is what makes a step capturable into a HIP graph: run one step first (buffers, the
+// attention workspace and the GEMM plans are created on first use), then capture.
 
 // output[M, N] = input[M, K] . weight, weight.shape = {K, N} (or {N, K} with trans_b); M = input->shape[0], K = the
 // product of the remaining input dimensions.  shared_out_buf: write the second [M, N] half of a [2, M, N] output.
@@ -115,6 +118,7 @@ private:
     int   num_layer;
     int   hidden_units;
     float rmsnorm_eps;
+    hipStream_t stream;
     LLaMASelfAttentionLayer* selfAttn;
     LLaMAFFNLayer*           ffn;
 };

@@ -22,16 +22,18 @@ int onellm_layers_linear(int dtype, void* x, void* w, void* y, int M, int K, int
 /* A LlamaSelfDecoder (src/layers/decoder/self_decoder.h:10-74) with its layer weights and an allocator.
  * The ten `void**` are host arrays of L device pointers, in the order of LlamaLayerWeight::loadWeights
  * (src/weights/llama/layer_weights.h:32-41); with attn_bias == 0 the qkv / output biases are ignored; bdown[l] may be
- * NULL.  Weights are [in, out] row-major.  The weight buffers must outlive the decoder.  Returns NULL on failure. */
+ * NULL.  Weights are [in, out] row-major.  The weight buffers must outlive the decoder.  stream: where every step of
+ * this decoder is queued (NULL = the null stream).  Returns NULL on failure. */
 void* onellm_decoder_create(int dtype, int B, int Hq, int Hkv, int D, int inter_size, int L, int S, int rotary_dim,
                             float rope_base, float rmsnorm_eps, int attn_bias, void** attn_norm, void** ffn_norm,
                             void** wqkv, void** bqkv, void** wo, void** bo, void** wdown, void** bdown, void** wgate,
-                            void** wup, void* output_norm);
+                            void** wup, void* output_norm, onellm_stream_t stream);
 
 /* LlamaSelfDecoder::forward for one step: decoder_input [B, Hq*D] is the residual stream (updated), decoder_output
  * [B, Hq*D] receives the final normalised activations, the caches are [L, B, Hkv, S, D] and get row step-1 of every
- * layer.  step = attended positions including the new token, the same for the whole batch.  Queued on the null
- * stream; returns without synchronising. */
+ * layer.  step = attended positions including the new token, the same for the whole batch.  Queued on the
+ * decoder's stream; returns without synchronising.  After one ordinary step (which creates buffers and GEMM plans)
+ * further steps allocate nothing and may be captured into a HIP graph on that stream. */
 int onellm_decoder_forward(void* decoder, int step, void* decoder_input, void* decoder_output, void* k_cache, void* v_cache);
 
 void onellm_decoder_destroy(void* decoder);

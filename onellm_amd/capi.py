@@ -266,7 +266,7 @@ def layers_lib():
         L.onellm_layers_last_error.restype = ctypes.c_char_p
         L.onellm_layers_linear.argtypes = [_ci, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci]
         L.onellm_decoder_create.restype = _vp
-        L.onellm_decoder_create.argtypes = [_ci] * 9 + [_cf, _cf, _ci] + [pp] * 10 + [_vp]
+        L.onellm_decoder_create.argtypes = [_ci] * 9 + [_cf, _cf, _ci] + [pp] * 10 + [_vp, _vp]
         L.onellm_decoder_forward.argtypes = [_vp, _ci, _vp, _vp, _vp, _vp]
         L.onellm_decoder_destroy.argtypes = [_vp]
         _layers = L
@@ -275,11 +275,13 @@ def layers_lib():
 
 class SelfDecoder:
     """LlamaSelfDecoder over device tensors.  `layers`: list of dicts of torch device tensors with the keys attn_norm,
-    ffn_norm, wqkv, bqkv, wo, bo, wdown, bdown, wgate, wup (weights [in, out]; a bias may be None)."""
+    ffn_norm, wqkv, bqkv, wo, bo, wdown, bdown, wgate, wup (weights [in, out]; a bias may be None).  `stream`: raw
+    stream handle every step is queued on (None = the null stream)."""
 
     ORDER = ["attn_norm", "ffn_norm", "wqkv", "bqkv", "wo", "bo", "wdown", "bdown", "wgate", "wup"]
 
-    def __init__(self, dtype_code, B, Hq, Hkv, D, inter_size, S, rotary_dim, rope_base, eps, layers, output_norm, attn_bias=True):
+    def __init__(self, dtype_code, B, Hq, Hkv, D, inter_size, S, rotary_dim, rope_base, eps, layers, output_norm, attn_bias=True,
+                 stream=None):
         self.L = layers_lib()
         self._keep = (layers, output_norm)
         n = len(layers)
@@ -290,7 +292,7 @@ class SelfDecoder:
                 arr[l] = None if w[name] is None else _ptr(w[name])
             arrays.append(arr)
         self.handle = self.L.onellm_decoder_create(dtype_code, B, Hq, Hkv, D, inter_size, n, S, rotary_dim, rope_base, eps,
-                                                   int(attn_bias), *arrays, _ptr(output_norm))
+                                                   int(attn_bias), *arrays, _ptr(output_norm), stream)
         if not self.handle:
             raise RuntimeError(self.L.onellm_layers_last_error().decode())
 

@@ -1,6 +1,7 @@
 // The six launch* functions of oneLLM's decode path, with oneLLM's own signatures, as shims over
 // the C ABI.  Each unpacks shapes the way the reference launcher does (cited per function), calls
-// the C entry point on the null stream (the reference launches everything there) and throws
+// the C entry point on the null stream (the reference launches everything there; onellmSetLaunchStream names
+// another one for the calling thread) and throws
 // std::runtime_error when the entry point reports an error.  No printing, no device sync.
 #include <mutex>
 #include <stdexcept>
@@ -8,6 +9,14 @@
 #include <hip/hip_runtime_api.h>
 #include "onellm/kernels.h"
 #include "onellm_hip.h"
+
+namespace {
+thread_local hipStream_t t_launch_stream = nullptr;
+void* launch_stream() { return t_launch_stream; }
+}  // namespace
+
+void onellmSetLaunchStream(hipStream_t stream) { t_launch_stream = stream; }
+hipStream_t onellmGetLaunchStream() { return t_launch_stream; }
 
 namespace {
 
@@ -105,7 +114,7 @@ void launchDecoderMaskedMHA(Tensor* qkv_buf, BaseWeight& qkv, Tensor* k_cache, T
                                   batch_size, head_num, kv_head_num, head_size, cs.S, /*layer=*/0, cs.layers,
                                   cur_step, nullptr, cur_step,
                                   static_params.rotary_embedding_dim, static_params.rotary_embedding_base,
-                                  rope_pos_offset, /*flags=*/0u, ws, ws_bytes, nullptr);
+                                  rope_pos_offset, /*flags=*/0u, ws, ws_bytes, launch_stream());
     };
     int rc = call(nullptr, 0);
     if (rc == ONELLM_EWORKSPACE) {
@@ -123,7 +132,7 @@ void launchRMSNorm(Tensor* decoder_out, LayerNormWeight& attn_norm_weight, float
     const int num_tokens = decoder_out->shape[0];      // :90
     const int hidden_units = decoder_out->shape[1];    // :91
     const int rc = onellm_rmsnorm(abi_dtype(decoder_out, "launchRMSNorm"), decoder_out->data, attn_norm_weight.gamma,
-                                  eps, num_tokens, hidden_units, nullptr);
+                                  eps, num_tokens, hidden_units, launch_stream());
     throw_on_error(rc, "launchRMSNorm");
 }
 
@@ -134,7 +143,7 @@ void launchFusedAddBiasResidualRMSNorm(T* residual, T* decoder_out, const T* bia
 {
     const int dtype = std::is_same<T, half>::value ? ONELLM_FP16 : ONELLM_FP32;
     const int rc = onellm_fused_add_bias_residual_rmsnorm(dtype, residual, decoder_out, bias, scale, eps, num_tokens,
-                                                          hidden_units, nullptr);
+                                                          hidden_units, launch_stream());
     throw_on_error(rc, "launchFusedAddBiasResidualRMSNorm");
 }
 template void launchFusedAddBiasResidualRMSNorm(float*, float*, const float*, const float*, float, int, int);
@@ -155,7 +164,7 @@ void launchAppendKVCache(Tensor* k_src, Tensor* v_src, Tensor* layer_id, Tensor*
     const int rc = onellm_kv_append(abi_dtype(k_src, "launchAppendKVCache"), k_src->data, v_src->data, k_dst->data,
                                     v_dst->data, (const int*)cur_query_length->data, (const int*)history_length->data,
                                     batch_size, kv_head_num, max_q_len, cs.S, head_size, host_layer_id(layer_id),
-                                    cs.layers, nullptr);
+                                    cs.layers, launch_stream());
     throw_on_error(rc, "launchAppendKVCache");
 }
 
@@ -174,7 +183,7 @@ void launchTransposeKVCache(Tensor* k_cache_src, Tensor* v_cache_src, Tensor* co
     const int rc = onellm_kv_repeat(abi_dtype(k_cache_src, "launchTransposeKVCache"), k_cache_src->data,
                                     v_cache_src->data, k_cache_dst->data, v_cache_dst->data,
                                     (const int*)context_length->data, batch_size, head_num, cs.Hkv, cs.S, max_k_len,
-                                    head_size, host_layer_id(layer_id), cs.layers, nullptr);
+                                    head_size, host_layer_id(layer_id), cs.layers, launch_stream());
     throw_on_error(rc, "launchTransposeKVCache");
 }
 
@@ -183,7 +192,7 @@ void launchTransposeKVCache(Tensor* k_cache_src, Tensor* v_cache_src, Tensor* co
 void launchTopKforBeamSearch(const float* probs, const int batch_size, const int vocab_size, float* topk_workspace)
 {
     constexpr int beamwidth = 2;
-    const int rc = onellm_beam_topk(probs, batch_size, beamwidth, vocab_size, beamwidth, topk_workspace, nullptr);
+    const int rc = onellm_beam_topk(probs, batch_size, beamwidth, vocab_size, beamwidth, topk_workspace, launch_stream());
     throw_on_error(rc, "launchTopKforBeamSearch");
 }
 
@@ -206,7 +215,7 @@ void launchAddFusedQKVBiasTransposeAndRoPE(Tensor* q_buf, Tensor* k_buf, Tensor*
                                                   k_buf->data, v_buf->data, QKV->data, qkv.bias,
                                                   (const int*)padding_offset->data, (const int*)history_length->data,
                                                   batch_size, seq_len, token_num, head_num, kv_head_num, head_size,
-                                                  params.rotary_embedding_dim, params.rotary_embedding_base, nullptr);
+                                                  params.rotary_embedding_dim, params.rotary_embedding_base, launch_stream());
     throw_on_error(rc, "launchAddFusedQKVBiasTransposeAndRoPE");
 }
 
@@ -215,7 +224,7 @@ template <typename T>
 void launchAct(const T* input, T* out, const int batch_size, const int intermedia_size)
 {
     const int dtype = std::is_same<T, half>::value ? ONELLM_FP16 : ONELLM_FP32;
-    throw_on_error(onellm_silu_and_mul(dtype, input, out, batch_size, intermedia_size, nullptr), "launchAct");
+    throw_on_error(onellm_silu_and_mul(dtype, input, out, batch_size, intermedia_size, launch_stream()), "launchAct");
 }
 template void launchAct(const float*, float*, const int, const int);
 template void launchAct(const half*, half*, const int, const int);
@@ -232,6 +241,6 @@ void launchSampling(Tensor* topk_id, Tensor* topk_val, Tensor* seqlen, Tensor* i
     const int rc = onellm_topk_sample((const int*)topk_id->data, (const float*)topk_val->data, (int*)output_id->data,
                                       (int*)seqlen->data, (unsigned char*)is_finished->data, batch_size, K,
                                       (unsigned long long)(unsigned)params["step"], params["end_id"], params["vocab_size"],
-                                      nullptr);
+                                      launch_stream());
     throw_on_error(rc, "launchSampling");
 }

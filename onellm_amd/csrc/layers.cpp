@@ -62,7 +62,7 @@ void tune_once(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* ws, s
         std::lock_guard<std::mutex> g(g_tuned_mu);
         if (!g_autotune || !g_tuned.insert(std::make_tuple(dtype, M, K, N, ldy, w_is_nk)).second) return;
     }
-    (void)onellm_linear_tune(dtype, M, K, N, ldy, w_is_nk, ws, ws_bytes, nullptr, nullptr, nullptr);   // best effort
+    (void)onellm_linear_tune(dtype, M, K, N, ldy, w_is_nk, ws, ws_bytes, onellmGetLaunchStream(), nullptr, nullptr);   // best effort
 }
 
 Tensor* new_buffer(BaseAllocator* a, DataType t, std::vector<int> shape)
@@ -119,7 +119,7 @@ void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool tr
     const int dtype_code = input->dtype == FP32 ? ONELLM_FP32 : ONELLM_FP16;
     tune_once(dtype_code, M, K, N, ldy, trans_b ? 1 : 0, ws, g_gemm_ws.bytes);
     const int rc = onellm_linear(input->dtype == FP32 ? ONELLM_FP32 : ONELLM_FP16, input->data, weight.data, y, M, K, N, ldy,
-                                 trans_b ? 1 : 0, ws, g_gemm_ws.bytes, nullptr);
+                                 trans_b ? 1 : 0, ws, g_gemm_ws.bytes, onellmGetLaunchStream());
     if (rc != 0) throw std::runtime_error(std::string("[TM][ERROR] launchLinearGemm: ") + onellm_error_string(rc) + " \n");
 }
 
@@ -244,7 +244,7 @@ void LLaMAFFNLayer::forward(TensorMap& inputs, TensorMap& outputs, LLaMAFFNWeigh
 LlamaSelfDecoder::LlamaSelfDecoder(int head_num, int kv_head_num, int head_size, int inter_size, int num_layer,
                                    const LLaMAAttentionStaticParams& attn_params, float rmsnorm_eps, hipStream_t stream,
                                    cublasWrapper* cublas_wrapper, BaseAllocator* allocator, bool is_free_buffer_after_forward):
-    num_layer(num_layer), hidden_units(head_num * head_size), rmsnorm_eps(rmsnorm_eps),
+    num_layer(num_layer), hidden_units(head_num * head_size), rmsnorm_eps(rmsnorm_eps), stream(stream),
     selfAttn(new LLaMASelfAttentionLayer(head_num, kv_head_num, head_size, attn_params, stream, cublas_wrapper, allocator,
                                          is_free_buffer_after_forward)),
     ffn(new LLaMAFFNLayer(head_num, head_size, inter_size, stream, cublas_wrapper, allocator, is_free_buffer_after_forward))
@@ -276,13 +276,20 @@ void LlamaSelfDecoder::forward(TensorMap& input_tensors, const std::vector<Llama
                                TensorMap& output_tensors, LLaMAAttentionDynParams& dyn_params)
 {
     require((int)layerWeights.size() >= num_layer, "fewer layer weights than layers");
+    // a decoder constructed with a stream queues this step there; otherwise wherever the calling thread's launches go
+    struct StreamScope {
+        hipStream_t saved;
+        bool active;
+        StreamScope(hipStream_t s): saved(onellmGetLaunchStream()), active(s != nullptr) { if (active) onellmSetLaunchStream(s); }
+        ~StreamScope() { if (active) onellmSetLaunchStream(saved); }
+    } scope(stream);
     Tensor x = input_tensors["decoder_input"];      // residual stream
     Tensor y = output_tensors["decoder_output"];    // normalised activations / sub-layer results
     require(x.dtype == y.dtype && x.size() == y.size() && x.data != y.data, "decoder_input and decoder_output must be two buffers of one shape");
     const int rows = rows_of(&x);
     require(cols_of(&x) == hidden_units, "decoder_input is not [rows, head_num * head_size]");
 
-    hip_ok(hipMemcpyAsync(y.data, x.data, (size_t)x.size() * elt_bytes(x.dtype), hipMemcpyDeviceToDevice, nullptr), "decoder copy");
+    hip_ok(hipMemcpyAsync(y.data, x.data, (size_t)x.size() * elt_bytes(x.dtype), hipMemcpyDeviceToDevice, onellmGetLaunchStream()), "decoder copy");
     launchRMSNorm(&y, layerWeights[0]->attn_norm_weight, rmsnorm_eps);
 
     int layer_id = 0;

@@ -59,7 +59,8 @@ int onellm_layers_linear(int dtype, void* x, void* w, void* y, int M, int K, int
 // per-layer pointer arrays of length L, in the argument order of LlamaLayerWeight::loadWeights
 void* onellm_decoder_create(int dtype, int B, int Hq, int Hkv, int D, int I, int L, int S, int rotary_dim, float rope_base,
                         float eps, int attn_bias, void** attn_norm, void** ffn_norm, void** wqkv, void** bqkv, void** wo,
-                        void** bo, void** wdown, void** bdown, void** wgate, void** wup, void* output_norm)
+                        void** bo, void** wdown, void** bdown, void** wgate, void** wup, void* output_norm,
+                        onellm_stream_t stream)
 {
     Decoder* d = nullptr;
     const int rc = guarded([&] {
@@ -76,7 +77,7 @@ void* onellm_decoder_create(int dtype, int B, int Hq, int Hkv, int D, int I, int
         sp.rotary_embedding_base = rope_base;
         sp.max_position_embeddings = 2048;
         sp.use_dynamic_ntk = false;
-        d->decoder.reset(new LlamaSelfDecoder(Hq, Hkv, D, I, L, sp, eps, nullptr, nullptr, &d->allocator,
+        d->decoder.reset(new LlamaSelfDecoder(Hq, Hkv, D, I, L, sp, eps, static_cast<hipStream_t>(stream), nullptr, &d->allocator,
                                               /*is_free_buffer_after_forward=*/false));
     });
     if (rc != 0) {

@@ -150,6 +150,9 @@ int h_sampling(void* topk_id, void* topk_val, void* seqlen, void* finished, void
 }
 
 // the callers' pattern after every launch (src/layers/attention/masked_self_attention.cpp:73 in oneLLM)
+// onellmSetLaunchStream for the calling thread (NULL restores the null stream)
+void h_set_launch_stream(void* stream) { onellmSetLaunchStream(static_cast<hipStream_t>(stream)); }
+
 int h_sync_and_check()
 {
     return guarded([] { DeviceSyncAndCheckCudaError(); });

@@ -31,6 +31,8 @@ def H():
     L.h_prefill_rope.argtypes = [ci, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, cf]
     L.h_act.argtypes = [ci, vp, vp, ci, ci]
     L.h_sampling.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
+    L.h_set_launch_stream.argtypes = [vp]
+    L.h_set_launch_stream.restype = None
     return L
 
 
@@ -219,3 +221,87 @@ def test_launchSampling(H, ref, dev):
     np.testing.assert_array_equal(out.cpu().numpy(), want)
     np.testing.assert_array_equal(d[2].cpu().numpy(), seqlen)
     np.testing.assert_array_equal(d[3].cpu().numpy(), fin)
+
+
+@pytest.mark.gpu
+def test_every_launcher_queues_on_the_launch_stream(H, dev):
+    """onellmSetLaunchStream names the stream of the calling thread's launches.  All nine launchers are captured into
+    one HIP graph on a side stream (a launch that went to the null stream instead would be refused during capture or be
+    missing from the graph); the replay must reproduce what the same calls produce eagerly, bit for bit."""
+    import torch
+    announce("launchers under graph capture on a side stream")
+    torch.manual_seed(3)
+    B, Hq, Hkv, D, S, t, H_, I, V, K = 2, 8, 2, 128, 96, 70, 1024, 512, 4000, 4
+    G = Hq // Hkv
+    h = lambda *s: torch.randn(*s, device=dev).mul(0.5).half()
+    qkv, bias = h(B, Hq + 2 * Hkv, D), h((Hq + 2 * Hkv) * D)
+    kc0, vc0 = h(1, B, Hkv, S, D), h(1, B, Hkv, S, D)
+    x0, res0, gam, nb = h(B, H_), h(B, H_), torch.rand(H_, device=dev).add(0.5).half(), h(H_)
+    ks, vs = h(B, Hkv, 1, D), h(B, Hkv, 1, D)
+    cur = torch.ones(B, dtype=torch.int32, device=dev)
+    hist = torch.full((B,), t, dtype=torch.int32, device=dev)
+    ctx = torch.full((B,), t + 1, dtype=torch.int32, device=dev)
+    pair = h(B, 2, I)
+    logits = torch.randn(B * 2, V, device=dev)
+    pq, pk, pv = (torch.zeros(B, n, 4, D, dtype=torch.float16, device=dev) for n in (Hq, Hkv, Hkv))
+    pqkv = h(B * 4, Hq + 2 * Hkv, D)
+    pad = torch.zeros(B * 4, dtype=torch.int32, device=dev)
+    zeros_b = torch.zeros(B, dtype=torch.int32, device=dev)
+    four_b = torch.full((B,), 4, dtype=torch.int32, device=dev)
+    tid = torch.randint(0, V, (B, K), dtype=torch.int32, device=dev)
+    tval = torch.rand(B, K, device=dev)
+
+    kc, vc, x, res = kc0.clone(), vc0.clone(), x0.clone(), res0.clone()
+    out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+    rk, rv = (torch.zeros(B, Hq, S, D, dtype=torch.float16, device=dev) for _ in range(2))
+    act = torch.zeros(B, I, dtype=torch.float16, device=dev)
+    tws = torch.zeros((2 * B * 2 * 8 * 2 + 2 * B * 2), dtype=torch.float32, device=dev)
+    seqlen, fin, sampled = zeros_b.clone(), torch.zeros(B, dtype=torch.uint8, device=dev), zeros_b.clone()
+    state = (kc, vc, x, res, out, rk, rv, act, tws, pq, pk, pv, seqlen, fin, sampled)
+
+    def restore():
+        kc.copy_(kc0); vc.copy_(vc0); x.copy_(x0); res.copy_(res0)
+        for a in (out, rk, rv, act, tws, pq, pk, pv, seqlen, fin, sampled):
+            a.zero_()
+
+    def calls():
+        p = lambda a: a.data_ptr()
+        ok = [H.h_rmsnorm(1, p(x), p(gam), B, H_, 1e-5),
+              H.h_decode_mha(1, p(qkv), p(bias), p(kc), p(vc), p(out), B, Hq, Hkv, D, S, 1, t, 0, D, 10000.0),
+              H.h_fused_norm(1, p(res), p(x), p(nb), p(gam), B, H_, 1e-5),
+              H.h_append(1, p(ks), p(vs), p(kc), p(vc), p(cur), p(hist), B, Hkv, 1, S, D, 1, 0),
+              H.h_repeat(1, p(kc), p(vc), p(rk), p(rv), p(ctx), B, Hq, Hkv, S, S, D, 1, 0),
+              H.h_act(1, p(pair), p(act), B, I),
+              H.h_topk(p(logits), B, V, p(tws)),
+              H.h_prefill_rope(1, p(pq), p(pk), p(pv), p(pqkv), p(bias), p(pad), p(zeros_b), p(four_b), B, 4, B * 4, Hq, Hkv, D, D, 10000.0),
+              H.h_sampling(p(tid), p(tval), p(seqlen), p(fin), p(sampled), B, K, 5, 10, V)]
+        assert ok == [0] * 9, ok
+
+    restore()
+    calls()                                      # eager, null stream
+    torch.cuda.synchronize()
+    want = [a.clone() for a in state]
+
+    side = torch.cuda.Stream()
+    H.h_set_launch_stream(side.cuda_stream)
+    try:
+        restore()
+        torch.cuda.synchronize()
+        calls()                                  # eager on the side stream (also creates the attention workspace if needed)
+        torch.cuda.synchronize()
+        for a, b in zip(state, want):
+            assert torch.equal(a, b)
+        restore()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            calls()
+        for replay in range(3):
+            restore()
+            x0.float().sum().item()
+            g.replay()
+            torch.cuda.synchronize()
+            for i, (a, b) in enumerate(zip(state, want)):
+                assert torch.equal(a, b), f"replay {replay}: buffer {i} differs from the eager result"
+    finally:
+        H.h_set_launch_stream(None)

@@ -284,3 +284,60 @@ def test_standalone_cpp_driver_matches_the_oracle(ref):
     for l in range(L):
         np.testing.assert_allclose(rows["k_row"][l], kc[l, 0, 0, t - 1], rtol=1e-4, atol=1e-4)
         np.testing.assert_allclose(rows["v_row"][l], vc[l, 0, 0, t - 1], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
+def test_decoder_step_captured_into_a_graph_replays_identically(H, ref):
+    """A decoder built on a side stream: after one ordinary step (buffers, attention workspace and GEMM plans exist)
+    a step is captured into a HIP graph and replayed with eager work and synchronisations in between; every replay
+    must reproduce the eager step bit for bit (output, residual stream and caches)."""
+    import torch
+    from onellm_amd import capi
+    announce("decoder step under graph capture")
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(77)
+    dtype, B, Hq, Hkv, D, I, L, S, t = np.float16, 4, 16, 4, 128, 1536, 2, 600, 577
+    hidden = Hq * D
+    layers = _random_layers(rng, dtype, Hq, Hkv, D, I, L)
+    out_norm = rng.uniform(0.5, 1.5, hidden).astype(dtype)
+    x0 = _dev(torch, rng.standard_normal((B, hidden)).astype(dtype))
+    kc0 = _dev(torch, (rng.standard_normal((L, B, Hkv, S, D)) * 0.5).astype(dtype))
+    vc0 = _dev(torch, (rng.standard_normal((L, B, Hkv, S, D)) * 0.5).astype(dtype))
+    side = torch.cuda.Stream()
+    dl = [{k: (None if v is None else _dev(torch, v)) for k, v in w.items()} for w in layers]
+    dec = capi.SelfDecoder(capi.FP16, B, Hq, Hkv, D, I, S, D, 10000.0, 1e-5, dl, _dev(torch, out_norm), stream=side.cuda_stream)
+    x, y, kc, vc = x0.clone(), torch.zeros_like(x0), kc0.clone(), vc0.clone()
+
+    def restore():
+        x.copy_(x0); y.zero_(); kc.copy_(kc0); vc.copy_(vc0)
+
+    def snapshot():
+        torch.cuda.synchronize()
+        return [a.clone() for a in (x, y, kc, vc)]
+
+    try:
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            restore()
+            dec.forward(t, x, y, kc, vc)                   # eager, on the decoder's stream: also the warm-up
+        want = snapshot()
+        # against the oracle too, so that "identical" is not "identically wrong"
+        r_x, r_kc, r_vc = x0.cpu().numpy().copy(), kc0.cpu().numpy().copy(), vc0.cpu().numpy().copy()
+        r_y = ref.self_decoder_step(r_x, layers, out_norm, r_kc, r_vc, Hq, t, D, 10000.0, 1e-5)
+        np.testing.assert_allclose(want[1].cpu().numpy().astype(np.float64), r_y.astype(np.float64), **STEP_TOL[dtype])
+
+        restore()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            dec.forward(t, x, y, kc, vc)
+        for replay in range(4):
+            restore()
+            (x0.float() * 2).sum().item()                  # eager work and a synchronisation between replays
+            g.replay()
+            got = snapshot()
+            for a, b in zip(got, want):
+                assert torch.equal(a, b), f"replay {replay} differs from the eager step"
+    finally:
+        torch.cuda.synchronize()
+        dec.close()
