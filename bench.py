@@ -438,7 +438,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(t),
-                     "kernel": "decode_attn_split_kernel<__half,16,1,4,4>",
+                     "kernel": "decode_attn_split_kernel<__half,16,1,4,4,false>",
                      "algorithmic_bytes_per_launch": nbytes,
                      "note": "duration = HIP-event time per step on the launch stream; at this shape a step is exactly "
                              "one launch of the kernel (single sequence split, no merge pass). traffic = FETCH_SIZE + "

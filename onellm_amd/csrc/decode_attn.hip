@@ -44,6 +44,11 @@ struct AttnArgs {
     unsigned flags;
     float qscale;         // log2(e) / sqrt(D), folded into q
     size_t slab;          // element offset of the layer slab inside the cache
+    // balanced schedule (bal_nwg > 0): the grid is bal_nwg workgroups and each takes an equal,
+    // contiguous share of all work items (an item = item_rows history rows of one unit)
+    int bal_nwg;
+    int item_rows;
+    int gt;               // query heads per tile, for the merge kernel
 };
 
 // What one workgroup works on: a chunk of the history of one (sequence, kv-head) for up to GT query heads.
@@ -53,6 +58,9 @@ struct Unit {
     int split, last;       // this workgroup's split and the sequence's last split
     int r0, r1;            // history rows [r0, r1) of this split
     bool is_last;          // the last split also owns the new token's row
+    bool direct;           // the workgroup sees the whole unit: it writes the output, not a partial state
+    size_t pbase;          // partial-state entry of tile head g: pbase + g * pstride
+    int pstride;
 };
 
 // Workgroups are dealt to the 8 XCDs round-robin in linear block order.  The kv-head index is the
@@ -75,7 +83,181 @@ __device__ __forceinline__ bool locate_unit(const AttnArgs& a, Unit& u)
     u.r0 = u.split * a.chunk;
     u.r1 = min(u.r0 + a.chunk, u.t - 1);
     u.pos = u.t + a.pos_offset;
+    u.direct = a.nsplit == 1;
+    u.pbase = ((size_t)u.b * a.Hq + u.kvh * a.G + u.g0) * a.nsplit + u.split;
+    u.pstride = a.nsplit;
     return true;
+}
+
+// ---- balanced schedule -----------------------------------------------------------------------
+// All work of a step is cut into items of item_rows history rows; a unit (sequence, kv head, head
+// tile) of a sequence with t attended positions has max(1, ceil((t-1)/item_rows)) of them (the
+// last one also carries the new token's row).  Items are numbered sequence-major, then unit, then
+// row order, and workgroup i of N takes items [i*W/N, (i+1)*W/N): every workgroup streams the same
+// number of rows whatever the lengths are, crossing from one unit into the next where its share
+// does.  A unit seen whole by one workgroup is finished by it; otherwise each workgroup that
+// touches it leaves a partial state in entry (workgroup + global unit index) - unique, because
+// along the walk either the workgroup or the unit advances - and the merge kernel, which derives
+// the same boundaries from the same lengths, combines them.
+__device__ __forceinline__ int seq_items(const AttnArgs& a, int t)
+{
+    if (t < 1 || t > a.S) return 0;               // out-of-contract length: no work, nothing touched
+    const int n = (t - 1 + a.item_rows - 1) / a.item_rows;
+    return n < 1 ? 1 : n;
+}
+
+__device__ __forceinline__ long long wave_sum_i64(long long v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// items of all sequences, and of the sequences before `before` (every lane gets both)
+__device__ __forceinline__ void count_items(const AttnArgs& a, int before, long long& total, long long& prefix)
+{
+    if (!a.t_dev) {
+        const int it = seq_items(a, a.t_host);
+        total = (long long)a.B * it;
+        prefix = (long long)before * it;
+        return;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    long long tot = 0, pre = 0;
+    for (int bb = lane; bb < a.B; bb += kWave) {
+        const int it = seq_items(a, a.t_dev[bb]);
+        tot += it;
+        if (bb < before) pre += it;
+    }
+    total = wave_sum_i64(tot);
+    prefix = wave_sum_i64(pre);
+}
+
+// workgroup that owns item x when W items are dealt to N workgroups as [i*W/N, (i+1)*W/N)
+__device__ __forceinline__ int item_owner(long long x, long long W, int N)
+{
+    return (int)(((x + 1) * N - 1) / W);
+}
+
+// workgroups that take part: never more than there are items, so that no share is empty and the
+// workgroups of a unit are consecutive
+__device__ __forceinline__ int balanced_workgroups(const AttnArgs& a, long long W)
+{
+    return W < a.bal_nwg ? (int)W : a.bal_nwg;
+}
+
+struct Walk {
+    long long cur, hi;     // next item of this workgroup, end of its share
+    long long base;        // first item of sequence b
+    int b, items;          // current sequence and its items per unit
+    int nunits;            // units per sequence
+};
+
+// Positions the walk at the first item of workgroup blockIdx.x; false when its share is empty.
+__device__ __forceinline__ bool walk_begin(const AttnArgs& a, int nunits, Walk& w)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    long long total, unused;
+    count_items(a, 0, total, unused);
+    const long long W = total * nunits;
+    const int N = balanced_workgroups(a, W);
+    if ((int)blockIdx.x >= N) return false;
+    w.nunits = nunits;
+    w.cur = (long long)blockIdx.x * W / N;
+    w.hi = (long long)(blockIdx.x + 1) * W / N;         // > cur, because N <= W
+    const long long target = w.cur / nunits;       // the sequence that holds item `cur` holds per-unit item `target`
+    if (!a.t_dev) {
+        w.items = seq_items(a, a.t_host);
+        w.b = (int)(target / w.items);
+        w.base = (long long)w.b * w.items * nunits;
+        return true;
+    }
+    long long run = 0;
+    for (int c = 0; c < a.B; c += kWave) {
+        const int bb = c + lane;
+        const int it = bb < a.B ? seq_items(a, a.t_dev[bb]) : 0;
+        long long inc = it;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const long long v = __shfl_up(inc, off, kWave);
+            if (lane >= off) inc += v;
+        }
+        const long long tot = __shfl(inc, kWave - 1, kWave);
+        if (run + tot > target) {
+            const unsigned long long hit = __builtin_amdgcn_ballot_w64(run + inc > target);
+            const int f = __builtin_ctzll(hit);
+            w.b = c + f;
+            w.items = __shfl(it, f, kWave);
+            w.base = (run + __shfl(inc, f, kWave) - w.items) * nunits;
+            return true;
+        }
+        run += tot;
+    }
+    return false;                                   // not reached: target < total
+}
+
+// The unit piece at the walk's position (as many of the unit's remaining items as the share allows).
+template <int GT>
+__device__ __forceinline__ void walk_unit(const AttnArgs& a, const Walk& w, Unit& u, int& nitems)
+{
+    const int ngt = (a.G + GT - 1) / GT;
+    const long long rel = w.cur - w.base;
+    const int uib = (int)(rel / w.items);
+    const int item = (int)(rel % w.items);
+    const long long left = w.hi - w.cur;
+    nitems = w.items - item;
+    if (left < nitems) nitems = (int)left;
+    u.b = w.b;
+    u.kvh = uib / ngt;
+    u.g0 = (uib % ngt) * GT;
+    u.t = a.t_dev ? a.t_dev[w.b] : a.t_host;
+    u.pos = u.t + a.pos_offset;
+    u.split = 0;
+    u.last = 0;
+    u.r0 = item * a.item_rows;
+    u.r1 = min(u.r0 + nitems * a.item_rows, u.t - 1);
+    u.is_last = item + nitems == w.items;
+    u.direct = item == 0 && u.is_last;
+    u.pbase = ((size_t)blockIdx.x + (size_t)w.b * w.nunits + uib) * GT;
+    u.pstride = 1;
+}
+
+// Moves past nitems items; steps to the next sequence that has work when the current one is done.
+__device__ __forceinline__ void walk_advance(const AttnArgs& a, Walk& w, int nitems)
+{
+    w.cur += nitems;
+    if (w.cur >= w.hi) return;
+    if (w.cur == w.base + (long long)w.items * w.nunits) {
+        w.base = w.cur;
+        do {
+            if (++w.b >= a.B) {                      // lengths changed under the kernel (out of contract): stop
+                w.cur = w.hi;
+                return;
+            }
+            w.items = seq_items(a, a.t_dev ? a.t_dev[w.b] : a.t_host);
+        } while (w.items == 0);                      // cur < hi <= W: a later sequence has items
+    }
+}
+
+// Runs `body(unit)` for the one unit of the grid schedule, or for every unit piece of this
+// workgroup's share of the balanced schedule.
+template <int GT, bool BALANCED, typename F>
+__device__ __forceinline__ void for_each_unit(const AttnArgs& a, F&& body)
+{
+    Unit u;
+    if constexpr (!BALANCED) {
+        if (locate_unit<GT>(a, u)) body(u);
+    } else {
+        Walk w;
+        if (!walk_begin(a, a.Hkv * ((a.G + GT - 1) / GT), w)) return;
+        while (w.cur < w.hi) {
+            int nitems;
+            walk_unit<GT>(a, w, u, nitems);
+            body(u);
+            walk_advance(a, w, nitems);
+            if (w.cur < w.hi) __syncthreads();       // the next unit reuses the LDS staging
+        }
+    }
 }
 
 // q of the tile's heads (and, in the last split, the new k/v row): bias, RoPE, staging in LDS; the
@@ -168,10 +350,10 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, co
             O = fmaf(sv[d], w, O);
         }
         const int h = u.kvh * a.G + u.g0 + g;
-        if (a.nsplit == 1) {
+        if (u.direct) {
             static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + d] = from_f32<T>(O / L);
         } else {
-            const size_t pi = ((size_t)u.b * a.Hq + h) * a.nsplit + u.split;
+            const size_t pi = u.pbase + (size_t)g * u.pstride;
             a.part_o[pi * D + d] = O;
             if (d == 0) {
                 a.part_ml[pi * 2] = M;
@@ -182,8 +364,7 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, co
 }
 
 template <typename T, int LPR, int GT, int U, int NW>
-__global__ __launch_bounds__(NW * kWave)
-void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
+__device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds)
 {
     constexpr int VEC = Elt<T>::kVec;
     constexpr int D = LPR * VEC;
@@ -191,7 +372,6 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     constexpr int NRG = NW * RPW;               // row groups (independent softmax states) per workgroup
     constexpr int NTHR = NW * kWave;
 
-    extern __shared__ float lds[];
     float* sq = lds;                            // [GT][D]   roped q * qscale
     float* sk = sq + GT * D;                    // [D]       new k row (as stored)
     float* sv = sk + D;                         // [D]       new v row (as stored)
@@ -202,8 +382,6 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    Unit u;
-    if (!locate_unit<GT>(a, u)) return;
     const int r0 = u.r0, r1 = u.r1;
     const size_t head_off = a.slab + ((size_t)u.b * a.Hkv + u.kvh) * (size_t)a.S * D;
     T* kc = static_cast<T*>(a.k_cache) + head_off;
@@ -334,6 +512,14 @@ void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
     finish_unit<T, D, GT, NRG, NTHR>(a, u, st_ml, st_acc, snew, sv);
 }
 
+template <typename T, int LPR, int GT, int U, int NW, bool BALANCED>
+__global__ __launch_bounds__(NW * kWave)
+void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
+{
+    extern __shared__ float lds[];
+    for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { split_unit<T, LPR, GT, U, NW>(a, fr, u, lds); });
+}
+
 // ---------------------------------------------------------------------------------------------
 // Grouped-query form on the matrix cores (fp16 storage, D = 128; GT = 4, 8 or 16 query heads per
 // kv head and workgroup).
@@ -359,18 +545,20 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
-template <int GT, int NW>
-__global__ __launch_bounds__(NW * kWave)
-void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
+template <int D, int GT, int NW, bool DOUBLE_BUFFER>
+__device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds)
 {
     using T = __half;
     static_assert(GT == 4 || GT == 8 || GT == 16, "heads per tile");
-    constexpr int D = 128, VEC = 8;
+    static_assert(D == 64 || D == 128 || D == 256, "head size");
+    constexpr int VEC = 8;
     constexpr int NKB = D / 16;                 // k-blocks of the score product
+    constexpr int NKJ = D / 32;                 // 16-byte pieces of a K row per lane
+    constexpr int CG = D > 128 ? D / 128 : 1;   // groups of 128 output columns (16 lanes x 8)
+    constexpr int VSLOTS = D / VEC < 16 ? D / VEC : 16;   // lanes of a row of 16 that own distinct V columns
     constexpr int NTHR = NW * kWave;
     constexpr int RPI = NW * 16;                // rows per workgroup iteration
 
-    extern __shared__ float lds[];
     float* sq = lds;                            // [GT][D]
     float* sk = sq + GT * D;                    // [D]
     float* sv = sk + D;                         // [D]
@@ -383,26 +571,26 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
     const int wave = tid / kWave;
     const int slot = lane & 15;
     const int grp = lane >> 4;
-    Unit u;
-    if (!locate_unit<GT>(a, u)) return;
+    const int vslot = slot % VSLOTS;            // D = 64: lanes 8..15 of a row repeat lanes 0..7 (their results are unused)
     const int r0 = u.r0, r1 = u.r1;
     const size_t head_off = a.slab + ((size_t)u.b * a.Hkv + u.kvh) * (size_t)a.S * D;
     T* kc = static_cast<T*>(a.k_cache) + head_off;
     T* vc = static_cast<T*>(a.v_cache) + head_off;
     // K: lane (slot, grp) holds row `slot` of the batch, 16-byte pieces grp + 4*jp (columns grp*8 + jp*32 ..)
-    // V: lane (slot, grp) holds rows 4*grp + e of the batch, columns 8*slot .. 8*slot + 7
+    // V: lane (slot, grp) holds rows 4*grp + e of the batch, columns (cg*16 + slot)*8 .. +7
     const T* kp = kc + (size_t)(wave * 16 + slot) * D + grp * VEC;
-    const T* vp = vc + (size_t)(wave * 16 + 4 * grp) * D + slot * VEC;
+    const T* vp = vc + (size_t)(wave * 16 + 4 * grp) * D + vslot * VEC;
 
-    auto issue = [&](Vec16<T> (&kv)[4], Vec16<T> (&vv)[4], int rbase) {
+    auto issue = [&](Vec16<T> (&kv)[NKJ], Vec16<T> (&vv)[CG * 4], int rbase) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            kv[j] = load16_stream(kp + (size_t)rbase * D + j * 32);
-            vv[j] = load16_stream(vp + (size_t)(rbase + j) * D);
-        }
+        for (int j = 0; j < NKJ; ++j) kv[j] = load16_stream(kp + (size_t)rbase * D + j * 32);
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vv[cg * 4 + e] = load16_stream(vp + (size_t)(rbase + e) * D + cg * 128);
     };
     const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
-    Vec16<T> ka[4], va[4], kb[4], vb[4];
+    Vec16<T> ka[NKJ], va[CG * 4], kb[DOUBLE_BUFFER ? NKJ : 1], vb[DOUBLE_BUFFER ? CG * 4 : 1];
     if (nfull > 0) issue(ka, va, r0);
 
     stage_q_and_new_row<T, D, GT, NTHR>(a, fr, u, kc, vc, sq, sk, sv, snew);
@@ -413,7 +601,7 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
     {
         const float* qh = sq + (lane % GT) * D + grp * VEC;
 #pragma unroll
-        for (int jp = 0; jp < 4; ++jp)
+        for (int jp = 0; jp < NKJ; ++jp)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -427,15 +615,15 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
 
     // per lane: head (lane % GT); m is the same in every lane of a head, l is this lane's share
     float m = -INFINITY, l = 0.f;
-    f32x4 o[VEC];                               // o[c][r]: head (4*grp + r) % GT, column 8*slot + c
+    f32x4 o[CG * VEC];                          // o[cg*8 + c][r]: head (4*grp + r) % GT, column (cg*16 + slot)*8 + c
 #pragma unroll
-    for (int c = 0; c < VEC; ++c) o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < CG * VEC; ++c) o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto consume = [&](const Vec16<T> (&kv)[4], const Vec16<T> (&vv)[4], int rbase, auto masked_tag) {
+    auto consume = [&](const Vec16<T> (&kv)[NKJ], const Vec16<T> (&vv)[CG * 4], int rbase, auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int jp = 0; jp < 4; ++jp) {
+        for (int jp = 0; jp < NKJ; ++jp) {
             const f16x4 k0 = __builtin_shufflevector(kv[jp].raw, kv[jp].raw, 0, 1, 2, 3);
             const f16x4 k1 = __builtin_shufflevector(kv[jp].raw, kv[jp].raw, 4, 5, 6, 7);
             s0 = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qhi[jp * 2], s0, 0, 0, 0);
@@ -463,7 +651,7 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
 #pragma unroll
             for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, (lane & 48) | ((4 * grp + r) % GT), kWave);
 #pragma unroll
-            for (int c = 0; c < VEC; ++c)
+            for (int c = 0; c < CG * VEC; ++c)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) o[c][r] *= al[r];
             m = mnew;
@@ -477,42 +665,56 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
             phi[r] = hi;
             plo[r] = (_Float16)(p - (float)hi);
         }
-        u32x4 vw[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) vw[e] = __builtin_bit_cast(u32x4, vv[e].raw);
+        for (int cg = 0; cg < CG; ++cg) {
+            u32x4 vw[4];
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) {
-            // column c of the four rows: one byte-permute per pair of rows
-            constexpr unsigned kLow = 0x05040100u, kHigh = 0x07060302u;
-            const unsigned sel = (c & 1) ? kHigh : kLow;
-            const u32x2 packed = {__builtin_amdgcn_perm(vw[1][c / 2], vw[0][c / 2], sel),
-                                  __builtin_amdgcn_perm(vw[3][c / 2], vw[2][c / 2], sel)};
-            const f16x4 vcol = __builtin_bit_cast(f16x4, packed);
-            o[c] = __builtin_amdgcn_mfma_f32_16x16x16f16(phi, vcol, o[c], 0, 0, 0);
-            o[c] = __builtin_amdgcn_mfma_f32_16x16x16f16(plo, vcol, o[c], 0, 0, 0);
+            for (int e = 0; e < 4; ++e) vw[e] = __builtin_bit_cast(u32x4, vv[cg * 4 + e].raw);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+                // column c of the four rows: one byte-permute per pair of rows
+                constexpr unsigned kLow = 0x05040100u, kHigh = 0x07060302u;
+                const unsigned sel = (c & 1) ? kHigh : kLow;
+                const u32x2 packed = {__builtin_amdgcn_perm(vw[1][c / 2], vw[0][c / 2], sel),
+                                      __builtin_amdgcn_perm(vw[3][c / 2], vw[2][c / 2], sel)};
+                const f16x4 vcol = __builtin_bit_cast(f16x4, packed);
+                o[cg * VEC + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(phi, vcol, o[cg * VEC + c], 0, 0, 0);
+                o[cg * VEC + c] = __builtin_amdgcn_mfma_f32_16x16x16f16(plo, vcol, o[cg * VEC + c], 0, 0, 0);
+            }
         }
     };
 
     if (r1 > r0) {
         int rbase = r0;
-        for (int it = 0; it < nfull; it += 2) {
-            if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
-            consume(ka, va, rbase, std::false_type{});
-            if (it + 1 < nfull) {
-                if (it + 2 < nfull) issue(ka, va, rbase + 2 * RPI);
-                consume(kb, vb, rbase + RPI, std::false_type{});
+        if constexpr (DOUBLE_BUFFER) {
+            for (int it = 0; it < nfull; it += 2) {
+                if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
+                consume(ka, va, rbase, std::false_type{});
+                if (it + 1 < nfull) {
+                    if (it + 2 < nfull) issue(ka, va, rbase + 2 * RPI);
+                    consume(kb, vb, rbase + RPI, std::false_type{});
+                }
+                rbase += 2 * RPI;
             }
-            rbase += 2 * RPI;
+        } else {
+            // one register buffer: the other waves of the compute unit cover the load latency
+            for (int it = 0; it < nfull; ++it) {
+                consume(ka, va, rbase, std::false_type{});
+                rbase += RPI;
+                if (it + 1 < nfull) issue(ka, va, rbase);
+            }
         }
         rbase = r0 + nfull * RPI;
         if (rbase < r1) {
             // partial batch: rows past the end are read from the last valid row and masked
+            const int krow = min(rbase + wave * 16 + slot, r1 - 1);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int krow = min(rbase + wave * 16 + slot, r1 - 1);
-                const int vrow = min(rbase + wave * 16 + 4 * grp + j, r1 - 1);
-                ka[j] = load16_stream(kc + (size_t)krow * D + grp * VEC + j * 32);
-                va[j] = load16_stream(vc + (size_t)vrow * D + slot * VEC);
+            for (int j = 0; j < NKJ; ++j) ka[j] = load16_stream(kc + (size_t)krow * D + grp * VEC + j * 32);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int vrow = min(rbase + wave * 16 + 4 * grp + e, r1 - 1);
+#pragma unroll
+                for (int cg = 0; cg < CG; ++cg) va[cg * 4 + e] = load16_stream(vc + (size_t)vrow * D + vslot * VEC + cg * 128);
             }
             // a wave whose rows are all past the end must not touch its state (its scores are all -inf)
             if (rbase + wave * 16 < r1) consume(ka, va, rbase, std::true_type{});
@@ -526,24 +728,41 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
         st_ml[(wave * GT + slot) * 2] = m;
         st_ml[(wave * GT + slot) * 2 + 1] = l;
     }
-    if (4 * grp < GT) {
+    if (4 * grp < GT && slot < VSLOTS) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) st_acc[(size_t)(wave * GT + 4 * grp + r) * D + slot * VEC + c] = o[c][r];
+            for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+                for (int c = 0; c < VEC; ++c)
+                    st_acc[(size_t)(wave * GT + 4 * grp + r) * D + (cg * 16 + slot) * VEC + c] = o[cg * VEC + c][r];
     }
     __syncthreads();
     finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv);
 }
 
-template <int GT>
+template <int D, int GT, int NW, bool DOUBLE_BUFFER, bool BALANCED>
+__global__ __launch_bounds__(NW * kWave)
+void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
+{
+    extern __shared__ float lds[];
+    for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_unit<D, GT, NW, DOUBLE_BUFFER>(a, fr, u, lds); });
+}
+
+template <int D, int GT>
 int launch_gqa_mfma(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
-    constexpr int NW = 4, D = 128;
+    constexpr int NW = 4;
+    // rows of 512 bytes: one register buffer (two would not leave room for two waves per SIMD)
+    constexpr bool kDouble = D <= 128;
     const size_t lds_bytes = sizeof(float) * (size_t)(GT * D + 2 * D + GT + NW * GT * 2 + NW * GT * D);
+    if (lds_bytes > 64 * 1024) return ONELLM_EUNSUPPORTED;
     const int ngt = (a.G + GT - 1) / GT;
     const dim3 grid(a.Hkv * ngt, a.nsplit, a.B), block(NW * kWave);
-    hipLaunchKernelGGL((decode_attn_gqa_mfma_kernel<GT, NW>), grid, block, lds_bytes, st, a, fr);
+    if (a.bal_nwg > 0)
+        hipLaunchKernelGGL((decode_attn_gqa_mfma_kernel<D, GT, NW, kDouble, true>), dim3(a.bal_nwg), block, lds_bytes, st, a, fr);
+    else
+        hipLaunchKernelGGL((decode_attn_gqa_mfma_kernel<D, GT, NW, kDouble, false>), grid, block, lds_bytes, st, a, fr);
     return launch_status();
 }
 
@@ -580,6 +799,72 @@ void decode_attn_merge_kernel(const AttnArgs a, int D)
 #pragma unroll 8
         for (int s = 0; s < nvalid; ++s) O = fmaf(po[(size_t)s * D + d], w_s[s], O);
         static_cast<T*>(a.out)[(size_t)bh * D + d] = from_f32<T>(O * invL);
+    }
+}
+
+// The same merge for the balanced schedule: the workgroups that touched the unit of (sequence,
+// head) are found from the lengths exactly as the attention kernel found its shares; a unit one
+// workgroup saw whole was already written by it.  A unit can have more than 64 partial states
+// (one long sequence among short ones), so the passes run over blocks of 64 of them.
+template <typename T>
+__global__ __launch_bounds__(kWave)
+void decode_attn_merge_balanced_kernel(const AttnArgs a, int D)
+{
+    __shared__ float w_s[kWave];
+    const int bh = blockIdx.x, lane = threadIdx.x;
+    const int b = bh / a.Hq, h = bh % a.Hq;
+    const int t = a.t_dev ? a.t_dev[b] : a.t_host;
+    const int items = seq_items(a, t);
+    if (items == 0) return;
+    long long total, before;
+    count_items(a, b, total, before);
+    const int ngt = (a.G + a.gt - 1) / a.gt;
+    const int nunits = a.Hkv * ngt;
+    const int gi = h % a.G;
+    const int uib = (h / a.G) * ngt + gi / a.gt;
+    const int g = gi % a.gt;
+    const long long W = total * nunits;
+    const long long first = before * nunits + (long long)uib * items;
+    const int N = balanced_workgroups(a, W);
+    const int i0 = item_owner(first, W, N), i1 = item_owner(first + items - 1, W, N);
+    if (i0 == i1) return;
+    const int n = i1 - i0 + 1;
+    // entry of workgroup i0 + s: (i0 + s + global unit) * gt + g
+    const size_t e0 = ((size_t)i0 + (size_t)b * nunits + uib) * a.gt + g;
+    const float* ml = a.part_ml + e0 * 2;
+    const float* po = a.part_o + e0 * D;
+    const size_t step = (size_t)a.gt;
+    float M = -INFINITY;
+    for (int s = lane; s < n; s += kWave) M = fmaxf(M, ml[(size_t)s * step * 2]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, kWave));
+    float L = 0.f;
+    for (int s = lane; s < n; s += kWave)
+        L = fmaf(ml[(size_t)s * step * 2 + 1], __builtin_amdgcn_exp2f(ml[(size_t)s * step * 2] - M), L);
+    const float invL = 1.0f / wave_sum(L);
+    float O[8];                                               // D <= 512: 8 columns per lane
+#pragma unroll
+    for (int j = 0; j < 8; ++j) O[j] = 0.f;
+    for (int s0 = 0; s0 < n; s0 += kWave) {
+        const int cnt = min(kWave, n - s0);
+        __syncthreads();
+        w_s[lane] = lane < cnt ? __builtin_amdgcn_exp2f(ml[(size_t)(s0 + lane) * step * 2] - M) : 0.f;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int d = lane + j * kWave;
+            if (d < D) {
+                float acc = O[j];
+#pragma unroll 4
+                for (int s = 0; s < cnt; ++s) acc = fmaf(po[(size_t)(s0 + s) * step * D + d], w_s[s], acc);
+                O[j] = acc;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int d = lane + j * kWave;
+        if (d < D) static_cast<T*>(a.out)[(size_t)bh * D + d] = from_f32<T>(O[j] * invL);
     }
 }
 
@@ -726,7 +1011,10 @@ int launch_split(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     if (lds_bytes > 64 * 1024) return ONELLM_EUNSUPPORTED;
     const int ngt = (a.G + GT - 1) / GT;
     const dim3 grid(a.Hkv * ngt, a.nsplit, a.B), block(NW * kWave);
-    hipLaunchKernelGGL((decode_attn_split_kernel<T, LPR, GT, U, NW>), grid, block, lds_bytes, st, a, fr);
+    if (a.bal_nwg > 0)
+        hipLaunchKernelGGL((decode_attn_split_kernel<T, LPR, GT, U, NW, true>), dim3(a.bal_nwg), block, lds_bytes, st, a, fr);
+    else
+        hipLaunchKernelGGL((decode_attn_split_kernel<T, LPR, GT, U, NW, false>), grid, block, lds_bytes, st, a, fr);
     return launch_status();
 }
 
@@ -738,13 +1026,20 @@ int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     return launch_split<T, LPR, GT, 4, 4>(a, fr, st);
 }
 
+// head sizes the matrix-core kernel is built for (fp16 caches)
+constexpr bool mfma_head_size(int D) { return D == 64 || D == 128 || D == 256; }
+
 // query heads one workgroup serves (they share every K/V row it reads)
 int heads_per_tile(bool fp16, int D, int G)
 {
     if (G == 1) return 1;       // one head: memory-bound on either kernel (measured equal), keep the lighter one
-    // two or more query heads per kv head, fp16, D = 128: both products on the matrix cores, where
-    // up to 16 heads cost the same as 4
-    if (fp16 && D == 128 && tune_get("attn_gqa_valu") != 1) return G <= 4 ? 4 : (G <= 8 ? 8 : 16);
+    // two or more query heads per kv head, fp16: both products on the matrix cores, where up to 16
+    // heads cost the same as 4 (8 at D = 256: the per-wave states of 16 heads would not fit 64 KiB of LDS)
+    if (fp16 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1) {
+        const int cap = D == 256 ? 8 : 16;
+        const int gt = G <= 4 ? 4 : (G <= 8 ? 8 : 16);
+        return gt < cap ? gt : cap;
+    }
     return G == 2 ? 2 : 4;
 }
 
@@ -752,17 +1047,26 @@ template <typename T, int LPR>
 int launch_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
     constexpr bool kHalf = std::is_same<T, __half>::value;
-    switch (heads_per_tile(kHalf, LPR * Elt<T>::kVec, a.G)) {
+    constexpr int D = LPR * Elt<T>::kVec;
+    const int gt = heads_per_tile(kHalf, D, a.G);
+    if constexpr (kHalf && mfma_head_size(D)) {
+        if (a.G > 1 && tune_get("attn_gqa_valu") != 1) {
+            switch (gt) {
+                case 4: return launch_gqa_mfma<D, 4>(a, fr, st);
+                case 8: return launch_gqa_mfma<D, 8>(a, fr, st);
+                case 16:
+                    if constexpr (D <= 128) return launch_gqa_mfma<D, 16>(a, fr, st);
+                    break;
+                default: break;
+            }
+            return ONELLM_EUNSUPPORTED;
+        }
+    }
+    switch (gt) {
         case 1: return launch_shape<T, LPR, 1>(a, fr, st);
         case 2: return launch_shape<T, LPR, 2>(a, fr, st);
-        case 8: return launch_gqa_mfma<8>(a, fr, st);
-        case 16: return launch_gqa_mfma<16>(a, fr, st);
-        default: break;
+        default: return launch_shape<T, LPR, 4>(a, fr, st);
     }
-    if constexpr (kHalf && LPR == 16) {
-        if (tune_get("attn_gqa_valu") != 1) return launch_gqa_mfma<4>(a, fr, st);
-    }
-    return launch_shape<T, LPR, 4>(a, fr, st);
 }
 
 template <typename T>
@@ -780,6 +1084,23 @@ int launch_lpr(int lpr, const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     }
 }
 
+constexpr int kBalancedWorkgroups = 512;   // two 4-wave workgroups per compute unit: what the register budgets keep resident
+
+// rows per work item of the balanced schedule: one workgroup iteration of the kernel that runs
+int item_rows_for(bool fp16, int D, int G)
+{
+    if (G > 1 && fp16 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1) return 64;
+    const int lpr = D * (fp16 ? 2 : 4) / 16;
+    const int rpi = 1024 / lpr;               // 4 waves x (64 / lpr) rows x 4 per row group
+    return rpi < 64 ? 64 : rpi;
+}
+
+// Off unless asked for (tuning knob attn_balanced = 1).  Measured on MI355X it equalises the rows per workgroup as
+// designed, but every shape it helps pays for it with the merge launch (~8 us) that the grid schedule often avoids,
+// and where both need the merge the hardware dispatcher already balances the grid schedule's chunks as well:
+// ragged batch 32 x 8 kv heads, lengths 1024..8192: 106 us grid, 108-110 us balanced; 384 equal units: 125 vs 127 us.
+bool balanced_by_default() { return false; }
+
 int max_splits(int max_t)
 {
     int n = (max_t + kMinChunk - 1) / kMinChunk;
@@ -793,7 +1114,12 @@ extern "C" size_t onellm_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int
 {
     (void)Hkv;
     if (B <= 0 || Hq <= 0 || D <= 0 || max_t <= 0) return 256;
-    const size_t n = (size_t)B * Hq * onellm::max_splits(max_t) * (size_t)(D + 2) * sizeof(float);
+    // grid schedule: one partial state per (sequence, head, split); balanced schedule: one per
+    // (workgroup + unit) and tile head - at most 16 heads per tile, and the padded tiles of all
+    // units hold less than twice the query heads
+    const size_t grid_entries = (size_t)B * Hq * onellm::max_splits(max_t);
+    const size_t bal_entries = (size_t)onellm::kBalancedWorkgroups * 2 * 16 + (size_t)B * Hq * 2;
+    const size_t n = (grid_entries > bal_entries ? grid_entries : bal_entries) * (size_t)(D + 2) * sizeof(float);
     return (n + 255) & ~(size_t)255;
 }
 
@@ -845,7 +1171,9 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     const int ngt = (G + gt - 1) / gt;
     const long base_wgs = (long)B * Hkv * ngt;
     const int user_target = tune_get("attn_target_wgs");
-    const int target = user_target > 0 ? user_target : (t_dev ? 4096 : 256);
+    // (the matrix-core kernel at D = 64 has half the bytes in flight per workgroup: two per compute unit)
+    const bool mfma64 = dtype == ONELLM_FP16 && D == 64 && G > 1 && tune_get("attn_gqa_valu") != 1;
+    const int target = user_target > 0 ? user_target : (t_dev ? 4096 : (mfma64 ? 512 : 256));
     int nsplit = (int)((target + base_wgs - 1) / base_wgs);
     int cap = max_splits(max_t);
     if (user_target <= 0) {
@@ -862,8 +1190,34 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     nsplit = (max_t + chunk - 1) / chunk;
     a.chunk = chunk;
     a.nsplit = nsplit;
+    a.gt = gt;
 
-    if (nsplit > 1) {
+    // Balanced schedule: a fixed number of workgroups (what the chip holds at once) share the rows
+    // of the step equally, whatever the lengths and however the units divide among compute units.
+    const long nunits = (long)Hkv * ngt;
+    bool merge_needed = nsplit > 1;
+    const int bal = tune_get("attn_balanced");
+    if (forced <= 0 && (bal == 1 || (bal != 0 && balanced_by_default()))) {
+        a.item_rows = item_rows_for(dtype == ONELLM_FP16, D, G);
+        const long long items = (max_t - 1 + a.item_rows - 1) / a.item_rows;
+        const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);
+        const int user_wgs = tune_get("attn_balanced_wgs");
+        long long nwg = user_wgs > 0 ? user_wgs : kBalancedWorkgroups;
+        if (nwg > kBalancedWorkgroups * 2) nwg = kBalancedWorkgroups * 2;
+        // no workgroup for fewer than four items
+        if (nwg > (wmax + 3) / 4) nwg = (wmax + 3) / 4;
+        // equal lengths and as many units as workgroups or more: whole units per workgroup when they divide evenly
+        a.bal_nwg = (int)nwg;
+        a.nsplit = 1;
+        merge_needed = !(!t_dev && (B * nunits) % nwg == 0);
+        const size_t entries = ((size_t)a.bal_nwg + (size_t)B * nunits) * gt;
+        if (merge_needed) {
+            const size_t need = entries * (size_t)(D + 2) * sizeof(float);
+            if (!workspace || workspace_bytes < need) return ONELLM_EWORKSPACE;
+        }
+        a.part_o = static_cast<float*>(workspace);
+        a.part_ml = a.part_o + entries * D;
+    } else if (nsplit > 1) {
         const size_t need = (size_t)B * Hq * nsplit * (size_t)(D + 2) * sizeof(float);
         if (!workspace || workspace_bytes < need) return ONELLM_EWORKSPACE;
         a.part_o = static_cast<float*>(workspace);
@@ -876,11 +1230,17 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     hipStream_t st = static_cast<hipStream_t>(stream);
     int rc = dtype == ONELLM_FP16 ? launch_lpr<__half>(lpr, a, fr, st) : launch_lpr<float>(lpr, a, fr, st);
     if (rc != 0) return rc;
-    if (nsplit > 1) {
-        if (dtype == ONELLM_FP16)
+    if (merge_needed) {
+        if (a.bal_nwg > 0) {
+            if (dtype == ONELLM_FP16)
+                hipLaunchKernelGGL((decode_attn_merge_balanced_kernel<__half>), dim3(B * Hq), dim3(kWave), 0, st, a, D);
+            else
+                hipLaunchKernelGGL((decode_attn_merge_balanced_kernel<float>), dim3(B * Hq), dim3(kWave), 0, st, a, D);
+        } else if (dtype == ONELLM_FP16) {
             hipLaunchKernelGGL((decode_attn_merge_kernel<__half>), dim3(B * Hq), dim3(kWave), 0, st, a, D);
-        else
+        } else {
             hipLaunchKernelGGL((decode_attn_merge_kernel<float>), dim3(B * Hq), dim3(kWave), 0, st, a, D);
+        }
         rc = launch_status();
     }
     return rc;

@@ -16,6 +16,8 @@ Knob g_knobs[] = {
     {"norm_tpr", {-1}},          // threads per row of the norm kernels: 64 .. 1024
     {"attn_target_wgs", {-1}},   // workgroups the sequence split of decode attention aims for
     {"attn_nsplit", {-1}},       // force the number of sequence splits
+    {"attn_balanced", {-1}},     // 1 / 0: force the balanced workgroup schedule of decode attention on / off
+    {"attn_balanced_wgs", {-1}}, // workgroups of the balanced schedule
     {"attn_gqa_valu", {-1}},     // 1: grouped-query heads on the vector ALU kernel instead of the MFMA one
 };
 }  // namespace

@@ -254,39 +254,80 @@ def test_constant_value_rows_at_full_size(capi, dev):
     assert (out.float() - 0.375).abs().max().item() <= 1e-3
 
 
-def test_options_on_the_matrix_core_kernel(capi, ref, dev):
-    """The same option matrix as test_options on a shape that takes the MFMA grouped-query kernel (fp16, D = 128,
-    4 query heads per kv head), with one and with several sequence splits."""
-    announce("attn options, mfma kernel")
-    qkv, bias, kc, vc = _case(np.float16, 2, 8, 2, 128, 200, 2, seed=23, std=0.5)
+@pytest.mark.parametrize("D,Hq", [(128, 8), (64, 8), (256, 8), (64, 32), (256, 12)])
+def test_options_on_the_matrix_core_kernel(capi, ref, dev, D, Hq):
+    """The same option matrix as test_options on shapes that take the MFMA grouped-query kernel (fp16, head size 64,
+    128 or 256, 4 / 6 / 16 query heads per kv head), with one and with several sequence splits."""
+    announce("attn options, mfma kernel", D, Hq)
+    qkv, bias, kc, vc = _case(np.float16, 2, Hq, 2, D, 200, 2, seed=23 + D, std=0.5)
     for nsplit in (-1, 3):
         capi.tune_set("attn_nsplit", nsplit)
         try:
-            _assert_parity(_run_both(capi, ref, dev, qkv, None, kc, vc, 8, 177, 128, layer=1), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 0), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 64), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 128, pos_offset=-1, layer=1), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 128, base=500000.0), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 128, flags=capi.ATTN_NO_V_BIAS), np.float16)
-            res = _run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 177, 128, flags=capi.ATTN_NO_CACHE_WRITE)
+            _assert_parity(_run_both(capi, ref, dev, qkv, None, kc, vc, Hq, 177, D, layer=1), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, 0), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D // 2), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, pos_offset=-1, layer=1), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, base=500000.0), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, flags=capi.ATTN_NO_V_BIAS), np.float16)
+            res = _run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, flags=capi.ATTN_NO_CACHE_WRITE)
             _assert_parity(res, np.float16)
             np.testing.assert_array_equal(_bits(res[2]), _bits(kc))
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, 8, 200, 128), np.float16)       # t == S
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 200, D), np.float16)       # t == S
+            for t in (1, 2, 16, 17, 63, 65):                                                           # short and partial batches
+                _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), np.float16)
         finally:
             capi.tune_set("attn_nsplit", -1)
 
 
+@pytest.mark.parametrize("dtype,Hq,Hkv,D", [(np.float16, 8, 2, 128), (np.float16, 4, 4, 128), (np.float16, 14, 2, 128),
+                                            (np.float16, 40, 2, 128), (np.float16, 8, 1, 64), (np.float16, 12, 2, 256),
+                                            (np.float16, 6, 3, 32), (np.float32, 8, 2, 64), (np.float32, 3, 3, 128)])
+@pytest.mark.parametrize("nwg", [1, 3, 50, 512, 1024])
+def test_balanced_schedule(capi, ref, dev, dtype, Hq, Hkv, D, nwg):
+    """The balanced workgroup schedule (equal shares of rows per workgroup, units split wherever a share ends) on
+    ragged and equal lengths: lengths of 1 and 2, one long sequence among short ones (a unit with many partial
+    states), more workgroups than work items."""
+    announce("attn balanced", dtype.__name__, Hq, Hkv, D, "nwg", nwg)
+    B, S = 7, 1500
+    qkv, bias, kc, vc = _case(dtype, B, Hq, Hkv, D, S, 2, seed=nwg * 31 + Hq + D, std=0.5)
+    capi.tune_set("attn_balanced", 1)
+    capi.tune_set("attn_balanced_wgs", nwg)
+    try:
+        _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, np.array([1, 1500, 64, 65, 2, 777, 130]), D, layer=1), dtype)
+        _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, np.array([1, 1, 1, 1, 1, 1, 1]), D), dtype)
+        _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, np.array([3, 2, 1400, 2, 1, 1, 9]), D), dtype)
+        for t in (1, 2, 129, 640, 1500):
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), dtype)
+    finally:
+        capi.tune_set("attn_balanced", -1)
+        capi.tune_set("attn_balanced_wgs", -1)
+
+
+def test_balanced_schedule_many_sequences(capi, ref, dev):
+    """More sequences than a wave has lanes: the length scan of the balanced schedule runs over several blocks."""
+    announce("attn balanced, 150 sequences")
+    B, Hq, Hkv, D, S = 150, 4, 2, 128, 96
+    qkv, bias, kc, vc = _case(np.float16, B, Hq, Hkv, D, S, 1, seed=151, std=0.5)
+    t = np.random.default_rng(9).integers(1, S + 1, size=B)
+    capi.tune_set("attn_balanced", 1)
+    try:
+        for nwg in (5, 512):
+            capi.tune_set("attn_balanced_wgs", nwg)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), np.float16)
+    finally:
+        capi.tune_set("attn_balanced", -1)
+        capi.tune_set("attn_balanced_wgs", -1)
+
+
 def test_random_shapes_sweep(capi, ref, dev):
-    """Forty seeded random (dtype, heads, group size, head size, lengths, split count) combinations, ragged lengths
+    """Sixty seeded random (dtype, heads, group size, head size, lengths, split count, schedule) combinations, ragged lengths
     included: every kernel variant and padded head tile gets shapes nobody picked by hand."""
     rng = np.random.default_rng(2024)
-    for case in range(40):
+    for case in range(60):
         dtype = [np.float16, np.float32][int(rng.integers(0, 2))]
         D = int(rng.choice([16, 32, 64, 128, 128, 128, 256]))
         Hkv = int(rng.integers(1, 4))
         G = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 20]))
-        if D >= 256:
-            G = min(G, 4)
         Hq = Hkv * G
         B = int(rng.integers(1, 5))
         S = int(rng.integers(8, 420))
@@ -295,10 +336,17 @@ def test_random_shapes_sweep(capi, ref, dev):
         t = lens if ragged else int(lens.max())
         nsplit = int(rng.choice([-1, -1, 1, 2, 3, 7]))
         rot = int(rng.choice([D, D, D // 2, 0]))
-        announce("attn sweep", case, dtype.__name__, "B", B, "Hq", Hq, "Hkv", Hkv, "D", D, "S", S, "t", t, "nsplit", nsplit, "rot", rot)
+        balanced = int(rng.choice([-1, 0, 1])) if nsplit == -1 else -1
+        nwg = int(rng.choice([-1, 2, 9, 100]))
+        announce("attn sweep", case, dtype.__name__, "B", B, "Hq", Hq, "Hkv", Hkv, "D", D, "S", S, "t", t, "nsplit", nsplit, "rot", rot,
+                 "balanced", balanced, "nwg", nwg)
         qkv, bias, kc, vc = _case(dtype, B, Hq, Hkv, D, S, 1, seed=5000 + case, std=0.5)
         capi.tune_set("attn_nsplit", nsplit)
+        capi.tune_set("attn_balanced", balanced)
+        capi.tune_set("attn_balanced_wgs", nwg)
         try:
             _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, rot), dtype)
         finally:
             capi.tune_set("attn_nsplit", -1)
+            capi.tune_set("attn_balanced", -1)
+            capi.tune_set("attn_balanced_wgs", -1)
