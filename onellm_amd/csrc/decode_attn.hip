@@ -106,6 +106,26 @@ __device__ __forceinline__ int seq_items(const AttnArgs& a, int t)
     return n < 1 ? 1 : n;
 }
 
+// The schedule is the same in every lane; saying so keeps it in scalar registers (the kernels that
+// walk it are short of vector registers).
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ long long uniform(long long v)
+{
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(unsigned long long)v);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)((unsigned long long)v >> 32));
+    return (long long)(((unsigned long long)hi << 32) | lo);
+}
+
+// Thread index as a value the compiler takes as new each time it is asked for: everything a unit
+// derives from it (addresses, masks, lane roles) is then recomputed per unit instead of being
+// hoisted out of the loop over units and held in registers across the streaming loop.
+__device__ __forceinline__ int lane_id_per_unit()
+{
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    return tid;
+}
+
 __device__ __forceinline__ long long wave_sum_i64(long long v)
 {
 #pragma unroll
@@ -129,8 +149,8 @@ __device__ __forceinline__ void count_items(const AttnArgs& a, int before, long 
         tot += it;
         if (bb < before) pre += it;
     }
-    total = wave_sum_i64(tot);
-    prefix = wave_sum_i64(pre);
+    total = uniform(wave_sum_i64(tot));
+    prefix = uniform(wave_sum_i64(pre));
 }
 
 // workgroup that owns item x when W items are dealt to N workgroups as [i*W/N, (i+1)*W/N)
@@ -163,8 +183,8 @@ __device__ __forceinline__ bool walk_begin(const AttnArgs& a, int nunits, Walk& 
     const int N = balanced_workgroups(a, W);
     if ((int)blockIdx.x >= N) return false;
     w.nunits = nunits;
-    w.cur = (long long)blockIdx.x * W / N;
-    w.hi = (long long)(blockIdx.x + 1) * W / N;         // > cur, because N <= W
+    w.cur = uniform((long long)blockIdx.x * W / N);
+    w.hi = uniform((long long)(blockIdx.x + 1) * W / N);         // > cur, because N <= W
     const long long target = w.cur / nunits;       // the sequence that holds item `cur` holds per-unit item `target`
     if (!a.t_dev) {
         w.items = seq_items(a, a.t_host);
@@ -187,11 +207,11 @@ __device__ __forceinline__ bool walk_begin(const AttnArgs& a, int nunits, Walk& 
             const unsigned long long hit = __builtin_amdgcn_ballot_w64(run + inc > target);
             const int f = __builtin_ctzll(hit);
             w.b = c + f;
-            w.items = __shfl(it, f, kWave);
-            w.base = (run + __shfl(inc, f, kWave) - w.items) * nunits;
+            w.items = uniform(__shfl(it, f, kWave));
+            w.base = (run + uniform(__shfl(inc, f, kWave)) - w.items) * nunits;
             return true;
         }
-        run += tot;
+        run += uniform(tot);
     }
     return false;                                   // not reached: target < total
 }
@@ -202,15 +222,16 @@ __device__ __forceinline__ void walk_unit(const AttnArgs& a, const Walk& w, Unit
 {
     const int ngt = (a.G + GT - 1) / GT;
     const long long rel = w.cur - w.base;
-    const int uib = (int)(rel / w.items);
-    const int item = (int)(rel % w.items);
+    const int uib = uniform((int)(rel / w.items));
+    const int item = uniform((int)(rel - (long long)uib * w.items));
     const long long left = w.hi - w.cur;
     nitems = w.items - item;
     if (left < nitems) nitems = (int)left;
+    nitems = uniform(nitems);
     u.b = w.b;
     u.kvh = uib / ngt;
     u.g0 = (uib % ngt) * GT;
-    u.t = a.t_dev ? a.t_dev[w.b] : a.t_host;
+    u.t = uniform(a.t_dev ? a.t_dev[w.b] : a.t_host);
     u.pos = u.t + a.pos_offset;
     u.split = 0;
     u.last = 0;
@@ -234,7 +255,7 @@ __device__ __forceinline__ void walk_advance(const AttnArgs& a, Walk& w, int nit
                 w.cur = w.hi;
                 return;
             }
-            w.items = seq_items(a, a.t_dev ? a.t_dev[w.b] : a.t_host);
+            w.items = uniform(seq_items(a, a.t_dev ? a.t_dev[w.b] : a.t_host));
         } while (w.items == 0);                      // cur < hi <= W: a later sequence has items
     }
 }
@@ -267,7 +288,7 @@ template <typename T, int D, int GT, int NTHR>
 __device__ __forceinline__ void stage_q_and_new_row(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, T* kc, T* vc,
                                                     float* sq, float* sk, float* sv, float* snew)
 {
-    const int tid = threadIdx.x;
+    const int tid = lane_id_per_unit();
     const T* qkv = static_cast<const T*>(a.qkv) + (size_t)u.b * (a.Hq + 2 * a.Hkv) * D;
     const T* bias = static_cast<const T*>(a.bias);
     for (int i = tid; i < GT * (D / 2); i += NTHR) {
@@ -333,7 +354,7 @@ template <typename T, int D, int GT, int NST, int NTHR>
 __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, const float* st_ml, const float* st_acc,
                                             const float* snew, const float* sv)
 {
-    for (int i = threadIdx.x; i < GT * D; i += NTHR) {
+    for (int i = lane_id_per_unit(); i < GT * D; i += NTHR) {
         const int g = i / D, d = i % D;
         if (u.g0 + g >= a.G) continue;
         float M = u.is_last ? snew[g] : -INFINITY;
@@ -379,7 +400,7 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
     float* st_ml = snew + GT;                   // [NRG][GT][2]
     float* st_acc = st_ml + NRG * GT * 2;       // [NRG][GT][D]
 
-    const int tid = threadIdx.x;
+    const int tid = lane_id_per_unit();
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const int r0 = u.r0, r1 = u.r1;
@@ -566,7 +587,7 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
     float* st_ml = snew + GT;                   // [NW][GT][2]
     float* st_acc = st_ml + NW * GT * 2;        // [NW][GT][D]
 
-    const int tid = threadIdx.x;
+    const int tid = lane_id_per_unit();
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const int slot = lane & 15;
@@ -774,31 +795,50 @@ template <typename T>
 __global__ __launch_bounds__(kWave)
 void decode_attn_merge_kernel(const AttnArgs a, int D)
 {
-    __shared__ float w_s[kWave];
+    constexpr int PRE = 16;                                    // splits whose partial sums are requested up front
     const int bh = blockIdx.x, lane = threadIdx.x;
     const int b = bh / a.Hq;
+    const float* ml = a.part_ml + (size_t)bh * a.nsplit * 2;
+    const float* po = a.part_o + (size_t)bh * a.nsplit * D;
+    // everything that does not depend on the length is requested before the length is looked at: the
+    // (m, l) pairs of all splits and the first block of partial sums.  Entries of splits past the
+    // sequence's end hold stale bytes; they are selected away below, never multiplied.
+    float m_raw = 0.f, l_raw = 0.f;
+    if (lane < a.nsplit) {
+        m_raw = ml[lane * 2];
+        l_raw = ml[lane * 2 + 1];
+    }
+    const int npre = min(a.nsplit, PRE);
+    float o_pre[PRE];
+#pragma unroll
+    for (int s = 0; s < PRE; ++s) o_pre[s] = (s < npre && lane < D) ? po[(size_t)s * D + lane] : 0.f;
     const int t = a.t_dev ? a.t_dev[b] : a.t_host;
     if (t < 1 || t > a.S) return;
     const int nvalid = min((t - 1) / a.chunk + 1, a.nsplit);   // t above max_t is out of contract: stay in bounds
-    const float* ml = a.part_ml + (size_t)bh * a.nsplit * 2;
-    const float* po = a.part_o + (size_t)bh * a.nsplit * D;
-    float m = -INFINITY, l = 0.f;
-    if (lane < nvalid) {
-        m = ml[lane * 2];
-        l = ml[lane * 2 + 1];
-    }
+    const float m = lane < nvalid ? m_raw : -INFINITY;
+    const float l = lane < nvalid ? l_raw : 0.f;
     float M = m;
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, kWave));
     const float w = __builtin_amdgcn_exp2f(m - M);          // 0 for the lanes without a split
     const float invL = 1.0f / wave_sum(l * w);
-    w_s[lane] = w;
-    __syncthreads();
-    for (int d = lane; d < D; d += kWave) {
+    // the loops are uniform over the wave (the weights travel by lane exchange); only the accesses are guarded
+    for (int d0 = 0; d0 < D; d0 += kWave) {
+        const int d = d0 + lane;
         float O = 0.f;
-#pragma unroll 8
-        for (int s = 0; s < nvalid; ++s) O = fmaf(po[(size_t)s * D + d], w_s[s], O);
-        static_cast<T*>(a.out)[(size_t)bh * D + d] = from_f32<T>(O * invL);
+        int s = 0;
+        if (d0 == 0) {
+#pragma unroll
+            for (; s < PRE; ++s) {
+                const float ws = __shfl(w, s, kWave);
+                if (s < nvalid) O = fmaf(o_pre[s], ws, O);
+            }
+        }
+        for (; s < nvalid; ++s) {
+            const float ws = __shfl(w, s, kWave);
+            if (d < D) O = fmaf(po[(size_t)s * D + d], ws, O);
+        }
+        if (d < D) static_cast<T*>(a.out)[(size_t)bh * D + d] = from_f32<T>(O * invL);
     }
 }
 
@@ -1095,11 +1135,17 @@ int item_rows_for(bool fp16, int D, int G)
     return rpi < 64 ? 64 : rpi;
 }
 
-// Off unless asked for (tuning knob attn_balanced = 1).  Measured on MI355X it equalises the rows per workgroup as
-// designed, but every shape it helps pays for it with the merge launch (~8 us) that the grid schedule often avoids,
-// and where both need the merge the hardware dispatcher already balances the grid schedule's chunks as well:
-// ragged batch 32 x 8 kv heads, lengths 1024..8192: 106 us grid, 108-110 us balanced; 384 equal units: 125 vs 127 us.
-bool balanced_by_default() { return false; }
+// When the balanced schedule is the default (tuning knob attn_balanced = 1 / 0 forces it on / off): per-sequence
+// lengths on the matrix-core kernel with no more units than workgroups.  Measured on MI355X against the grid
+// schedule (us per step, lengths uniform in [S/8, S]): 32 q / 8 kv heads, batch 32, S 8192: 117 -> 102; 64 q / 8 kv,
+// batch 16: 81 -> 57; batch 8, S 16384: 97 -> 61; D = 256, batch 16, S 4096: 90 -> 74.  With equal lengths the grid
+// schedule needs no merge launch and is as fast or faster; with more units than workgroups (batch 128) and on the
+// vector-ALU kernel (which keeps four workgroups per compute unit resident) the hardware dispatcher balances the
+// grid schedule's chunks as well as the fixed shares do.
+bool balanced_by_default(bool ragged, bool mfma, long units)
+{
+    return ragged && mfma && units <= kBalancedWorkgroups;
+}
 
 int max_splits(int max_t)
 {
@@ -1197,7 +1243,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     const long nunits = (long)Hkv * ngt;
     bool merge_needed = nsplit > 1;
     const int bal = tune_get("attn_balanced");
-    if (forced <= 0 && (bal == 1 || (bal != 0 && balanced_by_default()))) {
+    if (forced <= 0 && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, dtype == ONELLM_FP16 && G > 1 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1, (long)B * nunits)))) {
         a.item_rows = item_rows_for(dtype == ONELLM_FP16, D, G);
         const long long items = (max_t - 1 + a.item_rows - 1) / a.item_rows;
         const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);

@@ -3,7 +3,9 @@
 // the C entry point on the null stream (the reference launches everything there; onellmSetLaunchStream names
 // another one for the calling thread) and throws
 // std::runtime_error when the entry point reports an error.  No printing, no device sync.
+#include <map>
 #include <mutex>
+#include <utility>
 #include <stdexcept>
 #include <string>
 #include <hip/hip_runtime_api.h>
@@ -35,26 +37,33 @@ int abi_dtype(const Tensor* t, const char* what)
 }
 
 // The reference signature of the attention launcher has no workspace parameter, so the shim owns
-// one grow-only device buffer per process (freed at exit by the runtime).
+// grow-only device buffers (freed at exit by the runtime): one per (device, launch stream), so
+// that steps queued on different streams or devices never share scratch.
 struct Workspace {
+    struct Buffer {
+        void* ptr = nullptr;
+        size_t bytes = 0;
+    };
     std::mutex mu;
-    void* ptr = nullptr;
-    size_t bytes = 0;
-    void* get(size_t need)
+    std::map<std::pair<int, hipStream_t>, Buffer> buffers;
+    void* get(size_t need, hipStream_t stream)
     {
+        int device = 0;
+        throw_on_error((int)hipGetDevice(&device), "workspace device");
         std::lock_guard<std::mutex> g(mu);
-        if (need > bytes) {
-            // the old buffer may still be in use by work queued earlier on the null stream
-            if (ptr) {
-                throw_on_error((int)hipDeviceSynchronize(), "workspace sync");
-                throw_on_error((int)hipFree(ptr), "workspace free");
-                ptr = nullptr;
-                bytes = 0;
+        Buffer& b = buffers[std::make_pair(device, stream)];
+        if (need > b.bytes) {
+            // the old buffer may still be in use by work queued earlier on its stream
+            if (b.ptr) {
+                throw_on_error((int)hipStreamSynchronize(stream), "workspace sync");
+                throw_on_error((int)hipFree(b.ptr), "workspace free");
+                b.ptr = nullptr;
+                b.bytes = 0;
             }
-            throw_on_error((int)hipMalloc(&ptr, need), "workspace alloc");
-            bytes = need;
+            throw_on_error((int)hipMalloc(&b.ptr, need), "workspace alloc");
+            b.bytes = need;
         }
-        return ptr;
+        return b.ptr;
     }
 };
 Workspace g_attn_ws;
@@ -119,7 +128,7 @@ void launchDecoderMaskedMHA(Tensor* qkv_buf, BaseWeight& qkv, Tensor* k_cache, T
     int rc = call(nullptr, 0);
     if (rc == ONELLM_EWORKSPACE) {
         const size_t ws_bytes = onellm_decode_attn_workspace_bytes(batch_size, head_num, kv_head_num, head_size, cur_step);
-        rc = call(g_attn_ws.get(ws_bytes), ws_bytes);
+        rc = call(g_attn_ws.get(ws_bytes, t_launch_stream), ws_bytes);
     }
     throw_on_error(rc, "launchDecoderMaskedMHA");
 }

@@ -1,5 +1,6 @@
 // Decode-side layers of oneLLM over this backend (declared in onellm/layers.h): they sequence the launch*
 // functions and the projection GEMMs for one decode step and own no arithmetic of their own.
+#include <map>
 #include <mutex>
 #include <set>
 #include <tuple>
@@ -32,19 +33,27 @@ int cols_of(const Tensor* t)
     return n;
 }
 
-// scratch for the GEMM library's split-K algorithms: one per process, created on first use
+// scratch for the GEMM library's split-K algorithms: one per device, created on first use there
 struct GemmWorkspace {
-    std::once_flag once;
-    void* ptr = nullptr;
-    size_t bytes = 0;
-    void* get()
+    struct Buffer {
+        void* ptr = nullptr;
+        size_t bytes = 0;
+    };
+    std::mutex mu;
+    std::map<int, Buffer> buffers;
+    Buffer get()
     {
-        std::call_once(once, [this] {
-            const size_t want = onellm_linear_workspace_bytes();
-            if (hipMalloc(&ptr, want) == hipSuccess) bytes = want;
-            else { ptr = nullptr; (void)hipGetLastError(); }
-        });
-        return ptr;
+        int device = 0;
+        hip_ok(hipGetDevice(&device), "gemm workspace device");
+        std::lock_guard<std::mutex> g(mu);
+        auto it = buffers.find(device);
+        if (it != buffers.end()) return it->second;
+        Buffer b;
+        const size_t want = onellm_linear_workspace_bytes();
+        if (hipMalloc(&b.ptr, want) == hipSuccess) b.bytes = want;
+        else { b.ptr = nullptr; (void)hipGetLastError(); }      // the library then keeps to algorithms that need none
+        buffers[device] = b;
+        return b;
     }
 };
 GemmWorkspace g_gemm_ws;
@@ -115,11 +124,11 @@ void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool tr
         require(!shared_out_buf, "launchLinearGemm: shared_out_buf needs a {2, M, N} output");
         require(rows_of(output) == M && cols_of(output) == N, "launchLinearGemm: output shape");
     }
-    void* ws = g_gemm_ws.get();
+    const GemmWorkspace::Buffer ws = g_gemm_ws.get();
     const int dtype_code = input->dtype == FP32 ? ONELLM_FP32 : ONELLM_FP16;
-    tune_once(dtype_code, M, K, N, ldy, trans_b ? 1 : 0, ws, g_gemm_ws.bytes);
-    const int rc = onellm_linear(input->dtype == FP32 ? ONELLM_FP32 : ONELLM_FP16, input->data, weight.data, y, M, K, N, ldy,
-                                 trans_b ? 1 : 0, ws, g_gemm_ws.bytes, onellmGetLaunchStream());
+    tune_once(dtype_code, M, K, N, ldy, trans_b ? 1 : 0, ws.ptr, ws.bytes);
+    const int rc = onellm_linear(dtype_code, input->data, weight.data, y, M, K, N, ldy, trans_b ? 1 : 0, ws.ptr, ws.bytes,
+                                 onellmGetLaunchStream());
     if (rc != 0) throw std::runtime_error(std::string("[TM][ERROR] launchLinearGemm: ") + onellm_error_string(rc) + " \n");
 }
 
