@@ -104,11 +104,14 @@ def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=
     bias = torch.randn((Hq + 2 * Hkv) * D, device=dev).mul_(0.5).half()
     out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
     max_t = t if t_dev is None else int(t_dev.max().item())
-    ws = torch.empty(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, max_t), dtype=torch.uint8, device=dev)
+    # zero-filled once and declared so, as the launcher shim does with the workspace it owns: shapes whose sequences
+    # are split are then finished inside the attention kernel instead of by a merge launch
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, max_t), dtype=torch.uint8, device=dev)
 
     def step(i):
         kc, vc = sets[i % nsets]
-        capi.decode_attn(qkv, bias, kc, vc, out, Hq, max_t, D, 10000.0, t_dev=t_dev, max_t=max_t, workspace=ws)
+        capi.decode_attn(qkv, bias, kc, vc, out, Hq, max_t, D, 10000.0, t_dev=t_dev, max_t=max_t, workspace=ws,
+                         flags=capi.ATTN_ZEROED_WORKSPACE)
 
     ms = time_steps(step, steps, warmup)
     bench_attention.last_step = step

@@ -37,6 +37,12 @@ extern "C" {
 #define ONELLM_ATTN_NO_V_BIAS     0x1u /* skip the v-bias add (reference decode kernel behaviour,
                                           src/kernels/decoder_masked_attn.cu:257-258)            */
 #define ONELLM_ATTN_NO_CACHE_WRITE 0x2u /* do not store the new k/v row (read-only caches)        */
+#define ONELLM_ATTN_ZEROED_WORKSPACE 0x4u /* the caller zero-filled the whole workspace once, after
+                                          allocating it, and nothing but onellm_decode_attn has written
+                                          it since.  A split sequence is then finished inside the one
+                                          kernel (per-unit arrival counters at the front of the workspace,
+                                          left at zero by every call) instead of by a second launch.
+                                          Calls that share a workspace must not overlap.              */
 
 typedef void* onellm_stream_t;
 
@@ -70,6 +76,7 @@ const char* onellm_error_string(int code);
  *              that the prefill kernel uses, qkv_bias_and_RoPE.cu:140)
  *   workspace  device scratch of at least onellm_decode_attn_workspace_bytes() bytes, 256-byte
  *              aligned; contents on entry are irrelevant and nothing is carried between calls
+ *              (unless ONELLM_ATTN_ZEROED_WORKSPACE says otherwise)
  *
  * Arithmetic is fp32 throughout; with ONELLM_FP16 the cache, qkv, bias and out are fp16 and the
  * new k/v rows are rounded to fp16 before they take part in this step's scores.

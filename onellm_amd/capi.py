@@ -14,6 +14,7 @@ FP32, FP16 = 0, 1
 EINVAL, EUNSUPPORTED, EWORKSPACE = -1, -2, -3
 ATTN_NO_V_BIAS = 0x1
 ATTN_NO_CACHE_WRITE = 0x2
+ATTN_ZEROED_WORKSPACE = 0x4
 TOPK_BLOCKS_PER_ROW = 8
 
 # every symbol include/onellm_hip.h declares: name -> (restype, argtypes)

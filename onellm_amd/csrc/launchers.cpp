@@ -61,6 +61,9 @@ struct Workspace {
                 b.bytes = 0;
             }
             throw_on_error((int)hipMalloc(&b.ptr, need), "workspace alloc");
+            // zero-filled once: the attention entry point may then finish split sequences in one launch
+            // (ONELLM_ATTN_ZEROED_WORKSPACE); only that entry point ever writes the buffer
+            throw_on_error((int)hipMemsetAsync(b.ptr, 0, need, stream), "workspace clear");
             b.bytes = need;
         }
         return b.ptr;
@@ -123,11 +126,12 @@ void launchDecoderMaskedMHA(Tensor* qkv_buf, BaseWeight& qkv, Tensor* k_cache, T
                                   batch_size, head_num, kv_head_num, head_size, cs.S, /*layer=*/0, cs.layers,
                                   cur_step, nullptr, cur_step,
                                   static_params.rotary_embedding_dim, static_params.rotary_embedding_base,
-                                  rope_pos_offset, /*flags=*/0u, ws, ws_bytes, launch_stream());
+                                  rope_pos_offset, ONELLM_ATTN_ZEROED_WORKSPACE, ws, ws_bytes, launch_stream());
     };
     int rc = call(nullptr, 0);
     if (rc == ONELLM_EWORKSPACE) {
-        const size_t ws_bytes = onellm_decode_attn_workspace_bytes(batch_size, head_num, kv_head_num, head_size, cur_step);
+        // sized for the cache's whole length, so that it is created once and not regrown as the step advances
+        const size_t ws_bytes = onellm_decode_attn_workspace_bytes(batch_size, head_num, kv_head_num, head_size, cs.S);
         rc = call(g_attn_ws.get(ws_bytes, t_launch_stream), ws_bytes);
     }
     throw_on_error(rc, "launchDecoderMaskedMHA");

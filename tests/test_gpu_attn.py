@@ -319,6 +319,45 @@ def test_balanced_schedule_many_sequences(capi, ref, dev):
         capi.tune_set("attn_balanced_wgs", -1)
 
 
+@pytest.mark.parametrize("dtype,Hq,Hkv,D", [(np.float16, 8, 2, 128), (np.float16, 4, 4, 128), (np.float16, 40, 2, 128),
+                                            (np.float16, 8, 1, 64), (np.float16, 12, 2, 256), (np.float32, 8, 2, 64),
+                                            (np.float32, 3, 3, 128)])
+@pytest.mark.parametrize("schedule", ["grid2", "grid5", "grid64", "balanced3", "balanced50", "balanced512"])
+def test_fused_finish_with_a_zeroed_workspace(capi, ref, dev, dtype, Hq, Hkv, D, schedule):
+    """ONELLM_ATTN_ZEROED_WORKSPACE: the piece of a split sequence that arrives last merges the sequence inside the
+    attention kernel (no merge launch).  One workspace, zero-filled once, serves a series of calls with different
+    lengths and splits: every call must leave its arrival counters at zero for the next."""
+    announce("attn fused finish", dtype.__name__, Hq, Hkv, D, schedule)
+    B, S = 7, 1500
+    qkv, bias, kc, vc = _case(dtype, B, Hq, Hkv, D, S, 2, seed=len(schedule) * 17 + Hq + D, std=0.5)
+    d_qkv, d_bias = torch.from_numpy(qkv).to(dev), torch.from_numpy(bias).to(dev)
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    if schedule.startswith("grid"):
+        capi.tune_set("attn_nsplit", int(schedule[4:]))
+    else:
+        capi.tune_set("attn_balanced", 1)
+        capi.tune_set("attn_balanced_wgs", int(schedule[8:]))
+    try:
+        for rep, t in enumerate([np.array([1, 1500, 64, 65, 2, 777, 130]), 1500, np.array([3, 2, 1400, 2, 1, 1, 9]), 640,
+                                 np.array([1, 1, 1, 1, 1, 1, 1]), np.array([1500, 1499, 1498, 700, 701, 702, 64]), 129]):
+            d_kc, d_vc = torch.from_numpy(kc).to(dev), torch.from_numpy(vc).to(dev)
+            out = torch.zeros(B, Hq * D, dtype=d_qkv.dtype, device=dev)
+            ragged = isinstance(t, np.ndarray)
+            t_dev = torch.from_numpy(t.astype(np.int32)).to(dev) if ragged else None
+            max_t = int(t.max()) if ragged else t
+            capi.decode_attn(d_qkv, d_bias, d_kc, d_vc, out, Hq, max_t, D, 10000.0, layer=1, t_dev=t_dev, max_t=max_t,
+                             flags=capi.ATTN_ZEROED_WORKSPACE, workspace=ws)
+            r_kc, r_vc = kc.copy(), vc.copy()
+            want = ref.decode_attn(qkv, bias, r_kc, r_vc, Hq, t, D, 10000.0, layer=1)
+            _assert_parity((out.cpu().numpy(), want, d_kc.cpu().numpy(), d_vc.cpu().numpy(), r_kc, r_vc), dtype)
+            # (there is one counter per unit and at least one unit per kv head)
+            assert int(ws[:B * Hkv * 4].view(torch.int32).abs().max().item()) == 0, "arrival counters not back at zero (call %d)" % rep
+    finally:
+        capi.tune_set("attn_nsplit", -1)
+        capi.tune_set("attn_balanced", -1)
+        capi.tune_set("attn_balanced_wgs", -1)
+
+
 def test_random_shapes_sweep(capi, ref, dev):
     """Sixty seeded random (dtype, heads, group size, head size, lengths, split count, schedule) combinations, ragged lengths
     included: every kernel variant and padded head tile gets shapes nobody picked by hand."""
