@@ -1215,6 +1215,7 @@ int launch_lpr(int lpr, const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     }
 }
 
+constexpr size_t kCounterBytes = 64 * 1024; // arrival counters of the fused finish: the first bytes of every workspace
 constexpr int kBalancedWorkgroups = 512;   // two 4-wave workgroups per compute unit: what the register budgets keep resident
 
 // rows per work item of the balanced schedule: one workgroup iteration of the kernel that runs
@@ -1256,8 +1257,7 @@ extern "C" size_t onellm_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int
     // units hold less than twice the query heads
     const size_t grid_entries = (size_t)B * Hq * onellm::max_splits(max_t);
     const size_t bal_entries = (size_t)onellm::kBalancedWorkgroups * 2 * 16 + (size_t)B * Hq * 2;
-    const size_t counters = (((size_t)B * Hq * sizeof(int)) + 255) & ~(size_t)255;      // one per unit at most
-    const size_t n = counters + (grid_entries > bal_entries ? grid_entries : bal_entries) * (size_t)(D + 2) * sizeof(float);
+    const size_t n = onellm::kCounterBytes + (grid_entries > bal_entries ? grid_entries : bal_entries) * (size_t)(D + 2) * sizeof(float);
     return (n + 255) & ~(size_t)255;
 }
 
@@ -1335,10 +1335,11 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     const long nunits = (long)Hkv * ngt;
     bool merge_needed = nsplit > 1;
     // arrival counters of the fused finish sit at the front of a workspace the caller keeps zeroed
-    // (the region is set aside whether or not this call uses it, so that calls with and without
-    // the flag can share one workspace)
-    const size_t counter_bytes = ((size_t)B * nunits * sizeof(int) + 255) & ~(size_t)255;
-    const bool fused_finish = (flags & ONELLM_ATTN_ZEROED_WORKSPACE) && tune_get("attn_fused_finish") != 0;
+    // (the region has one size for every shape and is set aside whether or not this call uses it, so
+    // that calls of any shapes, with and without the flag, can share one workspace)
+    const size_t counter_bytes = kCounterBytes;
+    const bool fused_finish = (flags & ONELLM_ATTN_ZEROED_WORKSPACE) && tune_get("attn_fused_finish") != 0
+                              && (size_t)B * nunits * sizeof(int) <= kCounterBytes;
     float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + counter_bytes);
     const int bal = tune_get("attn_balanced");
     if (forced <= 0 && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, dtype == ONELLM_FP16 && G > 1 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1, (long)B * nunits)))) {

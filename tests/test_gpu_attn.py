@@ -358,6 +358,34 @@ def test_fused_finish_with_a_zeroed_workspace(capi, ref, dev, dtype, Hq, Hkv, D,
         capi.tune_set("attn_balanced_wgs", -1)
 
 
+def test_fused_finish_at_full_size_matches_the_merge_launch(capi, dev):
+    """Config-3 size (batch 32, 32 query heads over 8 kv heads, 8192-row caches) and a small-batch split shape: the
+    in-kernel finish gives the merge launch's result (same pieces, merged in piece order either way) and is
+    bit-identical from run to run, over a series of length vectors on one workspace."""
+    torch.manual_seed(33)
+    B, Hq, Hkv, D, S = 32, 32, 8, 128, 8192
+    kc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+    vc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+    qkv = torch.randn(B, Hq + 2 * Hkv, D, device=dev).mul_(0.5).half()
+    bias = torch.randn((Hq + 2 * Hkv) * D, device=dev).mul_(0.5).half()
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    rng = np.random.default_rng(33)
+    outs = [torch.zeros(B, Hq * D, dtype=torch.float16, device=dev) for _ in range(3)]
+    for rep in range(12):
+        nb = [32, 32, 4, 1][rep % 4]
+        if rep % 3 == 2:
+            t, t_dev = int(rng.integers(2000, S + 1)), None
+        else:
+            lens = rng.integers(1, S + 1, size=nb).astype(np.int32)
+            t, t_dev = int(lens.max()), torch.from_numpy(lens).to(dev)
+        announce("attn fused finish full size, rep", rep, "batch", nb, "t", t, "ragged", t_dev is not None)
+        for o, fl in zip(outs, (0, capi.ATTN_ZEROED_WORKSPACE, capi.ATTN_ZEROED_WORKSPACE)):
+            capi.decode_attn(qkv[:nb], bias, kc[:, :nb].contiguous() if nb != B else kc, vc[:, :nb].contiguous() if nb != B else vc,
+                             o[:nb], Hq, t, D, 10000.0, t_dev=t_dev, max_t=t, workspace=ws, flags=fl | capi.ATTN_NO_CACHE_WRITE)
+        assert torch.equal(outs[1][:nb], outs[2][:nb])
+        assert (outs[0][:nb].float() - outs[1][:nb].float()).abs().max().item() <= 1e-3
+
+
 def test_random_shapes_sweep(capi, ref, dev):
     """Sixty seeded random (dtype, heads, group size, head size, lengths, split count, schedule) combinations, ragged lengths
     included: every kernel variant and padded head tile gets shapes nobody picked by hand."""
