@@ -441,7 +441,7 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, co
     __syncthreads();
     if (*arrived != u.npieces - 1) return;
     if (tid == 0) __hip_atomic_store(a.counters + u.counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
-    constexpr int BATCH = 8;                                    // pieces whose loads are in flight together
+    constexpr int BATCH = 16;                                   // pieces whose loads are in flight together
     for (int i = tid; i < GT * D; i += NTHR) {
         const int g = i / D, d = i % D;
         if (u.g0 + g >= a.G) continue;
