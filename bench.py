@@ -24,7 +24,7 @@ HBM_PEAK_GBPS = 8000.0   # MI355X, published
 
 # HBM bytes per launch of the headline kernel as counted by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
 # each scaled by the same counter's reading for a 1 GiB device copy: x2.0000 and x1.0000), keyed by context.
-MEASURED_TRAFFIC_BYTES = {4096: 1074413568}
+MEASURED_TRAFFIC_BYTES = {4096: 1074432616}
 
 
 def attn_bytes(B, Hq, Hkv, D, t_list, e):
