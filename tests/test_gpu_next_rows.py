@@ -26,10 +26,17 @@ def _pack(B, seq_len, lens):
 
 @pytest.mark.parametrize("dtype,Hq,Hkv,D,rd", [(np.float32, 2, 1, 8, 128), (np.float16, 32, 32, 128, 128),
                                                (np.float16, 32, 8, 128, 64), (np.float32, 4, 2, 64, 64),
-                                               (np.float16, 4, 4, 12, 12), (np.float32, 3, 1, 6, 6)])
+                                               (np.float16, 4, 4, 12, 12), (np.float32, 3, 1, 6, 6),
+                                               (np.float16, 5, 1, 8, 8), (np.float16, 6, 2, 16, 6), (np.float16, 3, 3, 32, 32),
+                                               (np.float16, 40, 8, 64, 32), (np.float16, 9, 3, 256, 256), (np.float16, 2, 1, 512, 100),
+                                               (np.float32, 7, 7, 4, 4), (np.float32, 3, 1, 128, 128), (np.float32, 2, 2, 256, 254)])
 @pytest.mark.parametrize("with_bias", [True, False])
-def test_prefill_matches_oracle(capi, ref, dev, dtype, Hq, Hkv, D, rd, with_bias):
-    announce("prefill rope", dtype.__name__, Hq, Hkv, D, rd, with_bias)
+@pytest.mark.parametrize("kernel", ["rows", "index"])
+def test_prefill_matches_oracle(capi, ref, dev, dtype, Hq, Hkv, D, rd, with_bias, kernel):
+    # "rows": the kernel whose threads keep one (token, piece) and walk the heads (rows of a power-of-two number of
+    # 16-byte pieces); "index": the general kernel, forced for every shape
+    announce("prefill rope", dtype.__name__, Hq, Hkv, D, rd, with_bias, kernel)
+    capi.tune_set("prefill_generic", 1 if kernel == "index" else -1)
     rng = np.random.default_rng(Hq * 100 + D)
     B, S = 4, 40
     lens = [40, 17, 1, 0]
@@ -45,6 +52,7 @@ def test_prefill_matches_oracle(capi, ref, dev, dtype, Hq, Hkv, D, rd, with_bias
     d_bias = torch.from_numpy(bias).to(dev) if with_bias else None
     capi.qkv_bias_rope_transpose(d[0], d[1], d[2], d[3], d_bias, torch.from_numpy(po).to(dev), torch.from_numpy(hist).to(dev),
                                  rd, 10000.0)
+    capi.tune_set("prefill_generic", -1)
     ref.qkv_bias_rope_transpose(q, k, v, qkv, bias, po, hist, rd, 10000.0)
     for got, want in zip(d[:3], (q, k, v)):
         np.testing.assert_array_equal(_bits(got.cpu().numpy()), _bits(want))
