@@ -54,6 +54,12 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m onellm_amd.build` "
                                "(there is no CPU fallback)")
+        # torch first: its wheel ships a HIP runtime of its own under the same soname, and the copy that is loaded
+        # first is the one every library of the process has to share (tensors come from torch's)
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SYMBOLS.items():
             fn = getattr(L, name)
