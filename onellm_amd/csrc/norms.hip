@@ -59,6 +59,14 @@ void norm_rows_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __
 
     Vec16<T> x[RPT][NV];
     float ss[RPT];
+    // gamma is requested with the row, not after the reduction: by then it has arrived, instead of
+    // costing every workgroup a second memory round trip between its barrier and its stores
+    Vec16<T> g[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int idx = lane + j * TPR;
+        if (idx < nvec) g[j] = load16(gamma + idx * VEC);
+    }
 #pragma unroll
     for (int k = 0; k < RPT; ++k) {
         ss[k] = 0.f;
@@ -111,13 +119,12 @@ void norm_rows_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __
         for (int j = 0; j < NV; ++j) {
             const int idx = lane + j * TPR;
             if (idx < nvec) {
-                const Vec16<T> g = load16(gamma + idx * VEC);
 #pragma unroll
                 for (int k = 0; k < RPT; ++k) {
                     if (row0 + k < N) {
                         const float inv = rsqrtf(ss[k] / (float)H + eps);
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) x[k][j].set(e, g.get(e) * r[k][j][e] * inv);
+                        for (int e = 0; e < VEC; ++e) x[k][j].set(e, g[j].get(e) * r[k][j][e] * inv);
                         store16_stream(out + (size_t)(row0 + k) * H + idx * VEC, x[k][j]);
                     }
                 }
@@ -142,13 +149,12 @@ void norm_rows_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __
         for (int j = 0; j < NV; ++j) {
             const int idx = lane + j * TPR;
             if (idx < nvec) {
-                const Vec16<T> g = load16(gamma + idx * VEC);
 #pragma unroll
                 for (int k = 0; k < RPT; ++k) {
                     if (row0 + k < N) {
                         const float inv = rsqrtf(ss[k] / (float)H + eps);
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) x[k][j].set(e, g.get(e) * x[k][j].get(e) * inv);
+                        for (int e = 0; e < VEC; ++e) x[k][j].set(e, g[j].get(e) * x[k][j].get(e) * inv);
                         store16_stream(out + (size_t)(row0 + k) * H + idx * VEC, x[k][j]);
                     }
                 }
@@ -233,12 +239,13 @@ int launch_norm(T* out, T* residual, const T* bias, const T* gamma, float eps, i
         return launch_status();
     }
     const int nvec = H / VEC;
-    // team size: two 16-byte vectors per thread and row measured best (8 KiB fp16 rows -> 256
-    // threads, 16 KiB -> 512)
+    // team size: one 16-byte vector per thread and row up to 512 threads, then more vectors per thread
+    // (8 KiB fp16 rows -> 512 threads x 1: 23.3 / 44.4 us plain / fused at 8192 rows against 23.5 / 45.6 with
+    // 256 x 2; 16 KiB rows -> 512 x 2: 44.7 / 90.8 against 47.2 / 90.4 with 1024 x 1)
     int tpr = tune_get("norm_tpr");
     if (tpr != 64 && tpr != 128 && tpr != 256 && tpr != 512 && tpr != 1024) {
         tpr = 64;
-        while (tpr < 1024 && nvec > tpr * 2) tpr *= 2;
+        while (tpr < 512 && nvec > tpr) tpr *= 2;
     }
     while (tpr < 1024 && nvec > tpr * 16) tpr *= 2;
     // several rows per team (2 or 4, all loads issued up front) were measured too and gave nothing
