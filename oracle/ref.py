@@ -11,7 +11,9 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libonellm_ref.so")
+# ONELLM_REF_LIB selects another build of the same source, e.g. oracle/libonellm_ref_asan.so (`make -C oracle
+# check-asan` runs the oracle's tests against it under AddressSanitizer + UBSan)
+_LIB_PATH = os.environ.get("ONELLM_REF_LIB") or os.path.join(_HERE, "libonellm_ref.so")
 
 FP32, FP16 = 0, 1
 ATTN_NO_V_BIAS = 0x1
@@ -22,7 +24,7 @@ def build(force=False):
     """Compile the oracle with gcc (a few hundred ms)."""
     if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(
             os.path.join(_HERE, "onellm_ref.c")):
-        subprocess.run(["make", "-C", _HERE, "-B", "libonellm_ref.so"], check=True, capture_output=True)
+        subprocess.run(["make", "-C", _HERE, "-B", os.path.basename(_LIB_PATH)], check=True, capture_output=True)
     return _LIB_PATH
 
 
