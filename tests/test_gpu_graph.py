@@ -11,8 +11,11 @@ from conftest import announce
 pytestmark = pytest.mark.gpu
 
 
-def test_captured_decode_step_replays_bit_identically(capi, dev):
-    announce("graph capture of a decode step")
+@pytest.mark.parametrize("fused_finish", [False, True])
+def test_captured_decode_step_replays_bit_identically(capi, dev, fused_finish):
+    # fused_finish: the attention workspace is zero-filled once and declared so; the split sequences are then
+    # finished inside the attention kernel (arrival counters, reset by every call) instead of by a merge launch
+    announce("graph capture of a decode step, fused finish", fused_finish)
     torch.manual_seed(11)
     B, Hq, Hkv, D, S, t, H, I, V = 4, 32, 8, 128, 2048, 1500, 4096, 2048, 8000
     x0 = torch.randn(B, H, device=dev).half()
@@ -22,7 +25,8 @@ def test_captured_decode_step_replays_bit_identically(capi, dev):
     kc0 = torch.randn(1, B, Hkv, S, D, device=dev).mul(0.5).half()
     vc0 = torch.randn(1, B, Hkv, S, D, device=dev).mul(0.5).half()
     t_dev = torch.tensor([1500, 700, 33, 1], dtype=torch.int32, device=dev)
-    ws = torch.empty(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, t), dtype=torch.uint8, device=dev)
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, t), dtype=torch.uint8, device=dev)
+    attn_flags = capi.ATTN_ZEROED_WORKSPACE if fused_finish else 0
     act_in0 = torch.randn(B, 2, I, device=dev).half()
     logits = torch.randn(B * 2, V, device=dev)
     topk_ws = torch.empty(capi.beam_topk_workspace_bytes(B, 2, 4) // 4, dtype=torch.float32, device=dev)
@@ -38,7 +42,7 @@ def test_captured_decode_step_replays_bit_identically(capi, dev):
 
     def step():
         capi.rmsnorm(x, gamma, 1e-5)
-        capi.decode_attn(qkv0, bias, kc, vc, attn_out, Hq, t, D, 10000.0, t_dev=t_dev, max_t=t, workspace=ws)
+        capi.decode_attn(qkv0, bias, kc, vc, attn_out, Hq, t, D, 10000.0, t_dev=t_dev, max_t=t, workspace=ws, flags=attn_flags)
         capi.fused_add_bias_residual_rmsnorm(res, x, None, gamma, 1e-5)
         capi.silu_and_mul(act_in0, act_out)
         capi.beam_topk(logits, B, 2, 4, workspace=topk_ws)
