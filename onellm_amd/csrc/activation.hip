@@ -5,7 +5,9 @@
 namespace onellm {
 namespace {
 
-__device__ __forceinline__ float silu_mul(float x, float y) { return (x / (1.0f + __expf(-x))) * y; }
+// the reciprocal is the hardware's (v_rcp_f32, 1 ulp) rather than an IEEE division: ten instructions fewer per
+// element in a kernel whose vector ALU is more than half busy
+__device__ __forceinline__ float silu_mul(float x, float y) { return (x * __builtin_amdgcn_rcpf(1.0f + __expf(-x))) * y; }
 
 template <typename T, int NV>
 __global__ __launch_bounds__(256)
