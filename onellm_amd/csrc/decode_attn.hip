@@ -1171,6 +1171,9 @@ int heads_per_tile(bool fp16, int D, int G)
         const int gt = G <= 4 ? 4 : (G <= 8 ? 8 : 16);
         return gt < cap ? gt : cap;
     }
+    // fp32 caches: a lane holds 4 columns, so 8 heads per tile still fit the registers and more than 4 heads
+    // per kv head need no second pass over the rows
+    if (!fp16 && G > 4) return 8;
     return G == 2 ? 2 : 4;
 }
 
@@ -1196,6 +1199,9 @@ int launch_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     switch (gt) {
         case 1: return launch_shape<T, LPR, 1>(a, fr, st);
         case 2: return launch_shape<T, LPR, 2>(a, fr, st);
+        case 8:
+            if constexpr (!kHalf) return launch_shape<T, LPR, 8>(a, fr, st);
+            return ONELLM_EUNSUPPORTED;
         default: return launch_shape<T, LPR, 4>(a, fr, st);
     }
 }
