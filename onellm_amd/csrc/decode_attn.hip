@@ -386,7 +386,7 @@ __device__ __forceinline__ float fetch(const float* p)
 // split) and write either the output (single split) or this split's partial state.  The caller has
 // synchronised the workgroup on st_ml / st_acc / snew.
 template <typename T, int D, int GT, int NST, int NTHR>
-__device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, const float* st_ml, const float* st_acc,
+__device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, float* st_ml, const float* st_acc,
                                             const float* snew, const float* sv)
 {
     for (int i = lane_id_per_unit(); i < GT * D; i += NTHR) {
@@ -434,7 +434,7 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, co
     // moves through these scoped accesses, and nobody waits on anybody.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                                            // all stores done; st_ml no longer read
-    int* arrived = reinterpret_cast<int*>(const_cast<float*>(st_ml));
+    int* arrived = reinterpret_cast<int*>(st_ml);                  // the merged states are no longer needed: reuse a word
     const int tid = lane_id_per_unit();
     if (tid == 0)
         *arrived = __hip_atomic_fetch_add(a.counters + u.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
