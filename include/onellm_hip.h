@@ -81,8 +81,9 @@ const char* onellm_error_string(int code);
  * Arithmetic is fp32 throughout; with ONELLM_FP16 the cache, qkv, bias and out are fp16 and the
  * new k/v rows are rounded to fp16 before they take part in this step's scores.
  * Shapes: Hq % Hkv == 0, 1 <= t <= S, D <= 512, B <= 65535.  Head sizes whose rows are a power of
- * two number of bytes (16..1024) in 16-byte aligned caches run the tiled kernels; anything else
- * (D = 96, 80, ..., odd D, unaligned caches) runs a slower scalar kernel with the same results.
+ * two number of bytes (16..1024), or 10, 12, 20, 24, 40 or 48 16-byte pieces (D = 80, 96, 160, 192,
+ * 320, 384 in fp16), in 16-byte aligned caches run the tiled kernels; anything else (odd D,
+ * D = 72, 100, ..., unaligned caches) runs a slower scalar kernel with the same results.
  */
 int onellm_decode_attn(int dtype,
                        const void* qkv, const void* qkv_bias,

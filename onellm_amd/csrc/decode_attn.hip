@@ -475,11 +475,16 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, fl
     }
 }
 
-template <typename T, int LPR, int GT, int U, int NW>
+// DP = 16-byte pieces a cache row really has (D = DP * VEC); LPR = the lanes that share a row, the
+// power of two at or above DP.  With DP < LPR (head sizes 80, 96, 160, 192, ...) the surplus lanes of
+// a row group re-read the row's first piece with a zero q (they add nothing to the dot product) and
+// keep no result; the memory traffic is unchanged, a load instruction just carries fewer distinct bytes.
+template <typename T, int LPR, int DP, int GT, int U, int NW>
 __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds)
 {
+    static_assert(DP >= 1 && DP <= LPR && 2 * DP > LPR, "pieces per row and lanes per row");
     constexpr int VEC = Elt<T>::kVec;
-    constexpr int D = LPR * VEC;
+    constexpr int D = DP * VEC;
     constexpr int RPW = kWave / LPR;            // cache rows per wave per load instruction
     constexpr int NRG = NW * RPW;               // row groups (independent softmax states) per workgroup
     constexpr int NTHR = NW * kWave;
@@ -501,7 +506,8 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
 
     // ---- the first rows of the chunk are requested before anything else: they do not depend on q,
     // and their latency then hides the q / new-row set-up below
-    const int col = (lane % LPR) * VEC;         // first of this lane's VEC columns
+    const bool owner = DP == LPR || lane % LPR < DP;        // this lane owns VEC columns of the row
+    const int col = owner ? (lane % LPR) * VEC : 0;         // first of this lane's VEC columns
     const int rg = wave * RPW + lane / LPR;     // row group of this lane
     constexpr int RPI = U * NRG;                // rows per workgroup iteration
     const T* kp = kc + col;
@@ -525,7 +531,7 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
 #pragma unroll
     for (int g = 0; g < GT; ++g)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) qr[g][e] = sq[g * D + col + e];
+        for (int e = 0; e < VEC; ++e) qr[g][e] = owner ? sq[g * D + col + e] : 0.f;
 
     // ---- stream the history rows of this chunk
     float m[GT], l[GT], acc[GT][VEC];
@@ -617,8 +623,10 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
             st_ml[(rg * GT + g) * 2] = m[g];
             st_ml[(rg * GT + g) * 2 + 1] = l[g];
         }
+        if (owner) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) st_acc[(size_t)(rg * GT + g) * D + col + e] = acc[g][e];
+            for (int e = 0; e < VEC; ++e) st_acc[(size_t)(rg * GT + g) * D + col + e] = acc[g][e];
+        }
     }
     __syncthreads();
     finish_unit<T, D, GT, NRG, NTHR>(a, u, st_ml, st_acc, snew, sv);
@@ -629,7 +637,16 @@ __global__ __launch_bounds__(NW * kWave)
 void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
 {
     extern __shared__ float lds[];
-    for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { split_unit<T, LPR, GT, U, NW>(a, fr, u, lds); });
+    for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { split_unit<T, LPR, LPR, GT, U, NW>(a, fr, u, lds); });
+}
+
+// the same kernel for rows that do not fill their lanes (grid schedule only)
+template <typename T, int LPR, int DP, int GT>
+__global__ __launch_bounds__(4 * kWave)
+void decode_attn_split_padded_kernel(const AttnArgs a, const RopeFreqs fr)
+{
+    extern __shared__ float lds[];
+    for_each_unit<GT, false>(a, [&](const Unit& u) { split_unit<T, LPR, DP, GT, 4, 4>(a, fr, u, lds); });
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1149,6 +1166,42 @@ int launch_split(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     return launch_status();
 }
 
+template <typename T, int LPR, int DP, int GT>
+int launch_padded(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    constexpr int D = DP * Elt<T>::kVec;
+    constexpr int NRG = 4 * (kWave / LPR);
+    const size_t lds_bytes = sizeof(float) * (size_t)(GT * D + 2 * D + GT + NRG * GT * 2 + (size_t)NRG * GT * D);
+    if (lds_bytes > 64 * 1024) return ONELLM_EUNSUPPORTED;
+    const int ngt = (a.G + GT - 1) / GT;
+    const dim3 grid(a.Hkv * ngt, a.nsplit, a.B), block(4 * kWave);
+    hipLaunchKernelGGL((decode_attn_split_padded_kernel<T, LPR, DP, GT>), grid, block, lds_bytes, st, a, fr);
+    return launch_status();
+}
+
+// head sizes between the powers of two that the tiled kernel is built for, in 16-byte pieces per row
+constexpr bool padded_pieces(int dp) { return dp == 10 || dp == 12 || dp == 20 || dp == 24 || dp == 40 || dp == 48; }
+
+template <typename T, int LPR, int DP>
+int launch_padded_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    return a.G == 1 ? launch_padded<T, LPR, DP, 1>(a, fr, st) : launch_padded<T, LPR, DP, 4>(a, fr, st);
+}
+
+template <typename T>
+int launch_padded_dp(int dp, const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    switch (dp) {
+        case 10: return launch_padded_gt<T, 16, 10>(a, fr, st);
+        case 12: return launch_padded_gt<T, 16, 12>(a, fr, st);
+        case 20: return launch_padded_gt<T, 32, 20>(a, fr, st);
+        case 24: return launch_padded_gt<T, 32, 24>(a, fr, st);
+        case 40: return launch_padded_gt<T, 64, 40>(a, fr, st);
+        case 48: return launch_padded_gt<T, 64, 48>(a, fr, st);
+        default: return ONELLM_EUNSUPPORTED;
+    }
+}
+
 template <typename T, int LPR, int GT>
 int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
@@ -1284,10 +1337,12 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     const int esz = dtype == ONELLM_FP16 ? 2 : 4;
     const int row_bytes = D * esz;
     if (D > 2 * kMaxPairs || B > 65535) return ONELLM_EUNSUPPORTED;
-    // rows of a power-of-two number of bytes in 16-byte aligned caches take the tiled kernels; any
-    // other head size or alignment takes the scalar kernel
-    const bool tiled = row_bytes >= 16 && row_bytes <= 1024 && !(row_bytes & (row_bytes - 1)) && aligned16(k_cache)
-                       && aligned16(v_cache);
+    // rows of a power-of-two number of bytes - or of 10, 12, 20, 24, 40 or 48 16-byte pieces (head sizes 80, 96,
+    // 160, 192, ... in fp16) - in 16-byte aligned caches take the tiled kernels; any other head size or alignment
+    // takes the scalar kernel
+    const bool padded = row_bytes % 16 == 0 && padded_pieces(row_bytes / 16);
+    const bool tiled = row_bytes >= 16 && row_bytes <= 1024 && (!(row_bytes & (row_bytes - 1)) || padded)
+                       && aligned16(k_cache) && aligned16(v_cache);
     const int lpr = row_bytes / 16;
 
     AttnArgs a{};
@@ -1311,7 +1366,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // needs no merge pass.  Per-sequence lengths: finer chunks (about 16 workgroups per compute unit,
     // at least 256 rows each) so that the dispatcher can balance ragged work.
     const int G = a.G;
-    const int gt = heads_per_tile(dtype == ONELLM_FP16, D, G);
+    const int gt = padded ? (G == 1 ? 1 : 4) : heads_per_tile(dtype == ONELLM_FP16, D, G);
     const int ngt = (G + gt - 1) / gt;
     const long base_wgs = (long)B * Hkv * ngt;
     const int user_target = tune_get("attn_target_wgs");
@@ -1351,7 +1406,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
                               && (size_t)B * nunits * sizeof(int) <= kCounterBytes;
     float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + counter_bytes);
     const int bal = tune_get("attn_balanced");
-    if (forced <= 0 && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, dtype == ONELLM_FP16 && G > 1 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1, (long)B * nunits)))) {
+    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, dtype == ONELLM_FP16 && G > 1 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1, (long)B * nunits)))) {
         a.item_rows = item_rows_for(dtype == ONELLM_FP16, D, G);
         const long long items = (max_t - 1 + a.item_rows - 1) / a.item_rows;
         const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);
@@ -1389,7 +1444,9 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     fill_rope_freqs(fr, D, rotary_dim, rope_base);
 
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int rc = dtype == ONELLM_FP16 ? launch_lpr<__half>(lpr, a, fr, st) : launch_lpr<float>(lpr, a, fr, st);
+    int rc;
+    if (padded) rc = dtype == ONELLM_FP16 ? launch_padded_dp<__half>(lpr, a, fr, st) : launch_padded_dp<float>(lpr, a, fr, st);
+    else rc = dtype == ONELLM_FP16 ? launch_lpr<__half>(lpr, a, fr, st) : launch_lpr<float>(lpr, a, fr, st);
     if (rc != 0) return rc;
     if (merge_needed) {
         if (a.bal_nwg > 0) {

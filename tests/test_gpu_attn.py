@@ -92,6 +92,10 @@ def test_example_driver_shape_two_layers(capi, ref, dev):
     (np.float16, 3, 1, 128), (np.float16, 12, 2, 256), (np.float16, 2, 2, 8), (np.float16, 4, 2, 16), (np.float16, 2, 1, 512),
     (np.float32, 4, 4, 128), (np.float32, 8, 2, 64), (np.float32, 3, 1, 32), (np.float32, 2, 2, 256),
     (np.float32, 4, 1, 4), (np.float32, 10, 2, 16),
+    # rows of 10, 12, 20, 24, 40 or 48 16-byte pieces: the tiled kernel with idle lanes in every row group
+    (np.float16, 4, 2, 96), (np.float16, 8, 8, 80), (np.float16, 6, 2, 160), (np.float16, 4, 1, 192), (np.float16, 2, 2, 320),
+    (np.float16, 3, 1, 384), (np.float32, 4, 2, 40), (np.float32, 5, 5, 48), (np.float32, 8, 2, 80), (np.float32, 2, 1, 96),
+    (np.float32, 2, 2, 160), (np.float32, 6, 1, 192),
 ])
 @pytest.mark.parametrize("t", [1, 2, 63, 64, 65, 300])
 def test_shapes_and_lengths(capi, ref, dev, dtype, Hq, Hkv, D, t):
@@ -100,12 +104,13 @@ def test_shapes_and_lengths(capi, ref, dev, dtype, Hq, Hkv, D, t):
     _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), dtype)
 
 
-@pytest.mark.parametrize("dtype,Hq,Hkv,D", [(np.float16, 4, 2, 96), (np.float16, 8, 8, 80), (np.float32, 2, 1, 7),
+@pytest.mark.parametrize("dtype,Hq,Hkv,D", [(np.float16, 4, 2, 72), (np.float16, 8, 8, 100), (np.float32, 2, 1, 7),
                                             (np.float32, 3, 3, 100), (np.float16, 2, 1, 2), (np.float32, 2, 2, 1),
-                                            (np.float16, 2, 1, 500)])
+                                            (np.float16, 2, 1, 500), (np.float16, 2, 2, 112)])
 @pytest.mark.parametrize("t", [1, 2, 70])
 def test_head_sizes_outside_the_tiled_kernels(capi, ref, dev, dtype, Hq, Hkv, D, t):
-    # rows that are not a power-of-two number of bytes run the scalar kernel: same parity bars
+    # rows the tiled kernels are not built for (not a whole number of 16-byte pieces, or a piece count outside
+    # their list) run the scalar kernel: same parity bars
     announce("attn generic", dtype.__name__, Hq, Hkv, D, "t", t)
     qkv, bias, kc, vc = _case(dtype, 2, Hq, Hkv, D, 72, 2, seed=D * 7 + t, std=0.5)
     _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D, layer=1), dtype)
@@ -387,12 +392,12 @@ def test_fused_finish_at_full_size_matches_the_merge_launch(capi, dev):
 
 
 def test_random_shapes_sweep(capi, ref, dev):
-    """Sixty seeded random (dtype, heads, group size, head size, lengths, split count, schedule) combinations, ragged lengths
+    """Eighty seeded random (dtype, heads, group size, head size, lengths, split count, schedule) combinations, ragged lengths
     included: every kernel variant and padded head tile gets shapes nobody picked by hand."""
     rng = np.random.default_rng(2024)
-    for case in range(60):
+    for case in range(80):
         dtype = [np.float16, np.float32][int(rng.integers(0, 2))]
-        D = int(rng.choice([16, 32, 64, 128, 128, 128, 256]))
+        D = int(rng.choice([16, 32, 64, 128, 128, 128, 256, 96, 80, 192]))
         Hkv = int(rng.integers(1, 4))
         G = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 20]))
         Hq = Hkv * G
