@@ -105,6 +105,34 @@ def test_launchDecoderMaskedMHA(H, ref, dev, dtype, five_d):
 
 
 @pytest.mark.gpu
+def test_launchDecoderMaskedMHA_with_a_sequence_split(H, ref, dev):
+    """One or two sequences with a long history: the entry point splits the sequence, the launcher creates its
+    zero-filled workspace and the pieces are merged inside the attention kernel.  Several steps of different lengths
+    reuse that workspace."""
+    import torch
+    rng = np.random.default_rng(7)
+    B, Hq, Hkv, D, S = 2, 8, 2, 128, 1100
+    qkv = (rng.standard_normal((B, Hq + 2 * Hkv, D)) * 0.5).astype(np.float16)
+    bias = (rng.standard_normal((Hq + 2 * Hkv) * D) * 0.5).astype(np.float16)
+    kc = (rng.standard_normal((1, B, Hkv, S, D)) * 0.5).astype(np.float16)
+    vc = (rng.standard_normal((1, B, Hkv, S, D)) * 0.5).astype(np.float16)
+    d_qkv, d_bias = _dev(qkv, dev), _dev(bias, dev)
+    for t in (1000, 300, 1100, 129, 1000):
+        announce("launchDecoderMaskedMHA split, step", t)
+        d_kc, d_vc = _dev(kc, dev), _dev(vc, dev)
+        out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+        rc = H.h_decode_mha(1, d_qkv.data_ptr(), d_bias.data_ptr(), d_kc.data_ptr(), d_vc.data_ptr(), out.data_ptr(),
+                            B, Hq, Hkv, D, S, 1, t, 0, D, 10000.0)
+        assert rc == 0, H.h_last_error()
+        assert H.h_sync_and_check() == 0, H.h_last_error()
+        r_kc, r_vc = kc.copy(), vc.copy()
+        want = ref.decode_attn(qkv, bias, r_kc, r_vc, Hq, t, D, 10000.0)
+        np.testing.assert_allclose(out.cpu().numpy().astype(np.float64), want.astype(np.float64), rtol=1e-2, atol=2e-3)
+        np.testing.assert_array_equal(d_kc.cpu().numpy().view(np.uint16), r_kc.view(np.uint16))
+        np.testing.assert_array_equal(d_vc.cpu().numpy().view(np.uint16), r_vc.view(np.uint16))
+
+
+@pytest.mark.gpu
 def test_launchRMSNorm_and_fused_norm(H, ref, dev):
     import torch
     announce("launchRMSNorm / launchFusedAddBiasResidualRMSNorm")
