@@ -32,6 +32,18 @@ __device__ __forceinline__ Key make_key(float v, int id)
 }
 __device__ __forceinline__ int key_id(Key k) { return k == 0 ? -1 : (int)(0xFFFFFFFFu - (unsigned)(k & 0xFFFFFFFFu)); }
 
+// The value a key was made from.  The key's high word is an invertible map of the float's bits, except that -0 was
+// folded onto +0: a zero is therefore read back from the logits (the stored bits must be the input's bits); every
+// other value is decoded from the key, which spares the kernels a dependent memory round trip before their stores.
+__device__ __forceinline__ float key_value(Key k, int id, const float* __restrict__ logits)
+{
+    if (id < 0) return -INFINITY;
+    unsigned u = (unsigned)(k >> 32);
+    u ^= (u & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu;
+    const float v = __uint_as_float(u);
+    return v == 0.0f ? logits[id] : v;
+}
+
 __device__ __forceinline__ void cmp_exchange(Key& hi, Key& lo)
 {
     const bool sw = lo > hi;
@@ -184,7 +196,7 @@ void topk_stage1_kernel(const float* __restrict__ logits, int V, int nblk, int v
         for (int i = 0; i < KP; ++i) {
             if (i < K) {
                 const int id = key_id(t.k[i]);
-                vals[(size_t)blockIdx.x * K + i] = id < 0 ? -INFINITY : logits[id];
+                vals[(size_t)blockIdx.x * K + i] = key_value(t.k[i], id, logits);
                 ids[(size_t)blockIdx.x * K + i] = id;
             }
         }
@@ -211,7 +223,7 @@ void topk_stage2_kernel(const float* __restrict__ logits, const float* __restric
         for (int i = 0; i < KP; ++i) {
             if (i < K) {
                 const int id = key_id(t.k[i]);
-                fvals[(size_t)b * K + i] = id < 0 ? -INFINITY : logits[id];
+                fvals[(size_t)b * K + i] = key_value(t.k[i], id, logits);
                 fids[(size_t)b * K + i] = id;
             }
         }

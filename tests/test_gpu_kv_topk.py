@@ -163,3 +163,25 @@ def test_topk_negative_infinity_and_run_to_run(capi, ref, dev):
     a = fi.clone()
     _, _, _, _, fi2 = capi.beam_topk(d, 1, 2, 4)
     assert torch.equal(a, fi2)
+
+
+def test_topk_zeros_of_both_signs_and_extreme_values(capi, ref, dev):
+    """-0.0 and +0.0 tie (the lower index wins) and every stored value carries the bits of the input it came from:
+    zeros keep their sign, denormals, the largest finite value and infinities come back unchanged."""
+    announce("topk signed zeros and extreme values")
+    B, beam, V, K = 2, 2, 600, 4
+    logits = -np.abs(np.random.default_rng(17).standard_normal((B * beam, V)).astype(np.float32)) - 1.0
+    logits[0, [5, 300, 599]] = [-0.0, 0.0, -0.0]                 # three zeros on top: indices 5, 300, 599 in this order
+    logits[1, [7, 8]] = [0.0, -0.0]
+    logits[2, [1, 2, 3, 4]] = [np.float32(1e-45), np.float32(-1e-45), np.finfo(np.float32).max, np.inf]
+    logits[3, [10, 11]] = [np.finfo(np.float32).tiny, -np.inf]
+    _, v1, i1, fv, fi = capi.beam_topk(torch.from_numpy(logits).to(dev), B, beam, K)
+    w1v, w1i, wfv, wfi = ref.beam_topk(logits, B, beam, K)
+    np.testing.assert_array_equal(i1.cpu().numpy(), w1i)
+    np.testing.assert_array_equal(v1.cpu().numpy().view(np.uint32), w1v.view(np.uint32))
+    np.testing.assert_array_equal(fi.cpu().numpy(), wfi)
+    np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), wfv.view(np.uint32))
+    got_i, got_v = fi.cpu().numpy(), fv.cpu().numpy()
+    np.testing.assert_array_equal(got_i[0], [5, 300, 599, V + 7])
+    flat = logits.reshape(-1)
+    np.testing.assert_array_equal(got_v.view(np.uint32), flat[got_i].view(np.uint32))   # the input's own bits
