@@ -895,6 +895,188 @@ int launch_gqa_mfma(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     return launch_status();
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same for fp32 caches (D = 128, more than four query heads per kv head): both products on
+// v_mfma_f32_16x16x4_f32, every operand an fp32 register exactly as loaded - no splitting, no
+// packing.  A K load register of lane (slot, grp) holds four columns of row `slot`; each of them is
+// the A operand of one product (k = grp); q sits in 32 B-operand registers (column by column, the GT
+// heads repeated over the 16 tile columns).  The score tile leaves lane (slot, grp) with rows
+// 4*grp + {0..3} of head slot % GT, and score register r is the A operand of output product r
+// (k = grp <-> row 4*grp + r), against V loaded as rows 4*grp + {0..3}, four columns per lane.
+// 64 products of 32 cycles per 16 rows (16 KiB of K and V): about a third of what the memory stream
+// leaves per SIMD.  One register buffer (two would leave one wave per SIMD).
+template <int GT, int NW>
+__device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds)
+{
+    using T = float;
+    static_assert(GT == 8 || GT == 16, "heads per tile");
+    constexpr int D = 128, VEC = 4;
+    constexpr int NKJ = D / VEC / 4;            // 16-byte pieces of a K row per lane: 8
+    constexpr int CG = D / (16 * VEC);          // groups of 64 output columns (16 lanes x 4): 2
+    constexpr int NTHR = NW * kWave;
+    constexpr int RPI = NW * 16;                // rows per workgroup iteration
+
+    float* sq = lds;                            // [GT][D]
+    float* sk = sq + GT * D;                    // [D]
+    float* sv = sk + D;                         // [D]
+    float* snew = sv + D;                       // [GT]
+    float* st_ml = snew + GT;                   // [NW][GT][2]
+    float* st_acc = st_ml + NW * GT * 2;        // [NW][GT][D]
+
+    const int tid = lane_id_per_unit();
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int slot = lane & 15;
+    const int grp = lane >> 4;
+    const int r0 = u.r0, r1 = u.r1;
+    const size_t head_off = a.slab + ((size_t)u.b * a.Hkv + u.kvh) * (size_t)a.S * D;
+    T* kc = static_cast<T*>(a.k_cache) + head_off;
+    T* vc = static_cast<T*>(a.v_cache) + head_off;
+    // K: lane (slot, grp) holds row `slot` of the batch, pieces grp + 4*j (columns (grp + 4*j)*4 ..)
+    // V: lane (slot, grp) holds rows 4*grp + e of the batch, columns (cg*16 + slot)*4 .. +3
+    const T* kp = kc + (size_t)(wave * 16 + slot) * D + grp * VEC;
+    const T* vp = vc + (size_t)(wave * 16 + 4 * grp) * D + slot * VEC;
+
+    auto issue = [&](Vec16<T> (&kv)[NKJ], Vec16<T> (&vv)[CG * 4], int rbase) {
+#pragma unroll
+        for (int j = 0; j < NKJ; ++j) kv[j] = load16_stream(kp + (size_t)rbase * D + j * 16);
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vv[cg * 4 + e] = load16_stream(vp + (size_t)(rbase + e) * D + cg * 64);
+    };
+    const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
+    Vec16<T> ka[NKJ], va[CG * 4];
+    if (nfull > 0) issue(ka, va, r0);
+
+    stage_q_and_new_row<T, D, GT, NTHR>(a, fr, u, kc, vc, sq, sk, sv, snew);
+
+    // B operand of the score products: column (lane % 16) is head (lane % GT); product (j, e) reduces
+    // over the columns (grp + 4*j)*4 + e, grp = 0..3 - the ones the K registers hold there
+    float qb[NKJ][VEC];
+    {
+        const float* qh = sq + (lane % GT) * D + grp * VEC;
+#pragma unroll
+        for (int j = 0; j < NKJ; ++j)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) qb[j][e] = qh[j * 16 + e];
+    }
+
+    float m = -INFINITY, l = 0.f;               // per lane: head lane % GT; l is this lane's share
+    f32x4 o[CG * VEC];                          // o[cg*4 + c][r]: head (4*grp + r) % GT, column (cg*16 + slot)*4 + c
+#pragma unroll
+    for (int c = 0; c < CG * VEC; ++c) o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto consume = [&](const Vec16<T> (&kv)[NKJ], const Vec16<T> (&vv)[CG * 4], int rbase, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < NKJ; ++j)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[j].raw[e], qb[j][e], sc, 0, 0, 0);
+        float s[4];
+        float bm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s[r] = sc[r];                       // score of row 4*grp + r of the batch, head lane % GT
+            if constexpr (MASKED) s[r] = (rbase + wave * 16 + 4 * grp + r < r1) ? s[r] : -INFINITY;
+            bm = fmaxf(bm, s[r]);
+        }
+        if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+            bm = fmaxf(bm, __shfl_xor(bm, 16, kWave));
+            bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
+            const float mnew = fmaxf(m, bm);    // finite: some row of the batch is valid
+            const float alpha = __builtin_amdgcn_exp2f(m - mnew);
+            l *= alpha;
+            float al[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, (lane & 48) | ((4 * grp + r) % GT), kWave);
+#pragma unroll
+            for (int c = 0; c < CG * VEC; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[c][r] *= al[r];
+            m = mnew;
+        }
+        float p[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            p[r] = __builtin_amdgcn_exp2f(s[r] - m);
+            l += p[r];
+        }
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+            for (int c = 0; c < VEC; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    o[cg * VEC + c] = __builtin_amdgcn_mfma_f32_16x16x4f32(p[r], vv[cg * 4 + r].raw[c], o[cg * VEC + c], 0, 0, 0);
+    };
+
+    if (r1 > r0) {
+        int rbase = r0;
+        // one register buffer: the other waves of the compute unit cover the load latency
+        for (int it = 0; it < nfull; ++it) {
+            consume(ka, va, rbase, std::false_type{});
+            rbase += RPI;
+            if (it + 1 < nfull) issue(ka, va, rbase);
+        }
+        rbase = r0 + nfull * RPI;
+        if (rbase < r1) {
+            // partial batch: rows past the end are read from the last valid row and masked
+            const int krow = min(rbase + wave * 16 + slot, r1 - 1);
+#pragma unroll
+            for (int j = 0; j < NKJ; ++j) ka[j] = load16_stream(kc + (size_t)krow * D + grp * VEC + j * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int vrow = min(rbase + wave * 16 + 4 * grp + e, r1 - 1);
+#pragma unroll
+                for (int cg = 0; cg < CG; ++cg) va[cg * 4 + e] = load16_stream(vc + (size_t)vrow * D + slot * VEC + cg * 64);
+            }
+            if (rbase + wave * 16 < r1) consume(ka, va, rbase, std::true_type{});
+        }
+    }
+
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (grp == 0 && slot < GT) {
+        st_ml[(wave * GT + slot) * 2] = m;
+        st_ml[(wave * GT + slot) * 2 + 1] = l;
+    }
+    if (4 * grp < GT) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+                for (int c = 0; c < VEC; ++c)
+                    st_acc[(size_t)(wave * GT + 4 * grp + r) * D + (cg * 16 + slot) * VEC + c] = o[cg * VEC + c][r];
+    }
+    __syncthreads();
+    finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv);
+}
+
+template <int GT, int NW, bool BALANCED>
+__global__ __launch_bounds__(NW * kWave)
+void decode_attn_gqa_mfma_f32_kernel(const AttnArgs a, const RopeFreqs fr)
+{
+    extern __shared__ float lds[];
+    for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_f32_unit<GT, NW>(a, fr, u, lds); });
+}
+
+template <int GT>
+int launch_gqa_mfma_f32(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
+{
+    constexpr int NW = 4, D = 128;
+    const size_t lds_bytes = sizeof(float) * (size_t)(GT * D + 2 * D + GT + NW * GT * 2 + NW * GT * D);
+    const int ngt = (a.G + GT - 1) / GT;
+    const dim3 grid(a.Hkv * ngt, a.nsplit, a.B), block(NW * kWave);
+    if (a.bal_nwg > 0)
+        hipLaunchKernelGGL((decode_attn_gqa_mfma_f32_kernel<GT, NW, true>), dim3(a.bal_nwg), block, lds_bytes, st, a, fr);
+    else
+        hipLaunchKernelGGL((decode_attn_gqa_mfma_f32_kernel<GT, NW, false>), grid, block, lds_bytes, st, a, fr);
+    return launch_status();
+}
+
 // Merge the per-split partial states of one (sequence, query head) and normalise: one wave per
 // (sequence, head).  Lane s holds split s's (m, l), so the maximum, the weights and the denominator
 // are two wave reductions instead of loops of dependent loads; the weighted sum over splits then
@@ -1213,13 +1395,21 @@ int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 // head sizes the matrix-core kernel is built for (fp16 caches)
 constexpr bool mfma_head_size(int D) { return D == 64 || D == 128 || D == 256; }
 
+// shapes that run on the matrix cores: fp16 caches with two or more query heads per kv head at those head
+// sizes; fp32 caches at D = 128 with more than four (up to four the vector ALU keeps up with the stream)
+bool on_matrix_cores(bool fp16, int D, int G)
+{
+    if (tune_get("attn_gqa_valu") == 1) return false;
+    return fp16 ? (G > 1 && mfma_head_size(D)) : (G > 4 && D == 128);
+}
+
 // query heads one workgroup serves (they share every K/V row it reads)
 int heads_per_tile(bool fp16, int D, int G)
 {
     if (G == 1) return 1;       // one head: memory-bound on either kernel (measured equal), keep the lighter one
     // two or more query heads per kv head, fp16: both products on the matrix cores, where up to 16
     // heads cost the same as 4 (8 at D = 256: the per-wave states of 16 heads would not fit 64 KiB of LDS)
-    if (fp16 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1) {
+    if (on_matrix_cores(fp16, D, G)) {
         const int cap = D == 256 ? 8 : 16;
         const int gt = G <= 4 ? 4 : (G <= 8 ? 8 : 16);
         return gt < cap ? gt : cap;
@@ -1236,8 +1426,11 @@ int launch_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     constexpr bool kHalf = std::is_same<T, __half>::value;
     constexpr int D = LPR * Elt<T>::kVec;
     const int gt = heads_per_tile(kHalf, D, a.G);
+    if constexpr (!kHalf && D == 128) {
+        if (on_matrix_cores(false, D, a.G)) return gt == 8 ? launch_gqa_mfma_f32<8>(a, fr, st) : launch_gqa_mfma_f32<16>(a, fr, st);
+    }
     if constexpr (kHalf && mfma_head_size(D)) {
-        if (a.G > 1 && tune_get("attn_gqa_valu") != 1) {
+        if (on_matrix_cores(true, D, a.G)) {
             switch (gt) {
                 case 4: return launch_gqa_mfma<D, 4>(a, fr, st);
                 case 8: return launch_gqa_mfma<D, 8>(a, fr, st);
@@ -1280,7 +1473,7 @@ constexpr int kBalancedWorkgroups = 512;   // two 4-wave workgroups per compute 
 // rows per work item of the balanced schedule: one workgroup iteration of the kernel that runs
 int item_rows_for(bool fp16, int D, int G)
 {
-    if (G > 1 && fp16 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1) return 64;
+    if (on_matrix_cores(fp16, D, G)) return 64;
     const int lpr = D * (fp16 ? 2 : 4) / 16;
     const int rpi = 1024 / lpr;               // 4 waves x (64 / lpr) rows x 4 per row group
     return rpi < 64 ? 64 : rpi;
@@ -1406,7 +1599,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
                               && (size_t)B * nunits * sizeof(int) <= kCounterBytes;
     float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + counter_bytes);
     const int bal = tune_get("attn_balanced");
-    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, dtype == ONELLM_FP16 && G > 1 && mfma_head_size(D) && tune_get("attn_gqa_valu") != 1, (long)B * nunits)))) {
+    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, on_matrix_cores(dtype == ONELLM_FP16, D, G), (long)B * nunits)))) {
         a.item_rows = item_rows_for(dtype == ONELLM_FP16, D, G);
         const long long items = (max_t - 1 + a.item_rows - 1) / a.item_rows;
         const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);

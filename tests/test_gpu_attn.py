@@ -91,7 +91,7 @@ def test_example_driver_shape_two_layers(capi, ref, dev):
     (np.float16, 16, 2, 128), (np.float16, 14, 2, 128), (np.float16, 16, 1, 128), (np.float16, 40, 2, 128),
     (np.float16, 3, 1, 128), (np.float16, 12, 2, 256), (np.float16, 2, 2, 8), (np.float16, 4, 2, 16), (np.float16, 2, 1, 512),
     (np.float32, 4, 4, 128), (np.float32, 8, 2, 64), (np.float32, 3, 1, 32), (np.float32, 2, 2, 256),
-    (np.float32, 4, 1, 4), (np.float32, 10, 2, 16),
+    (np.float32, 4, 1, 4), (np.float32, 10, 2, 16), (np.float32, 16, 2, 128), (np.float32, 12, 1, 128), (np.float32, 40, 2, 128),
     # rows of 10, 12, 20, 24, 40 or 48 16-byte pieces: the tiled kernel with idle lanes in every row group
     (np.float16, 4, 2, 96), (np.float16, 8, 8, 80), (np.float16, 6, 2, 160), (np.float16, 4, 1, 192), (np.float16, 2, 2, 320),
     (np.float16, 3, 1, 384), (np.float32, 4, 2, 40), (np.float32, 5, 5, 48), (np.float32, 8, 2, 80), (np.float32, 2, 1, 96),
@@ -259,27 +259,29 @@ def test_constant_value_rows_at_full_size(capi, dev):
     assert (out.float() - 0.375).abs().max().item() <= 1e-3
 
 
-@pytest.mark.parametrize("D,Hq", [(128, 8), (64, 8), (256, 8), (64, 32), (256, 12)])
-def test_options_on_the_matrix_core_kernel(capi, ref, dev, D, Hq):
-    """The same option matrix as test_options on shapes that take the MFMA grouped-query kernel (fp16, head size 64,
-    128 or 256, 4 / 6 / 16 query heads per kv head), with one and with several sequence splits."""
-    announce("attn options, mfma kernel", D, Hq)
-    qkv, bias, kc, vc = _case(np.float16, 2, Hq, 2, D, 200, 2, seed=23 + D, std=0.5)
+@pytest.mark.parametrize("D,Hq,dtype", [(128, 8, np.float16), (64, 8, np.float16), (256, 8, np.float16), (64, 32, np.float16),
+                                        (256, 12, np.float16), (128, 16, np.float32), (128, 24, np.float32), (128, 40, np.float32)])
+def test_options_on_the_matrix_core_kernel(capi, ref, dev, D, Hq, dtype):
+    """The same option matrix as test_options on shapes that take the MFMA grouped-query kernels (fp16: head size 64,
+    128 or 256, 4 / 6 / 16 query heads per kv head; fp32: head size 128, 8 / 12 / 20 heads per kv head), with one and
+    with several sequence splits."""
+    announce("attn options, mfma kernel", D, Hq, dtype.__name__)
+    qkv, bias, kc, vc = _case(dtype, 2, Hq, 2, D, 200, 2, seed=23 + D, std=0.5)
     for nsplit in (-1, 3):
         capi.tune_set("attn_nsplit", nsplit)
         try:
-            _assert_parity(_run_both(capi, ref, dev, qkv, None, kc, vc, Hq, 177, D, layer=1), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, 0), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D // 2), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, pos_offset=-1, layer=1), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, base=500000.0), np.float16)
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, flags=capi.ATTN_NO_V_BIAS), np.float16)
+            _assert_parity(_run_both(capi, ref, dev, qkv, None, kc, vc, Hq, 177, D, layer=1), dtype)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, 0), dtype)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D // 2), dtype)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, pos_offset=-1, layer=1), dtype)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, base=500000.0), dtype)
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, flags=capi.ATTN_NO_V_BIAS), dtype)
             res = _run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 177, D, flags=capi.ATTN_NO_CACHE_WRITE)
-            _assert_parity(res, np.float16)
+            _assert_parity(res, dtype)
             np.testing.assert_array_equal(_bits(res[2]), _bits(kc))
-            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 200, D), np.float16)       # t == S
+            _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, 200, D), dtype)       # t == S
             for t in (1, 2, 16, 17, 63, 65):                                                           # short and partial batches
-                _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), np.float16)
+                _assert_parity(_run_both(capi, ref, dev, qkv, bias, kc, vc, Hq, t, D), dtype)
         finally:
             capi.tune_set("attn_nsplit", -1)
 
