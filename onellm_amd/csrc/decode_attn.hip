@@ -896,7 +896,7 @@ int launch_gqa_mfma(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 }
 
 // ---------------------------------------------------------------------------------------------
-// The same for fp32 caches (D = 128, more than four query heads per kv head): both products on
+// The same for fp32 caches (D = 64 or 128, more than four query heads per kv head): both products on
 // v_mfma_f32_16x16x4_f32, every operand an fp32 register exactly as loaded - no splitting, no
 // packing.  A K load register of lane (slot, grp) holds four columns of row `slot`; each of them is
 // the A operand of one product (k = grp); q sits in 32 B-operand registers (column by column, the GT
@@ -905,12 +905,13 @@ int launch_gqa_mfma(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 // (k = grp <-> row 4*grp + r), against V loaded as rows 4*grp + {0..3}, four columns per lane.
 // 64 products of 32 cycles per 16 rows (16 KiB of K and V): about a third of what the memory stream
 // leaves per SIMD.  One register buffer (two would leave one wave per SIMD).
-template <int GT, int NW>
+template <int D, int GT, int NW>
 __device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds)
 {
     using T = float;
     static_assert(GT == 8 || GT == 16, "heads per tile");
-    constexpr int D = 128, VEC = 4;
+    static_assert(D == 64 || D == 128, "head size");
+    constexpr int VEC = 4;
     constexpr int NKJ = D / VEC / 4;            // 16-byte pieces of a K row per lane: 8
     constexpr int CG = D / (16 * VEC);          // groups of 64 output columns (16 lanes x 4): 2
     constexpr int NTHR = NW * kWave;
@@ -1055,25 +1056,25 @@ __device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeF
     finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv);
 }
 
-template <int GT, int NW, bool BALANCED>
+template <int D, int GT, int NW, bool BALANCED>
 __global__ __launch_bounds__(NW * kWave)
 void decode_attn_gqa_mfma_f32_kernel(const AttnArgs a, const RopeFreqs fr)
 {
     extern __shared__ float lds[];
-    for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_f32_unit<GT, NW>(a, fr, u, lds); });
+    for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_f32_unit<D, GT, NW>(a, fr, u, lds); });
 }
 
-template <int GT>
+template <int D, int GT>
 int launch_gqa_mfma_f32(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
-    constexpr int NW = 4, D = 128;
+    constexpr int NW = 4;
     const size_t lds_bytes = sizeof(float) * (size_t)(GT * D + 2 * D + GT + NW * GT * 2 + NW * GT * D);
     const int ngt = (a.G + GT - 1) / GT;
     const dim3 grid(a.Hkv * ngt, a.nsplit, a.B), block(NW * kWave);
     if (a.bal_nwg > 0)
-        hipLaunchKernelGGL((decode_attn_gqa_mfma_f32_kernel<GT, NW, true>), dim3(a.bal_nwg), block, lds_bytes, st, a, fr);
+        hipLaunchKernelGGL((decode_attn_gqa_mfma_f32_kernel<D, GT, NW, true>), dim3(a.bal_nwg), block, lds_bytes, st, a, fr);
     else
-        hipLaunchKernelGGL((decode_attn_gqa_mfma_f32_kernel<GT, NW, false>), grid, block, lds_bytes, st, a, fr);
+        hipLaunchKernelGGL((decode_attn_gqa_mfma_f32_kernel<D, GT, NW, false>), grid, block, lds_bytes, st, a, fr);
     return launch_status();
 }
 
@@ -1396,11 +1397,11 @@ int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 constexpr bool mfma_head_size(int D) { return D == 64 || D == 128 || D == 256; }
 
 // shapes that run on the matrix cores: fp16 caches with two or more query heads per kv head at those head
-// sizes; fp32 caches at D = 128 with more than four (up to four the vector ALU keeps up with the stream)
+// sizes; fp32 caches at D = 64 or 128 with more than four (up to four the vector ALU keeps up with the stream)
 bool on_matrix_cores(bool fp16, int D, int G)
 {
     if (tune_get("attn_gqa_valu") == 1) return false;
-    return fp16 ? (G > 1 && mfma_head_size(D)) : (G > 4 && D == 128);
+    return fp16 ? (G > 1 && mfma_head_size(D)) : (G > 4 && (D == 128 || D == 64));
 }
 
 // query heads one workgroup serves (they share every K/V row it reads)
@@ -1426,8 +1427,8 @@ int launch_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     constexpr bool kHalf = std::is_same<T, __half>::value;
     constexpr int D = LPR * Elt<T>::kVec;
     const int gt = heads_per_tile(kHalf, D, a.G);
-    if constexpr (!kHalf && D == 128) {
-        if (on_matrix_cores(false, D, a.G)) return gt == 8 ? launch_gqa_mfma_f32<8>(a, fr, st) : launch_gqa_mfma_f32<16>(a, fr, st);
+    if constexpr (!kHalf && (D == 128 || D == 64)) {
+        if (on_matrix_cores(false, D, a.G)) return gt == 8 ? launch_gqa_mfma_f32<D, 8>(a, fr, st) : launch_gqa_mfma_f32<D, 16>(a, fr, st);
     }
     if constexpr (kHalf && mfma_head_size(D)) {
         if (on_matrix_cores(true, D, a.G)) {

@@ -260,7 +260,7 @@ def test_constant_value_rows_at_full_size(capi, dev):
 
 
 @pytest.mark.parametrize("D,Hq,dtype", [(128, 8, np.float16), (64, 8, np.float16), (256, 8, np.float16), (64, 32, np.float16),
-                                        (256, 12, np.float16), (128, 16, np.float32), (128, 24, np.float32), (128, 40, np.float32)])
+                                        (256, 12, np.float16), (128, 16, np.float32), (128, 24, np.float32), (128, 40, np.float32), (64, 16, np.float32), (64, 34, np.float32)])
 def test_options_on_the_matrix_core_kernel(capi, ref, dev, D, Hq, dtype):
     """The same option matrix as test_options on shapes that take the MFMA grouped-query kernels (fp16: head size 64,
     128 or 256, 4 / 6 / 16 query heads per kv head; fp32: head size 128, 8 / 12 / 20 heads per kv head), with one and
