@@ -125,17 +125,18 @@ def entry(ms, nbytes, cpu_us=None):
     return e
 
 
-def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=None):
+def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=None, fp32=False):
     import torch
     torch.manual_seed(2)
+    dt = torch.float32 if fp32 else torch.float16
     sets = []
     for _ in range(nsets):
-        kc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
-        vc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+        kc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).to(dt)
+        vc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).to(dt)
         sets.append((kc, vc))
-    qkv = torch.randn(B, Hq + 2 * Hkv, D, device=dev).mul_(0.5).half()
-    bias = torch.randn((Hq + 2 * Hkv) * D, device=dev).mul_(0.5).half()
-    out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+    qkv = torch.randn(B, Hq + 2 * Hkv, D, device=dev).mul_(0.5).to(dt)
+    bias = torch.randn((Hq + 2 * Hkv) * D, device=dev).mul_(0.5).to(dt)
+    out = torch.zeros(B, Hq * D, dtype=dt, device=dev)
     max_t = t if t_dev is None else int(t_dev.max().item())
     # zero-filled once and declared so, as the launcher shim does with the workspace it owns: shapes whose sequences
     # are split are then finished inside the attention kernel instead of by a merge launch
@@ -342,6 +343,10 @@ def extras_section(capi, dev, args, with_cpu):
     ex["decode_attn_gqa_fused_b32_q32_kv8_len8192"] = entry(ms_u, attn_bytes(B3, Hq3, Hkv3, D, [S3] * B3, 2))
     ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, 16, 64, Hkv3, D, S3, S3, nsets=3)
     ex["decode_attn_gqa_fused_b16_q64_kv8_len8192"] = entry(ms_u, attn_bytes(16, 64, Hkv3, D, [S3] * 16, 2))
+    torch.cuda.empty_cache()
+    # the same 64-over-8 head shape with fp32 caches (the reference's own element type), batch 8 (the same bytes)
+    ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, 8, 64, Hkv3, D, S3, S3, nsets=3, fp32=True)
+    ex["decode_attn_gqa_fused_fp32_b8_q64_kv8_len8192"] = entry(ms_u, attn_bytes(8, 64, Hkv3, D, [S3] * 8, 4))
     torch.cuda.empty_cache()
     # the reference-style path on the same data: concat the new row, repeat KV to 32 heads, attend over 32 heads
     hist = (t_dev - 1).contiguous()
