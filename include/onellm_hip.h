@@ -46,7 +46,7 @@ extern "C" {
 
 typedef void* onellm_stream_t;
 
-/* Library/ABI version: major*1000 + minor. */
+/* Library/ABI version: major*1000 + minor (1001: ONELLM_ATTN_ZEROED_WORKSPACE and the larger attention workspace). */
 int onellm_hip_version(void);
 
 /* Human-readable text for any code returned by this library.  Never NULL. */

@@ -33,7 +33,8 @@ int tune_get(const char* key)
 
 }  // namespace onellm
 
-extern "C" int onellm_hip_version(void) { return 1000; }
+// 1.1: ONELLM_ATTN_ZEROED_WORKSPACE, 64 KiB of arrival counters at the front of the attention workspace
+extern "C" int onellm_hip_version(void) { return 1001; }
 
 extern "C" int onellm_tune_set(const char* key, int value)
 {
