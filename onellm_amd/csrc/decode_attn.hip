@@ -107,8 +107,9 @@ __device__ __forceinline__ bool locate_unit(const AttnArgs& a, Unit& u)
 // number of rows whatever the lengths are, crossing from one unit into the next where its share
 // does.  A unit seen whole by one workgroup is finished by it; otherwise each workgroup that
 // touches it leaves a partial state in entry (workgroup + global unit index) - unique, because
-// along the walk either the workgroup or the unit advances - and the merge kernel, which derives
-// the same boundaries from the same lengths, combines them.
+// along the walk either the workgroup or the unit advances - and whoever merges them (the merge
+// kernel, or the piece that arrives last when the finish is fused) derives the same boundaries from
+// the same lengths.
 __device__ __forceinline__ int seq_items(const AttnArgs& a, int t)
 {
     if (t < 1 || t > a.S) return 0;               // out-of-contract length: no work, nothing touched
@@ -202,7 +203,7 @@ __device__ __forceinline__ bool walk_begin(const AttnArgs& a, int nunits, Walk& 
     const long long target = w.cur / nunits;       // the sequence that holds item `cur` holds per-unit item `target`
     if (!a.t_dev) {
         w.items = seq_items(a, a.t_host);
-        w.b = (int)(target / w.items);
+        w.b = uniform((int)(target / w.items));
         w.base = (long long)w.b * w.items * nunits;
         return true;
     }
