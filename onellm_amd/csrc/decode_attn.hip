@@ -383,6 +383,44 @@ __device__ __forceinline__ float fetch(const float* p)
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The fused finish's last step: the piece that arrived last reads the states of all pieces of its unit
+// (device-scope loads, BATCH pieces in flight at a time) and writes the unit's output.
+template <typename T, int D, int GT, int NTHR, int BATCH>
+__device__ __forceinline__ void merge_pieces(const AttnArgs& a, const Unit& u, int tid)
+{
+    for (int i = tid; i < GT * D; i += NTHR) {
+        const int g = i / D, d = i % D;
+        if (u.g0 + g >= a.G) continue;
+        const size_t e0 = u.p0 + (size_t)g * u.pstride;
+        float M = -INFINITY, L = 0.f, O = 0.f;
+        for (int s0 = 0; s0 < u.npieces; s0 += BATCH) {
+            float mm[BATCH], ll[BATCH], oo[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const size_t e = e0 + (size_t)min(s0 + j, u.npieces - 1) * u.sstride;
+                mm[j] = fetch(a.part_ml + e * 2);
+                ll[j] = fetch(a.part_ml + e * 2 + 1);
+                oo[j] = fetch(a.part_o + e * D + d);
+            }
+            float bm = M;
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) bm = s0 + j < u.npieces ? fmaxf(bm, mm[j]) : bm;
+            const float keep = __builtin_amdgcn_exp2f(M - bm);   // every piece has a finite maximum
+            L *= keep;
+            O *= keep;
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const float wgt = s0 + j < u.npieces ? __builtin_amdgcn_exp2f(mm[j] - bm) : 0.f;
+                L = fmaf(ll[j], wgt, L);
+                O = fmaf(oo[j], wgt, O);
+            }
+            M = bm;
+        }
+        const int h = u.kvh * a.G + u.g0 + g;
+        static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + d] = from_f32<T>(O / L);
+    }
+}
+
 // Merge the NST softmax states the workgroup left in LDS (plus the new token's row in the last
 // split) and write either the output (single split) or this split's partial state.  The caller has
 // synchronised the workgroup on st_ml / st_acc / snew.
@@ -442,38 +480,12 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, fl
     __syncthreads();
     if (*arrived != u.npieces - 1) return;
     if (tid == 0) __hip_atomic_store(a.counters + u.counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
-    constexpr int BATCH = 16;                                   // pieces whose loads are in flight together
-    for (int i = tid; i < GT * D; i += NTHR) {
-        const int g = i / D, d = i % D;
-        if (u.g0 + g >= a.G) continue;
-        const size_t e0 = u.p0 + (size_t)g * u.pstride;
-        float M = -INFINITY, L = 0.f, O = 0.f;
-        for (int s0 = 0; s0 < u.npieces; s0 += BATCH) {
-            float mm[BATCH], ll[BATCH], oo[BATCH];
-#pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                const size_t e = e0 + (size_t)min(s0 + j, u.npieces - 1) * u.sstride;
-                mm[j] = fetch(a.part_ml + e * 2);
-                ll[j] = fetch(a.part_ml + e * 2 + 1);
-                oo[j] = fetch(a.part_o + e * D + d);
-            }
-            float bm = M;
-#pragma unroll
-            for (int j = 0; j < BATCH; ++j) bm = s0 + j < u.npieces ? fmaxf(bm, mm[j]) : bm;
-            const float keep = __builtin_amdgcn_exp2f(M - bm);   // every piece has a finite maximum
-            L *= keep;
-            O *= keep;
-#pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                const float wgt = s0 + j < u.npieces ? __builtin_amdgcn_exp2f(mm[j] - bm) : 0.f;
-                L = fmaf(ll[j], wgt, L);
-                O = fmaf(oo[j], wgt, O);
-            }
-            M = bm;
-        }
-        const int h = u.kvh * a.G + u.g0 + g;
-        static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + d] = from_f32<T>(O / L);
-    }
+    // (pieces whose loads are in flight together: 16 at most, no more than the unit has - most have two or three -
+    // rounded up to a power of two; the surplus slots of a batch repeat the last piece's loads)
+    if (u.npieces <= 2) merge_pieces<T, D, GT, NTHR, 2>(a, u, tid);
+    else if (u.npieces <= 4) merge_pieces<T, D, GT, NTHR, 4>(a, u, tid);
+    else if (u.npieces <= 8) merge_pieces<T, D, GT, NTHR, 8>(a, u, tid);
+    else merge_pieces<T, D, GT, NTHR, 16>(a, u, tid);
 }
 
 // DP = 16-byte pieces a cache row really has (D = DP * VEC); LPR = the lanes that share a row, the
