@@ -26,6 +26,11 @@
 namespace onellm {
 namespace {
 
+constexpr size_t kCounterBytes = 64 * 1024; // arrival counters of the fused finish: the first bytes of every workspace
+constexpr int kBalancedWorkgroups = 512;   // two 4-wave workgroups per compute unit: what the register budgets keep resident
+constexpr long long kBalancedMinItems = 3072;   // the balanced schedule is not the default for a smaller step
+constexpr long long kFusedGridMaxItems = 8192;  // per-sequence lengths on the grid schedule: fused finish up to this size
+
 struct AttnArgs {
     const void* qkv;
     const void* bias;
@@ -170,11 +175,18 @@ __device__ __forceinline__ int item_owner(long long x, long long W, int N)
     return (int)(((x + 1) * N - 1) / W);
 }
 
-// workgroups that take part: never more than there are items, so that no share is empty and the
-// workgroups of a unit are consecutive
+// Workgroups that take part: never more than there are items, so that no share is empty and the
+// workgroups of a unit are consecutive - and, as the host sizes the grid for the longest length it
+// was given while the real lengths may be much shorter: no workgroup for fewer than four items, and
+// not between one and two workgroups per compute unit (some units would get two shares, the rest one:
+// better one larger share each).  The launch has one workgroup per compute unit or two (or what a sweep
+// asked for, taken as it is).
 __device__ __forceinline__ int balanced_workgroups(const AttnArgs& a, long long W)
 {
-    return W < a.bal_nwg ? (int)W : a.bal_nwg;
+    long long n = (W + 3) / 4;
+    if (n > a.bal_nwg) n = a.bal_nwg;
+    if (a.bal_nwg == kBalancedWorkgroups && n > kBalancedWorkgroups / 2 && n < kBalancedWorkgroups) n = kBalancedWorkgroups / 2;
+    return (int)n;
 }
 
 struct Walk {
@@ -1481,8 +1493,6 @@ int launch_lpr(int lpr, const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
     }
 }
 
-constexpr size_t kCounterBytes = 64 * 1024; // arrival counters of the fused finish: the first bytes of every workspace
-constexpr int kBalancedWorkgroups = 512;   // two 4-wave workgroups per compute unit: what the register budgets keep resident
 
 // rows per work item of the balanced schedule: one workgroup iteration of the kernel that runs
 int item_rows_for(bool fp16, int D, int G)
@@ -1499,10 +1509,14 @@ int item_rows_for(bool fp16, int D, int G)
 // batch 16: 81 -> 57; batch 8, S 16384: 97 -> 61; D = 256, batch 16, S 4096: 90 -> 74.  With equal lengths the grid
 // schedule needs no merge launch and is as fast or faster; with more units than workgroups (batch 128) and on the
 // vector-ALU kernel (which keeps four workgroups per compute unit resident) the hardware dispatcher balances the
-// grid schedule's chunks as well as the fixed shares do.
-bool balanced_by_default(bool ragged, bool mfma, long units)
+// grid schedule's chunks as well as the fixed shares do.  Nor for a small step (fewer than kBalancedMinItems items
+// if every length were the longest): the walk's set-up and its serial unit changes are then most of the time and
+// the grid schedule with the fused finish is faster (8 sequences of 256..2048 rows: 24.9 against 17.6 us; 4 of
+// 512..4096: 25.2 / 19.6; even at 3500..4100 items; the balanced schedule is ahead from ~7000: 16 sequences of
+// 1024..8192 rows 56.7 / 67.6).
+bool balanced_by_default(bool ragged, bool mfma, long units, long long max_items)
 {
-    return ragged && mfma && units <= kBalancedWorkgroups;
+    return ragged && mfma && units <= kBalancedWorkgroups && max_items >= kBalancedMinItems;
 }
 
 int max_splits(int max_t)
@@ -1613,15 +1627,19 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
                               && (size_t)B * nunits * sizeof(int) <= kCounterBytes;
     float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + counter_bytes);
     const int bal = tune_get("attn_balanced");
-    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, on_matrix_cores(dtype == ONELLM_FP16, D, G), (long)B * nunits)))) {
-        a.item_rows = item_rows_for(dtype == ONELLM_FP16, D, G);
-        const long long items = (max_t - 1 + a.item_rows - 1) / a.item_rows;
-        const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);
+    // (the step's size in work items if every sequence had the longest length: all the host knows)
+    const int item_rows = item_rows_for(dtype == ONELLM_FP16, D, G);
+    const long long items = (max_t - 1 + item_rows - 1) / item_rows;
+    const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);
+    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, on_matrix_cores(dtype == ONELLM_FP16, D, G), (long)B * nunits, wmax)))) {
+        a.item_rows = item_rows;
         const int user_wgs = tune_get("attn_balanced_wgs");
         long long nwg = user_wgs > 0 ? user_wgs : kBalancedWorkgroups;
         if (nwg > kBalancedWorkgroups * 2) nwg = kBalancedWorkgroups * 2;
-        // no workgroup for fewer than four items
+        // no workgroup for fewer than four items; between one and two workgroups per compute unit some units would
+        // get two shares and the rest one, so one larger share each (6 sequences of 1024..4096 rows: 28.9 -> 25.3 us)
         if (nwg > (wmax + 3) / 4) nwg = (wmax + 3) / 4;
+        if (user_wgs <= 0 && nwg > kBalancedWorkgroups / 2 && nwg < kBalancedWorkgroups) nwg = kBalancedWorkgroups / 2;
         // equal lengths and as many units as workgroups or more: whole units per workgroup when they divide evenly
         a.bal_nwg = (int)nwg;
         a.nsplit = 1;
@@ -1639,10 +1657,12 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
         a.part_o = partials;
         a.part_ml = a.part_o + (size_t)B * Hq * nsplit * D;
     }
-    // Not with the grid schedule's fine chunks for per-sequence lengths: thousands of pieces each pay the
-    // counter round trip and the merge launch is cheaper (batch 32 x 32 heads, lengths 512..4096: 181 -> 191 us).
-    // With a few hundred workgroups it saves 2-5 us per step (batch 4, 32 q / 8 kv heads, 8192 rows: 30.8 -> 27.5).
-    if (merge_needed && fused_finish && (a.bal_nwg > 0 || !t_dev || tune_get("attn_fused_finish") == 1)) {
+    // Not with the grid schedule's fine chunks for per-sequence lengths when the step is large: thousands of
+    // pieces each pay the counter round trip and the merge launch is cheaper (batch 32 x 32 heads, lengths
+    // 512..4096: 181 -> 191 us; 32 q / 8 kv heads, 32 sequences of 512..4096 rows: 79.3 -> 81.8).  With a few
+    // hundred workgroups it saves 2-5 us per step (batch 4, 32 q / 8 kv heads, 8192 rows: 30.8 -> 27.5; 8
+    // sequences of 256..2048 rows: 20.8 -> 17.6).
+    if (merge_needed && fused_finish && (a.bal_nwg > 0 || !t_dev || wmax <= kFusedGridMaxItems || tune_get("attn_fused_finish") == 1)) {
         a.counters = static_cast<int*>(workspace);
         merge_needed = false;                          // the last piece of every unit finishes it
     }

@@ -329,7 +329,7 @@ def test_balanced_schedule_many_sequences(capi, ref, dev):
 @pytest.mark.parametrize("dtype,Hq,Hkv,D", [(np.float16, 8, 2, 128), (np.float16, 4, 4, 128), (np.float16, 40, 2, 128),
                                             (np.float16, 8, 1, 64), (np.float16, 12, 2, 256), (np.float32, 8, 2, 64),
                                             (np.float32, 3, 3, 128)])
-@pytest.mark.parametrize("schedule", ["grid2", "grid5", "grid64", "balanced3", "balanced50", "balanced512"])
+@pytest.mark.parametrize("schedule", ["default", "grid2", "grid5", "grid64", "balanced3", "balanced50", "balanced512"])
 def test_fused_finish_with_a_zeroed_workspace(capi, ref, dev, dtype, Hq, Hkv, D, schedule):
     """ONELLM_ATTN_ZEROED_WORKSPACE: the piece of a split sequence that arrives last merges the sequence inside the
     attention kernel (no merge launch).  One workspace, zero-filled once, serves a series of calls with different
@@ -341,7 +341,7 @@ def test_fused_finish_with_a_zeroed_workspace(capi, ref, dev, dtype, Hq, Hkv, D,
     ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
     if schedule.startswith("grid"):
         capi.tune_set("attn_nsplit", int(schedule[4:]))
-    else:
+    elif schedule.startswith("balanced"):
         capi.tune_set("attn_balanced", 1)
         capi.tune_set("attn_balanced_wgs", int(schedule[8:]))
     try:
