@@ -499,7 +499,7 @@ template <typename T, int D, int GT, int NTHR, int INFLIGHT>
 __device__ __forceinline__ void merge_pieces_wide(const AttnArgs& a, const Unit& u, int tid, float* lds)
 {
     constexpr int E = (GT * D + NTHR - 1) / NTHR;             // elements per thread
-    constexpr int BATCH = INFLIGHT / E < 4 ? 4 : (INFLIGHT / E > 64 ? 64 : INFLIGHT / E);
+    constexpr int BATCH = INFLIGHT / E < 4 ? 4 : (INFLIGHT / E > 32 ? 32 : INFLIGHT / E);   // (more would cost the single-head kernel registers)
     constexpr int NWAVE = NTHR / kWave;
     const int P = u.npieces;
     float* lw = lds;                                          // [P][GT]: m, then the weight 2^(m - max)
