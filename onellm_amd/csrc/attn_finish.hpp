@@ -1,0 +1,339 @@
+// Decode attention: set-up of a unit (q, the new k/v row) and its finish (merge of the workgroup's states, partial states, fused finish).
+// (part of decode_attn.hip, which is the only file that includes it: everything here sits in its anonymous namespace)
+#pragma once
+#include "attn_schedule.hpp"
+#include "rope.hpp"
+
+namespace onellm {
+namespace {
+
+// q of the tile's heads (and, in the last split, the new k/v row): bias, RoPE, staging in LDS; the
+// last split also stores the new row to the cache and leaves its scores in snew.  Ends with the
+// whole workgroup synchronised on sq / sk / sv (snew is ready after the caller's next barrier).
+template <typename T, int D, int GT, int NTHR>
+__device__ __forceinline__ void stage_q_and_new_row(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, T* kc, T* vc,
+                                                    float* sq, float* sk, float* sv, float* snew)
+{
+    const int tid = lane_id_per_unit();
+    const T* qkv = static_cast<const T*>(a.qkv) + (size_t)u.b * (a.Hq + 2 * a.Hkv) * D;
+    const T* bias = static_cast<const T*>(a.bias);
+    // Everything this set-up reads from memory - q, the new k and v row, their biases - is requested before any
+    // of it is used or anything is stored: one memory round trip instead of three in a row (q; then k behind the
+    // stores of q's results; then v), which every workgroup pays before its first score (5.0 -> 2.4 us after
+    // entry with cold caches at 32 heads x 128).
+    constexpr int QI = (GT * (D / 2) + NTHR - 1) / NTHR;      // q pairs per thread
+    constexpr int KI = (D / 2 + NTHR - 1) / NTHR;             // k pairs per thread
+    constexpr int VI = (D + NTHR - 1) / NTHR;                 // v elements per thread
+    T q0[QI], q1[QI], qb0[QI], qb1[QI], k0[KI], k1[KI], kb0[KI], kb1[KI], v0[VI], vb0[VI];
+    const bool v_bias = bias && !(a.flags & ONELLM_ATTN_NO_V_BIAS);
+#pragma unroll
+    for (int k = 0; k < QI; ++k) {
+        const int i = tid + k * NTHR;
+        const int g = i / (D / 2), p = i % (D / 2);
+        q0[k] = q1[k] = qb0[k] = qb1[k] = from_f32<T>(0.f);
+        if (i < GT * (D / 2) && u.g0 + g < a.G) {
+            const int o = (u.kvh * a.G + u.g0 + g) * D + 2 * p;
+            q0[k] = qkv[o];
+            q1[k] = qkv[o + 1];
+            if (bias) {
+                qb0[k] = bias[o];
+                qb1[k] = bias[o + 1];
+            }
+        }
+    }
+    if (u.is_last) {
+#pragma unroll
+        for (int k = 0; k < KI; ++k) {
+            const int p = tid + k * NTHR;
+            k0[k] = k1[k] = kb0[k] = kb1[k] = from_f32<T>(0.f);
+            if (p < D / 2) {
+                const int o = (a.Hq + u.kvh) * D + 2 * p;
+                k0[k] = qkv[o];
+                k1[k] = qkv[o + 1];
+                if (bias) {
+                    kb0[k] = bias[o];
+                    kb1[k] = bias[o + 1];
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < VI; ++k) {
+            const int d = tid + k * NTHR;
+            v0[k] = vb0[k] = from_f32<T>(0.f);
+            if (d < D) {
+                const int o = (a.Hq + a.Hkv + u.kvh) * D + d;
+                v0[k] = qkv[o];
+                if (v_bias) vb0[k] = bias[o];
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < QI; ++k) {
+        const int i = tid + k * NTHR;
+        if (i < GT * (D / 2)) {
+            const int g = i / (D / 2), p = i % (D / 2);
+            float x0 = to_f32(q0[k]), x1 = to_f32(q1[k]);     // (zeros for a head past the group's end)
+            if (bias) {
+                x0 += to_f32(qb0[k]);
+                x1 += to_f32(qb1[k]);
+            }
+            if (u.g0 + g < a.G && 2 * p < a.rotary_dim) rope_pair(x0, x1, p, u.pos, fr);
+            sq[g * D + 2 * p] = x0 * a.qscale;
+            sq[g * D + 2 * p + 1] = x1 * a.qscale;
+        }
+    }
+    if (u.is_last) {
+        const bool store = u.g0 == 0 && !(a.flags & ONELLM_ATTN_NO_CACHE_WRITE);
+#pragma unroll
+        for (int k = 0; k < KI; ++k) {
+            const int p = tid + k * NTHR;
+            if (p < D / 2) {
+                float x0 = to_f32(k0[k]), x1 = to_f32(k1[k]);
+                if (bias) {
+                    x0 += to_f32(kb0[k]);
+                    x1 += to_f32(kb1[k]);
+                }
+                if (2 * p < a.rotary_dim) rope_pair(x0, x1, p, u.pos, fr);
+                const T r0 = from_f32<T>(x0), r1 = from_f32<T>(x1);
+                sk[2 * p] = to_f32(r0);
+                sk[2 * p + 1] = to_f32(r1);
+                if (store) {
+                    kc[(size_t)(u.t - 1) * D + 2 * p] = r0;
+                    kc[(size_t)(u.t - 1) * D + 2 * p + 1] = r1;
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < VI; ++k) {
+            const int d = tid + k * NTHR;
+            if (d < D) {
+                float x = to_f32(v0[k]);
+                if (v_bias) x += to_f32(vb0[k]);
+                const T v = from_f32<T>(x);
+                sv[d] = to_f32(v);
+                if (store) vc[(size_t)(u.t - 1) * D + d] = v;
+            }
+        }
+    }
+    __syncthreads();
+    if (u.is_last && tid < kWave) {
+        const int lane = tid;
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+            float part = 0.f;
+            for (int d = lane; d < D; d += kWave) part = fmaf(sq[g * D + d], sk[d], part);
+            part = wave_sum(part);
+            if (lane == 0) snew[g] = part;
+        }
+    }
+}
+
+// device-scope accesses for data that workgroups on different chip quarters hand to each other
+__device__ __forceinline__ void publish(float* p, float v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float fetch(const float* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The fused finish's last step: the piece that arrived last reads the states of all pieces of its unit
+// (device-scope loads, BATCH pieces in flight at a time) and writes the unit's output.
+template <typename T, int D, int GT, int NTHR, int BATCH>
+__device__ __forceinline__ void merge_pieces(const AttnArgs& a, const Unit& u, int tid)
+{
+    for (int i = tid; i < GT * D; i += NTHR) {
+        const int g = i / D, d = i % D;
+        if (u.g0 + g >= a.G) continue;
+        const size_t e0 = u.p0 + (size_t)g * u.pstride;
+        float M = -INFINITY, L = 0.f, O = 0.f;
+        for (int s0 = 0; s0 < u.npieces; s0 += BATCH) {
+            float mm[BATCH], ll[BATCH], oo[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const size_t e = e0 + (size_t)min(s0 + j, u.npieces - 1) * u.sstride;
+                mm[j] = fetch(a.part_ml + e * 2);
+                ll[j] = fetch(a.part_ml + e * 2 + 1);
+                oo[j] = fetch(a.part_o + e * D + d);
+            }
+            float bm = M;
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) bm = s0 + j < u.npieces ? fmaxf(bm, mm[j]) : bm;
+            const float keep = __builtin_amdgcn_exp2f(M - bm);   // every piece has a finite maximum
+            L *= keep;
+            O *= keep;
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const float wgt = s0 + j < u.npieces ? __builtin_amdgcn_exp2f(mm[j] - bm) : 0.f;
+                L = fmaf(ll[j], wgt, L);
+                O = fmaf(oo[j], wgt, O);
+            }
+            M = bm;
+        }
+        const int h = u.kvh * a.G + u.g0 + g;
+        static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + d] = from_f32<T>(O / L);
+    }
+}
+
+// The same for a unit with many pieces (a long sequence of a small batch is cut into up to 64): the (m, l)
+// pairs of all pieces go through LDS first - one round trip - where each head's maximum, its pieces' weights
+// and its sum are worked out once, a head per wave at a time; then only the partial sums are read, about 32
+// loads in flight per thread over all of its elements, instead of one element and sixteen pieces at a time
+// (eight round trips become two at 64 pieces and two elements per thread: the first batch of sums is
+// requested together with the pairs).  The order of every sum is
+// fixed, so the result does not depend on which piece arrived last.  `lds` holds (2 * npieces + 1) * GT floats.
+template <typename T, int D, int GT, int NTHR, int INFLIGHT>
+__device__ __forceinline__ void merge_pieces_wide(const AttnArgs& a, const Unit& u, int tid, float* lds)
+{
+    constexpr int E = (GT * D + NTHR - 1) / NTHR;             // elements per thread
+    constexpr int BATCH = INFLIGHT / E < 4 ? 4 : (INFLIGHT / E > 32 ? 32 : INFLIGHT / E);   // (more would cost the single-head kernel registers)
+    constexpr int NWAVE = NTHR / kWave;
+    const int P = u.npieces;
+    float* lw = lds;                                          // [P][GT]: m, then the weight 2^(m - max)
+    float* ll = lds + P * GT;                                 // [P][GT]: l
+    float* lL = ll + P * GT;                                  // [GT]: the head's sum
+    bool valid[E];
+    int hg[E];
+    const float* po[E];
+    float O[E];
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+        const int i = tid + k * NTHR;
+        hg[k] = i / D;
+        valid[k] = i < GT * D && u.g0 + hg[k] < a.G;
+        if (!valid[k]) hg[k] = 0;                             // (a thread without an element reads the tile's first head and stores nothing:
+        po[k] = a.part_o + (u.p0 + (size_t)hg[k] * u.pstride) * D + i % D;   //  the loads below stay free of branches)
+        O[k] = 0.f;
+    }
+    float oo[E][BATCH];
+    auto request = [&](int s0) {
+#pragma unroll
+        for (int k = 0; k < E; ++k)
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j)
+                oo[k][j] = fetch(po[k] + (size_t)min(s0 + j, P - 1) * u.sstride * D);
+    };
+    // the first batch of partial sums travels together with the (m, l) pairs
+    request(0);
+    for (int p = tid; p < P * GT; p += NTHR) {
+        const int sp = p / GT, g = p % GT;
+        if (u.g0 + g < a.G) {
+            const size_t e = u.p0 + (size_t)g * u.pstride + (size_t)sp * u.sstride;
+            lw[p] = fetch(a.part_ml + e * 2);
+            ll[p] = fetch(a.part_ml + e * 2 + 1);
+        }
+    }
+    __syncthreads();
+    {
+        const int lane = tid & (kWave - 1);
+        for (int g = tid / kWave; g < GT; g += NWAVE) {       // (uniform over the wave)
+            if (u.g0 + g >= a.G) continue;
+            float M = -INFINITY;
+            for (int sp = lane; sp < P; sp += kWave) M = fmaxf(M, lw[sp * GT + g]);
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, kWave));
+            float L = 0.f;
+            for (int sp = lane; sp < P; sp += kWave) {
+                const float wgt = __builtin_amdgcn_exp2f(lw[sp * GT + g] - M);   // every piece has a finite maximum
+                lw[sp * GT + g] = wgt;
+                L = fmaf(ll[sp * GT + g], wgt, L);
+            }
+            L = wave_sum(L);
+            if (lane == 0) lL[g] = L;
+        }
+    }
+    __syncthreads();
+    for (int s0 = 0; s0 < P; s0 += BATCH) {
+        if (s0 > 0) request(s0);
+#pragma unroll
+        for (int k = 0; k < E; ++k)
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const float wgt = lw[min(s0 + j, P - 1) * GT + hg[k]];
+                O[k] = fmaf(oo[k][j], s0 + j < P ? wgt : 0.f, O[k]);
+            }
+    }
+#pragma unroll
+    for (int k = 0; k < E; ++k)
+        if (valid[k]) {
+            const int i = tid + k * NTHR;
+            const int h = u.kvh * a.G + u.g0 + hg[k];
+            static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + i % D] = from_f32<T>(O[k] / lL[hg[k]]);
+        }
+}
+
+// Merge the NST softmax states the workgroup left in LDS (plus the new token's row in the last
+// split) and write either the output (single split) or this split's partial state.  The caller has
+// synchronised the workgroup on st_ml / st_acc / snew.
+template <typename T, int D, int GT, int NST, int NTHR>
+__device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, float* st_ml, float* st_acc,
+                                            const float* snew, const float* sv)
+{
+    for (int i = lane_id_per_unit(); i < GT * D; i += NTHR) {
+        const int g = i / D, d = i % D;
+        if (u.g0 + g >= a.G) continue;
+        float M = u.is_last ? snew[g] : -INFINITY;
+        for (int r = 0; r < NST; ++r) M = fmaxf(M, st_ml[(r * GT + g) * 2]);
+        float L = 0.f, O = 0.f;
+        for (int r = 0; r < NST; ++r) {
+            const float w = __builtin_amdgcn_exp2f(st_ml[(r * GT + g) * 2] - M);
+            L = fmaf(st_ml[(r * GT + g) * 2 + 1], w, L);
+            O = fmaf(st_acc[(size_t)(r * GT + g) * D + d], w, O);
+        }
+        if (u.is_last) {
+            const float w = __builtin_amdgcn_exp2f(snew[g] - M);
+            L += w;
+            O = fmaf(sv[d], w, O);
+        }
+        const int h = u.kvh * a.G + u.g0 + g;
+        if (u.direct) {
+            static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + d] = from_f32<T>(O / L);
+        } else if (!a.counters) {
+            const size_t pi = u.pbase + (size_t)g * u.pstride;
+            a.part_o[pi * D + d] = O;
+            if (d == 0) {
+                a.part_ml[pi * 2] = M;
+                a.part_ml[pi * 2 + 1] = L;
+            }
+        } else {
+            const size_t pi = u.pbase + (size_t)g * u.pstride;
+            publish(a.part_o + pi * D + d, O);
+            if (d == 0) {
+                publish(a.part_ml + pi * 2, M);
+                publish(a.part_ml + pi * 2 + 1, L);
+            }
+        }
+    }
+    if (u.direct || !a.counters) return;
+
+    // ---- fused finish.  Every piece of the unit has written its state with device-scope stores
+    // (written through to memory, not left in this chip quarter's L2) and then, once all of its
+    // threads' stores have completed, adds one to the unit's counter.  The piece whose add finds
+    // all the others there reads their states back with device-scope loads and merges them.  No
+    // cache write-back or invalidation is involved: the only data that crosses between workgroups
+    // moves through these scoped accesses, and nobody waits on anybody.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();                                            // all stores done; st_ml no longer read
+    int* arrived = reinterpret_cast<int*>(st_ml);                  // the merged states are no longer needed: reuse a word
+    const int tid = lane_id_per_unit();
+    if (tid == 0)
+        *arrived = __hip_atomic_fetch_add(a.counters + u.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*arrived != u.npieces - 1) return;
+    if (tid == 0) __hip_atomic_store(a.counters + u.counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
+    // (pieces whose loads are in flight together: 16 at most, no more than the unit has - most have two or three -
+    // rounded up to a power of two; the surplus slots of a batch repeat the last piece's loads)
+    if (u.npieces <= 2) merge_pieces<T, D, GT, NTHR, 2>(a, u, tid);
+    else if (u.npieces <= 4) merge_pieces<T, D, GT, NTHR, 4>(a, u, tid);
+    else if (u.npieces <= 8) merge_pieces<T, D, GT, NTHR, 8>(a, u, tid);
+    // (where a thread has 128 partial sums or more to read - measured: 32 q / 8 kv heads, batch 1, 8192 rows, 64 pieces x 2
+    // elements 16.9 -> 16.5 us; 64 q heads, 32768 rows, 32 x 4: 35.4 -> 32.3; batch 2, 32 x 2: 20.0 -> 21.1, hence
+    // not there.  st_acc: NST * GT * D floats, free by now)
+    else if (u.npieces * ((GT * D + NTHR - 1) / NTHR) >= 128 && 2 * u.npieces + 1 <= NST * D)
+        merge_pieces_wide<T, D, GT, NTHR, 32>(a, u, tid, st_acc);
+    else merge_pieces<T, D, GT, NTHR, 16>(a, u, tid);
+}
+
+}  // namespace
+}  // namespace onellm

@@ -1,0 +1,303 @@
+// Decode attention: launch arguments, what a workgroup works on, the grid and the balanced workgroup schedules.
+// (part of decode_attn.hip, which is the only file that includes it: everything here sits in its anonymous namespace)
+#pragma once
+#include "common.hpp"
+
+namespace onellm {
+namespace {
+
+constexpr size_t kCounterBytes = 64 * 1024; // arrival counters of the fused finish: the first bytes of every workspace
+constexpr int kBalancedWorkgroups = 512;   // two 4-wave workgroups per compute unit: what the register budgets keep resident
+constexpr long long kBalancedMinItems = 3072;   // the balanced schedule is not the default for a smaller step
+constexpr long long kFusedGridMaxItems = 8192;  // per-sequence lengths on the grid schedule: fused finish up to this size
+
+struct AttnArgs {
+    const void* qkv;
+    const void* bias;
+    void* k_cache;
+    void* v_cache;
+    void* out;
+    float* part_o;        // [B, Hq, nsplit, D]
+    float* part_ml;       // [B, Hq, nsplit, 2]
+    const int* t_dev;
+    int t_host;
+    int B, Hq, Hkv, G, S;
+    int chunk;            // cache rows per split
+    int nsplit;           // grid.x
+    int rotary_dim;
+    int pos_offset;
+    unsigned flags;
+    float qscale;         // log2(e) / sqrt(D), folded into q
+    size_t slab;          // element offset of the layer slab inside the cache
+    // balanced schedule (bal_nwg > 0): the grid is bal_nwg workgroups and each takes an equal,
+    // contiguous share of all work items (an item = item_rows history rows of one unit)
+    int bal_nwg;
+    int item_rows;
+    int gt;               // query heads per tile, for the merge kernel
+    // fused finish (counters != NULL): one arrival counter per unit, zero between calls; the piece
+    // that arrives last merges the unit's partial states itself and no merge kernel is launched
+    int* counters;
+};
+
+// What one workgroup works on: a chunk of the history of one (sequence, kv-head) for up to GT query heads.
+struct Unit {
+    int b, kvh, g0;        // sequence, kv head, first query head of the tile inside the group
+    int t, pos;            // attended positions of the sequence; RoPE position of the new token
+    int split, last;       // this workgroup's split and the sequence's last split
+    int r0, r1;            // history rows [r0, r1) of this split
+    bool is_last;          // the last split also owns the new token's row
+    bool direct;           // the workgroup sees the whole unit: it writes the output, not a partial state
+    size_t pbase;          // partial-state entry of tile head g: pbase + g * pstride
+    int pstride;
+    // for the fused finish: the unit's pieces are entries p0 + g * pstride + s * sstride, s < npieces
+    size_t p0;
+    int sstride, npieces, counter;
+};
+
+// Workgroups are dealt to the 8 XCDs round-robin in linear block order.  The kv-head index is the
+// fastest grid dimension so that every XCD sees the same mix of sequences and splits, and the split
+// index is rotated by the sequence index so that, with ragged lengths, the splits every sequence has
+// (the low ones) do not all land on the same XCDs.  Returns false when there is nothing to do.
+template <int GT>
+__device__ __forceinline__ bool locate_unit(const AttnArgs& a, Unit& u)
+{
+    const int ngt = (a.G + GT - 1) / GT;
+    u.kvh = blockIdx.x / ngt;
+    u.g0 = (blockIdx.x % ngt) * GT;
+    u.b = blockIdx.z;
+    u.split = (blockIdx.y + u.b) % a.nsplit;
+    u.t = a.t_dev ? a.t_dev[u.b] : a.t_host;
+    if (u.t < 1 || u.t > a.S) return false;      // out-of-contract length: touch nothing
+    u.last = (u.t - 1) / a.chunk;
+    if (u.split > u.last) return false;
+    u.is_last = u.split == u.last;
+    u.r0 = u.split * a.chunk;
+    u.r1 = min(u.r0 + a.chunk, u.t - 1);
+    u.pos = u.t + a.pos_offset;
+    u.direct = a.nsplit == 1 || (a.counters && u.last == 0);    // (with the fused finish a one-piece sequence needs no partial)
+    u.p0 = ((size_t)u.b * a.Hq + u.kvh * a.G + u.g0) * a.nsplit;
+    u.pbase = u.p0 + u.split;
+    u.pstride = a.nsplit;
+    u.sstride = 1;
+    u.npieces = min(u.last + 1, a.nsplit);       // (a length above max_t is out of contract: stay consistent)
+    u.counter = u.b * (a.Hkv * ngt) + blockIdx.x;
+    return true;
+}
+
+// ---- balanced schedule -----------------------------------------------------------------------
+// All work of a step is cut into items of item_rows history rows; a unit (sequence, kv head, head
+// tile) of a sequence with t attended positions has max(1, ceil((t-1)/item_rows)) of them (the
+// last one also carries the new token's row).  Items are numbered sequence-major, then unit, then
+// row order, and workgroup i of N takes items [i*W/N, (i+1)*W/N): every workgroup streams the same
+// number of rows whatever the lengths are, crossing from one unit into the next where its share
+// does.  A unit seen whole by one workgroup is finished by it; otherwise each workgroup that
+// touches it leaves a partial state in entry (workgroup + global unit index) - unique, because
+// along the walk either the workgroup or the unit advances - and whoever merges them (the merge
+// kernel, or the piece that arrives last when the finish is fused) derives the same boundaries from
+// the same lengths.
+__device__ __forceinline__ int seq_items(const AttnArgs& a, int t)
+{
+    if (t < 1 || t > a.S) return 0;               // out-of-contract length: no work, nothing touched
+    const int n = (t - 1 + a.item_rows - 1) / a.item_rows;
+    return n < 1 ? 1 : n;
+}
+
+// The schedule is the same in every lane; saying so keeps it in scalar registers (the kernels that
+// walk it are short of vector registers).
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ long long uniform(long long v)
+{
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(unsigned long long)v);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)((unsigned long long)v >> 32));
+    return (long long)(((unsigned long long)hi << 32) | lo);
+}
+
+// Thread index as a value the compiler takes as new each time it is asked for: everything a unit
+// derives from it (addresses, masks, lane roles) is then recomputed per unit instead of being
+// hoisted out of the loop over units and held in registers across the streaming loop.
+__device__ __forceinline__ int lane_id_per_unit()
+{
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    return tid;
+}
+
+__device__ __forceinline__ long long wave_sum_i64(long long v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// items of all sequences, and of the sequences before `before` (every lane gets both)
+__device__ __forceinline__ void count_items(const AttnArgs& a, int before, long long& total, long long& prefix)
+{
+    if (!a.t_dev) {
+        const int it = seq_items(a, a.t_host);
+        total = (long long)a.B * it;
+        prefix = (long long)before * it;
+        return;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    long long tot = 0, pre = 0;
+    for (int bb = lane; bb < a.B; bb += kWave) {
+        const int it = seq_items(a, a.t_dev[bb]);
+        tot += it;
+        if (bb < before) pre += it;
+    }
+    total = uniform(wave_sum_i64(tot));
+    prefix = uniform(wave_sum_i64(pre));
+}
+
+// workgroup that owns item x when W items are dealt to N workgroups as [i*W/N, (i+1)*W/N)
+__device__ __forceinline__ int item_owner(long long x, long long W, int N)
+{
+    return (int)(((x + 1) * N - 1) / W);
+}
+
+// Workgroups that take part: never more than there are items, so that no share is empty and the
+// workgroups of a unit are consecutive - and, as the host sizes the grid for the longest length it
+// was given while the real lengths may be much shorter: no workgroup for fewer than four items, and
+// not between one and two workgroups per compute unit (some units would get two shares, the rest one:
+// better one larger share each).  The launch has one workgroup per compute unit or two (or what a sweep
+// asked for, taken as it is).
+__device__ __forceinline__ int balanced_workgroups(const AttnArgs& a, long long W)
+{
+    long long n = (W + 3) / 4;
+    if (n > a.bal_nwg) n = a.bal_nwg;
+    if (a.bal_nwg == kBalancedWorkgroups && n > kBalancedWorkgroups / 2 && n < kBalancedWorkgroups) n = kBalancedWorkgroups / 2;
+    return (int)n;
+}
+
+struct Walk {
+    long long W;           // items of the whole step
+    int N;                 // workgroups that share them
+    long long cur, hi;     // next item of this workgroup, end of its share
+    long long base;        // first item of sequence b
+    int b, items;          // current sequence and its items per unit
+    int nunits;            // units per sequence
+};
+
+// Positions the walk at the first item of workgroup blockIdx.x; false when its share is empty.
+__device__ __forceinline__ bool walk_begin(const AttnArgs& a, int nunits, Walk& w)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    long long total, unused;
+    count_items(a, 0, total, unused);
+    const long long W = total * nunits;
+    const int N = balanced_workgroups(a, W);
+    if ((int)blockIdx.x >= N) return false;
+    w.nunits = nunits;
+    w.W = W;
+    w.N = N;
+    w.cur = uniform((long long)blockIdx.x * W / N);
+    w.hi = uniform((long long)(blockIdx.x + 1) * W / N);         // > cur, because N <= W
+    const long long target = w.cur / nunits;       // the sequence that holds item `cur` holds per-unit item `target`
+    if (!a.t_dev) {
+        w.items = seq_items(a, a.t_host);
+        w.b = uniform((int)(target / w.items));
+        w.base = (long long)w.b * w.items * nunits;
+        return true;
+    }
+    long long run = 0;
+    for (int c = 0; c < a.B; c += kWave) {
+        const int bb = c + lane;
+        const int it = bb < a.B ? seq_items(a, a.t_dev[bb]) : 0;
+        long long inc = it;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const long long v = __shfl_up(inc, off, kWave);
+            if (lane >= off) inc += v;
+        }
+        const long long tot = __shfl(inc, kWave - 1, kWave);
+        if (run + tot > target) {
+            const unsigned long long hit = __builtin_amdgcn_ballot_w64(run + inc > target);
+            const int f = __builtin_ctzll(hit);
+            w.b = c + f;
+            w.items = uniform(__shfl(it, f, kWave));
+            w.base = (run + uniform(__shfl(inc, f, kWave)) - w.items) * nunits;
+            return true;
+        }
+        run += uniform(tot);
+    }
+    return false;                                   // not reached: target < total
+}
+
+// The unit piece at the walk's position (as many of the unit's remaining items as the share allows).
+template <int GT>
+__device__ __forceinline__ void walk_unit(const AttnArgs& a, const Walk& w, Unit& u, int& nitems)
+{
+    const int ngt = (a.G + GT - 1) / GT;
+    const long long rel = w.cur - w.base;
+    const int uib = uniform((int)(rel / w.items));
+    const int item = uniform((int)(rel - (long long)uib * w.items));
+    const long long left = w.hi - w.cur;
+    nitems = w.items - item;
+    if (left < nitems) nitems = (int)left;
+    nitems = uniform(nitems);
+    u.b = w.b;
+    u.kvh = uib / ngt;
+    u.g0 = (uib % ngt) * GT;
+    u.t = uniform(a.t_dev ? a.t_dev[w.b] : a.t_host);
+    u.pos = u.t + a.pos_offset;
+    u.split = 0;
+    u.last = 0;
+    u.r0 = item * a.item_rows;
+    u.r1 = min(u.r0 + nitems * a.item_rows, u.t - 1);
+    u.is_last = item + nitems == w.items;
+    u.direct = item == 0 && u.is_last;
+    const size_t unit_index = (size_t)w.b * w.nunits + uib;
+    u.pbase = ((size_t)blockIdx.x + unit_index) * GT;
+    u.pstride = 1;
+    u.p0 = 0;
+    u.sstride = GT;
+    u.npieces = 1;
+    u.counter = (int)unit_index;
+    if (!u.direct && a.counters) {
+        const long long first = w.base + (long long)uib * w.items;
+        const int i0 = uniform(item_owner(first, w.W, w.N)), i1 = uniform(item_owner(first + w.items - 1, w.W, w.N));
+        u.p0 = ((size_t)i0 + unit_index) * GT;
+        u.npieces = i1 - i0 + 1;
+    }
+}
+
+// Moves past nitems items; steps to the next sequence that has work when the current one is done.
+__device__ __forceinline__ void walk_advance(const AttnArgs& a, Walk& w, int nitems)
+{
+    w.cur += nitems;
+    if (w.cur >= w.hi) return;
+    if (w.cur == w.base + (long long)w.items * w.nunits) {
+        w.base = w.cur;
+        do {
+            if (++w.b >= a.B) {                      // lengths changed under the kernel (out of contract): stop
+                w.cur = w.hi;
+                return;
+            }
+            w.items = uniform(seq_items(a, a.t_dev ? a.t_dev[w.b] : a.t_host));
+        } while (w.items == 0);                      // cur < hi <= W: a later sequence has items
+    }
+}
+
+// Runs `body(unit)` for the one unit of the grid schedule, or for every unit piece of this
+// workgroup's share of the balanced schedule.
+template <int GT, bool BALANCED, typename F>
+__device__ __forceinline__ void for_each_unit(const AttnArgs& a, F&& body)
+{
+    Unit u;
+    if constexpr (!BALANCED) {
+        if (locate_unit<GT>(a, u)) body(u);
+    } else {
+        Walk w;
+        if (!walk_begin(a, a.Hkv * ((a.G + GT - 1) / GT), w)) return;
+        while (w.cur < w.hi) {
+            int nitems;
+            walk_unit<GT>(a, w, u, nitems);
+            body(u);
+            walk_advance(a, w, nitems);
+            if (w.cur < w.hi) __syncthreads();       // the next unit reuses the LDS staging
+        }
+    }
+}
+
+}  // namespace
+}  // namespace onellm
