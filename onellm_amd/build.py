@@ -64,11 +64,39 @@ def _compile(src, force):
         return obj
     cmd = [HIPCC, "-c", path, "-o", obj] + COMMON
     if src.endswith(".hip"):
-        cmd += DEVICE
+        # (the compiler's per-kernel register / occupancy / scratch remarks are kept next to the object:
+        # tests/test_kernel_resources.py holds the kernels to their budgets)
+        cmd += DEVICE + ["-Rpass-analysis=kernel-resource-usage"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr[-4000:]))
+    if src.endswith(".hip"):
+        with open(resources_file(src), "w") as f:
+            f.write(r.stderr)
     return obj
+
+
+def resources_file(src):
+    """Where the build leaves hipcc's kernel-resource-usage remarks of one .hip source."""
+    return os.path.join(OBJ, os.path.splitext(src)[0] + ".resources.txt")
+
+
+def kernel_resources(src):
+    """{demangled-ish kernel symbol: {"vgprs", "agprs", "sgprs", "occupancy", "scratch", "lds"}} from the last build of src."""
+    import re
+    out = {}
+    with open(resources_file(src)) as f:
+        text = f.read()
+    for block in re.split(r"remark: [^\n]*Function Name: ", text)[1:]:
+        name = block.split("\n")[0].split(" ")[0]
+
+        def field(label):
+            m = re.search(label + r": (\d+)", block)
+            return int(m.group(1)) if m else None
+        out[name] = dict(vgprs=field("VGPRs"), agprs=field("AGPRs"), sgprs=field("SGPRs"),
+                         occupancy=field(r"Occupancy \[waves/SIMD\]"), scratch=field(r"ScratchSize \[bytes/lane\]"),
+                         lds=field(r"LDS Size \[bytes/block\]"))
+    return out
 
 
 def build(force=False, verbose=False):
