@@ -33,6 +33,7 @@ struct AttnArgs {
     // contiguous share of all work items (an item = item_rows history rows of one unit)
     int bal_nwg;
     int item_rows;
+    int unit_cost;        // what starting on another unit costs a workgroup, in items (set-up, finish, an emptied load queue)
     int gt;               // query heads per tile, for the merge kernel
     // fused finish (counters != NULL): one arrival counter per unit, zero between calls; the piece
     // that arrives last merges the unit's partial states itself and no merge kernel is launched
@@ -95,11 +96,17 @@ __device__ __forceinline__ bool locate_unit(const AttnArgs& a, Unit& u)
 // along the walk either the workgroup or the unit advances - and whoever merges them (the merge
 // kernel, or the piece that arrives last when the finish is fused) derives the same boundaries from
 // the same lengths.
+//
+// Changing units is not free for a workgroup (the finish of one, the set-up of the next and a load queue that
+// runs empty in between cost about as much as three items), so the shares are equal in cost rather than in
+// rows: every unit is preceded by unit_cost items that stand for that overhead and hold no rows.  A workgroup
+// whose share only touches those has nothing to do for the unit; the one whose share crosses into the rows
+// pays the overhead and gets correspondingly fewer rows.
 __device__ __forceinline__ int seq_items(const AttnArgs& a, int t)
 {
     if (t < 1 || t > a.S) return 0;               // out-of-contract length: no work, nothing touched
     const int n = (t - 1 + a.item_rows - 1) / a.item_rows;
-    return n < 1 ? 1 : n;
+    return (n < 1 ? 1 : n) + a.unit_cost;
 }
 
 // The schedule is the same in every lane; saying so keeps it in scalar registers (the kernels that
@@ -224,8 +231,9 @@ __device__ __forceinline__ bool walk_begin(const AttnArgs& a, int nunits, Walk& 
 }
 
 // The unit piece at the walk's position (as many of the unit's remaining items as the share allows).
+// (false: this piece lies inside the unit's overhead items - no rows, nothing to do)
 template <int GT>
-__device__ __forceinline__ void walk_unit(const AttnArgs& a, const Walk& w, Unit& u, int& nitems)
+__device__ __forceinline__ bool walk_unit(const AttnArgs& a, const Walk& w, Unit& u, int& nitems)
 {
     const int ngt = (a.G + GT - 1) / GT;
     const long long rel = w.cur - w.base;
@@ -242,10 +250,12 @@ __device__ __forceinline__ void walk_unit(const AttnArgs& a, const Walk& w, Unit
     u.pos = u.t + a.pos_offset;
     u.split = 0;
     u.last = 0;
-    u.r0 = item * a.item_rows;
-    u.r1 = min(u.r0 + nitems * a.item_rows, u.t - 1);
+    const int c0 = a.unit_cost;
+    const int lo = item > c0 ? item - c0 : 0, hi = item + nitems > c0 ? item + nitems - c0 : 0;   // items that hold rows
+    u.r0 = lo * a.item_rows;
+    u.r1 = min(hi * a.item_rows, u.t - 1);
     u.is_last = item + nitems == w.items;
-    u.direct = item == 0 && u.is_last;
+    u.direct = item <= c0 && u.is_last;          // every item that holds rows is here
     const size_t unit_index = (size_t)w.b * w.nunits + uib;
     u.pbase = ((size_t)blockIdx.x + unit_index) * GT;
     u.pstride = 1;
@@ -255,10 +265,11 @@ __device__ __forceinline__ void walk_unit(const AttnArgs& a, const Walk& w, Unit
     u.counter = (int)unit_index;
     if (!u.direct && a.counters) {
         const long long first = w.base + (long long)uib * w.items;
-        const int i0 = uniform(item_owner(first, w.W, w.N)), i1 = uniform(item_owner(first + w.items - 1, w.W, w.N));
+        const int i0 = uniform(item_owner(first + c0, w.W, w.N)), i1 = uniform(item_owner(first + w.items - 1, w.W, w.N));
         u.p0 = ((size_t)i0 + unit_index) * GT;
         u.npieces = i1 - i0 + 1;
     }
+    return hi > 0;
 }
 
 // Moves past nitems items; steps to the next sequence that has work when the current one is done.
@@ -291,10 +302,10 @@ __device__ __forceinline__ void for_each_unit(const AttnArgs& a, F&& body)
         if (!walk_begin(a, a.Hkv * ((a.G + GT - 1) / GT), w)) return;
         while (w.cur < w.hi) {
             int nitems;
-            walk_unit<GT>(a, w, u, nitems);
-            body(u);
+            const bool rows = walk_unit<GT>(a, w, u, nitems);
+            if (rows) body(u);
             walk_advance(a, w, nitems);
-            if (w.cur < w.hi) __syncthreads();       // the next unit reuses the LDS staging
+            if (rows && w.cur < w.hi) __syncthreads();   // the next unit reuses the LDS staging
         }
     }
 }

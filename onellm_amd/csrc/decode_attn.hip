@@ -114,7 +114,7 @@ void decode_attn_merge_balanced_kernel(const AttnArgs a, int D)
     const long long W = total * nunits;
     const long long first = before * nunits + (long long)uib * items;
     const int N = balanced_workgroups(a, W);
-    const int i0 = item_owner(first, W, N), i1 = item_owner(first + items - 1, W, N);
+    const int i0 = item_owner(first + a.unit_cost, W, N), i1 = item_owner(first + items - 1, W, N);   // (the items that hold rows)
     if (i0 == i1) return;
     const int n = i1 - i0 + 1;
     // entry of workgroup i0 + s: (i0 + s + global unit) * gt + g
@@ -565,12 +565,17 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);
     if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, on_matrix_cores(dtype == ONELLM_FP16, D, G), (long)B * nunits, wmax)))) {
         a.item_rows = item_rows;
+        // (what a change of unit costs a workgroup, in items: measured on the matrix-core kernel, where workgroups whose
+        // equal-row shares held one / two / three units finished at 82 / 90 / 94 us of a 101 us step)
+        const int user_cost = tune_get("attn_balanced_cost");
+        a.unit_cost = user_cost >= 0 ? user_cost : 3;
+        const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
         const int user_wgs = tune_get("attn_balanced_wgs");
         long long nwg = user_wgs > 0 ? user_wgs : kBalancedWorkgroups;
         if (nwg > kBalancedWorkgroups * 2) nwg = kBalancedWorkgroups * 2;
         // no workgroup for fewer than four items; between one and two workgroups per compute unit some units would
         // get two shares and the rest one, so one larger share each (6 sequences of 1024..4096 rows: 28.9 -> 25.3 us)
-        if (nwg > (wmax + 3) / 4) nwg = (wmax + 3) / 4;
+        if (nwg > (wmax_cost + 3) / 4) nwg = (wmax_cost + 3) / 4;
         if (user_wgs <= 0 && nwg > kBalancedWorkgroups / 2 && nwg < kBalancedWorkgroups) nwg = kBalancedWorkgroups / 2;
         // equal lengths and as many units as workgroups or more: whole units per workgroup when they divide evenly
         a.bal_nwg = (int)nwg;

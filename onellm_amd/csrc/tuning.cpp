@@ -18,6 +18,7 @@ Knob g_knobs[] = {
     {"attn_nsplit", {-1}},       // force the number of sequence splits
     {"attn_balanced", {-1}},     // 1 / 0: force the balanced workgroup schedule of decode attention on / off
     {"attn_balanced_wgs", {-1}}, // workgroups of the balanced schedule
+    {"attn_balanced_cost", {-1}}, // items a change of unit is charged with in the balanced schedule
     {"attn_fused_finish", {-1}}, // 0: keep the separate merge launch even when the workspace is declared zeroed
     {"prefill_generic", {-1}},   // 1: the index-walking prefill kernel also where the row-walking one applies
     {"attn_gqa_valu", {-1}},     // 1: grouped-query heads on the vector ALU kernel instead of the MFMA one
