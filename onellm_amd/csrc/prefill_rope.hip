@@ -149,6 +149,23 @@ void qkv_bias_rope_transpose_rows_kernel(const PrefillArgs a, const RopeFreqs fr
     const int D = NVEC * VEC, QKVH = a.Hq + 2 * a.Hkv;
     const int tok = blockIdx.x * TT + tl;
     if (tok >= token_num) return;
+    // the first heads of the token are requested before its destination is known: where it goes (padding
+    // offset -> sequence -> history length, two dependent loads) and the sin / cos of its pairs are worked out
+    // while they travel - every workgroup of the launch starts at the same time, so nothing else covers that wait
+    const T* in = static_cast<const T*>(a.qkv) + (size_t)tok * (a.Hq + 2 * a.Hkv) * (NVEC * VEC) + c;
+    const T* bias = static_cast<const T*>(a.bias);
+    Vec16<T> v[UNROLL], bv[UNROLL];
+    auto request = [&](int hb) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int h = hb + u * HPP;
+            if (h < a.Hq + 2 * a.Hkv) {
+                v[u] = load16_stream(in + (size_t)h * (NVEC * VEC));
+                if (bias) bv[u] = load16(bias + (size_t)h * (NVEC * VEC) + c);
+            }
+        }
+    };
+    request(h0);
     const long dst = (long)tok + a.padding_offset[tok];
     const long b = dst / a.seq_len;
     if (dst < 0 || b >= a.B) return;              // a token outside the batch touches nothing
@@ -163,22 +180,12 @@ void qkv_bias_rope_transpose_rows_kernel(const PrefillArgs a, const RopeFreqs fr
         cs[e] = 1.f;
         if (p < npair) sincos_fixed((float)pos / fr.f[p], sn[e], cs[e]);
     }
-    const T* in = static_cast<const T*>(a.qkv) + (size_t)tok * QKVH * D + c;
-    const T* bias = static_cast<const T*>(a.bias);
     T* qo = static_cast<T*>(a.q_buf) + ((size_t)b * a.Hq * a.seq_len + (size_t)srow) * D + c;
     T* ko = static_cast<T*>(a.k_buf) + ((size_t)b * a.Hkv * a.seq_len + (size_t)srow) * D + c;
     T* vo = static_cast<T*>(a.v_buf) + ((size_t)b * a.Hkv * a.seq_len + (size_t)srow) * D + c;
     const size_t head_step = (size_t)a.seq_len * D;
     for (int hb = h0; hb < QKVH; hb += HPP * UNROLL) {
-        Vec16<T> v[UNROLL], bv[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int h = hb + u * HPP;
-            if (h < QKVH) {
-                v[u] = load16_stream(in + (size_t)h * D);
-                if (bias) bv[u] = load16(bias + (size_t)h * D + c);
-            }
-        }
+        if (hb != h0) request(hb);
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int h = hb + u * HPP;
