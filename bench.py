@@ -29,7 +29,7 @@ MEASURED_TRAFFIC_BYTES = {4096: 1074432616}
 
 def attn_bytes(B, Hq, Hkv, D, t_list, e):
     """Algorithmic bytes of one decode step: history K+V read once, new row written, qkv + bias read, out written."""
-    hist = sum(2 * Hkv * (t - 1) * D * e for t in t_list)
+    hist = sum(2 * Hkv * (int(t) - 1) * D * e for t in t_list)     # (int: lengths may arrive as 32-bit numpy scalars)
     return hist + 2 * B * Hkv * D * e + B * (Hq + 2 * Hkv) * D * e + (Hq + 2 * Hkv) * D * e + B * Hq * D * e
 
 

@@ -32,21 +32,6 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
-// Two workgroups of the balanced schedule share a compute unit, and the one that came first gets its instructions
-// issued first whenever both are ready: it runs ~12 % faster and leaves the other to finish alone, at half the
-// unit's memory parallelism (finish times 80 / 90 us for the first / second 256 workgroups of a 101 us step).
-// The two take turns instead: wave priority follows a bit of the chip-wide constant-rate clock, opposite in
-// the two halves of the grid (workgroup i and i + 256 land on the same compute unit), ~5 us each way.
-__device__ __forceinline__ void take_turns(const AttnArgs& a)
-{
-    if (a.bal_nwg > 256) {
-        const bool second = blockIdx.x >= 256;
-        const bool phase = ((wall_clock64() >> 9) & 1) != 0;
-        if (phase != second) __builtin_amdgcn_s_setprio(1);
-        else __builtin_amdgcn_s_setprio(0);
-    }
-}
-
 template <int D, int GT, int NW, bool DOUBLE_BUFFER>
 __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds)
 {

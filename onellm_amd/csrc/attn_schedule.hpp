@@ -34,6 +34,7 @@ struct AttnArgs {
     int bal_nwg;
     int item_rows;
     int unit_cost;        // what starting on another unit costs a workgroup, in items (set-up, finish, an emptied load queue)
+    int turns;            // co-resident workgroups take turns at wave priority (take_turns below); 0: they do not
     int gt;               // query heads per tile, for the merge kernel
     // fused finish (counters != NULL): one arrival counter per unit, zero between calls; the piece
     // that arrives last merges the unit's partial states itself and no merge kernel is launched
@@ -286,6 +287,31 @@ __device__ __forceinline__ void walk_advance(const AttnArgs& a, Walk& w, int nit
             }
             w.items = uniform(seq_items(a, a.t_dev ? a.t_dev[w.b] : a.t_host));
         } while (w.items == 0);                      // cur < hi <= W: a later sequence has items
+    }
+}
+
+// Workgroups that share a compute unit do not share it fairly: the one that came first gets its instructions issued
+// first whenever several are ready, runs faster and leaves the others to finish alone, at a fraction of the unit's
+// memory parallelism.  Measured finish times: 80 / 90 us for the first / second 256 workgroups of the balanced
+// schedule's 512 matrix-core workgroups in a 101 us step (raising the wave priority of the second 256 flips it to
+// 92 / 80).  So they take turns: wave priority follows the chip-wide constant-rate clock (~5 us per turn), shifted
+// by the place the workgroup probably has among the co-resident ones of its unit - workgroups i, i + 256, i + 512,
+// ... land on the same compute unit.  Called once per iteration of the matrix-core kernels' streaming loops (86 / 88
+// us afterwards, 1-2 % per step).  Not in the vector-ALU kernel: its two workgroups per unit at config 2 finish
+// together as it is, and with four per unit (1024 workgroups: 96 / 130 us for the first / last 256 of a 159 us step)
+// taking turns made the step 1-3 % slower - there the staggered finish does no harm.
+__device__ __forceinline__ void take_turns(const AttnArgs& a)
+{
+    const unsigned total = gridDim.x * gridDim.y * gridDim.z;
+    if (total <= 256 || !a.turns) return;
+    const unsigned places = total > 768 ? 4 : (total + 255) / 256;
+    const unsigned id = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    const unsigned turn = ((unsigned)(wall_clock64() >> 9) + id / 256) % places;
+    switch (turn) {
+        case 0: __builtin_amdgcn_s_setprio(0); break;
+        case 1: __builtin_amdgcn_s_setprio(1); break;
+        case 2: __builtin_amdgcn_s_setprio(2); break;
+        default: __builtin_amdgcn_s_setprio(3); break;
     }
 }
 
