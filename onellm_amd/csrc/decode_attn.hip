@@ -564,7 +564,15 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     const int item_rows = item_rows_for(dtype == ONELLM_FP16, D, G);
     const long long items = (max_t - 1 + item_rows - 1) / item_rows;
     const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);
-    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && balanced_by_default(t_dev != nullptr, on_matrix_cores(dtype == ONELLM_FP16, D, G), (long)B * nunits, wmax)))) {
+    // Equal lengths whose grid does not fill the chip evenly - between one and two workgroups per compute unit (one
+    // and one and a half on the vector-ALU kernel, which loses less when a unit holds one workgroup): some units would
+    // run two workgroups and the rest one.  One equal share per compute unit instead (measured: 40 heads x batch 8 =
+    // 320 units 116 -> 101 us; 8 kv heads x batch 10, cut in four = 320 workgroups 75 -> 59 us; 8 kv heads x batch 48
+    // = 384 units 144 -> 130 us; 384 single-head units 121.5 -> 124.6, hence the lower bound there).
+    const bool mfma_kernel = on_matrix_cores(dtype == ONELLM_FP16, D, G);
+    const long grid_wgs = base_wgs * nsplit;
+    const bool uneven_grid = !t_dev && grid_wgs > 256 && grid_wgs < (mfma_kernel ? 512 : 384) && wmax >= 2048;
+    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && (uneven_grid || balanced_by_default(t_dev != nullptr, mfma_kernel, (long)B * nunits, wmax))))) {
         a.item_rows = item_rows;
         // (what a change of unit costs a workgroup, in items: measured on the matrix-core kernel, where workgroups whose
         // equal-row shares held one / two / three units finished at 82 / 90 / 94 us of a 101 us step)
@@ -572,7 +580,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
         a.unit_cost = user_cost >= 0 ? user_cost : 3;
         const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
         const int user_wgs = tune_get("attn_balanced_wgs");
-        long long nwg = user_wgs > 0 ? user_wgs : kBalancedWorkgroups;
+        long long nwg = user_wgs > 0 ? user_wgs : (uneven_grid && bal != 1 ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
         if (nwg > kBalancedWorkgroups * 2) nwg = kBalancedWorkgroups * 2;
         // no workgroup for fewer than four items; between one and two workgroups per compute unit some units would
         // get two shares and the rest one, so one larger share each (6 sequences of 1024..4096 rows: 28.9 -> 25.3 us)

@@ -393,6 +393,29 @@ def test_fused_finish_at_full_size_matches_the_merge_launch(capi, dev):
         assert (outs[0][:nb].float() - outs[1][:nb].float()).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,t", [(9, 32, 32, 600), (36, 32, 8, 600), (5, 64, 64, 1100), (20, 16, 8, 1300)])
+@pytest.mark.parametrize("zeroed", [False, True])
+def test_equal_lengths_on_an_uneven_grid(capi, ref, dev, B, Hq, Hkv, t, zeroed):
+    """Equal lengths with between one and two workgroups per compute unit (288, 320 units; 160 units cut in two): the
+    launcher hands every compute unit one equal share of the rows instead (balanced schedule, 256 workgroups), with
+    the merge launch or - on a zeroed workspace - the fused finish."""
+    announce("attn uneven grid", B, Hq, Hkv, t, zeroed)
+    D, S = 128, t + 20
+    qkv, bias, kc, vc = _case(np.float16, B, Hq, Hkv, D, S, 1, seed=B * 7 + t, std=0.5)
+    d_qkv, d_bias = torch.from_numpy(qkv).to(dev), torch.from_numpy(bias).to(dev)
+    d_kc, d_vc = torch.from_numpy(kc).to(dev), torch.from_numpy(vc).to(dev)
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    for rep in range(2):
+        out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+        g_kc, g_vc = d_kc.clone(), d_vc.clone()
+        capi.decode_attn(d_qkv, d_bias, g_kc, g_vc, out, Hq, t, D, 10000.0, workspace=ws,
+                         flags=capi.ATTN_ZEROED_WORKSPACE if zeroed else 0)
+        r_kc, r_vc = kc.copy(), vc.copy()
+        want = ref.decode_attn(qkv, bias, r_kc, r_vc, Hq, t, D, 10000.0)
+        _assert_parity((out.cpu().numpy(), want, g_kc.cpu().numpy(), g_vc.cpu().numpy(), r_kc, r_vc), np.float16)
+        assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0, "the counter region must stay zero either way"
+
+
 def test_random_shapes_sweep(capi, ref, dev):
     """Eighty seeded random (dtype, heads, group size, head size, lengths, split count, schedule) combinations, ragged lengths
     included: every kernel variant and padded head tile gets shapes nobody picked by hand."""
