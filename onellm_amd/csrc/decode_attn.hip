@@ -571,7 +571,10 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // = 384 units 144 -> 130 us; 384 single-head units 121.5 -> 124.6, hence the lower bound there).
     const bool mfma_kernel = on_matrix_cores(dtype == ONELLM_FP16, D, G);
     const long grid_wgs = base_wgs * nsplit;
-    const bool uneven_grid = !t_dev && grid_wgs > 256 && grid_wgs < (mfma_kernel ? 512 : 384) && wmax >= 2048;
+    // (the matrix-core kernels hold two workgroups per unit at most, so any grid that is not a whole number of such
+    // rounds ends with part of the chip idle: 576 units 227 -> 190 us, 640 units 265 -> 212, 768 units 284 -> 249)
+    const bool uneven_grid = !t_dev && wmax >= 2048 && grid_wgs > 256
+                             && (mfma_kernel ? (grid_wgs % 512 != 0 && grid_wgs < 4096) : grid_wgs < 384);
     if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && (uneven_grid || balanced_by_default(t_dev != nullptr, mfma_kernel, (long)B * nunits, wmax))))) {
         a.item_rows = item_rows;
         // (what a change of unit costs a workgroup, in items: measured on the matrix-core kernel, where workgroups whose
@@ -580,7 +583,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
         a.unit_cost = user_cost >= 0 ? user_cost : 3;
         const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
         const int user_wgs = tune_get("attn_balanced_wgs");
-        long long nwg = user_wgs > 0 ? user_wgs : (uneven_grid && bal != 1 ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
+        long long nwg = user_wgs > 0 ? user_wgs : (uneven_grid && bal != 1 && grid_wgs < 512 ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
         if (nwg > kBalancedWorkgroups * 2) nwg = kBalancedWorkgroups * 2;
         // no workgroup for fewer than four items; between one and two workgroups per compute unit some units would
         // get two shares and the rest one, so one larger share each (6 sequences of 1024..4096 rows: 28.9 -> 25.3 us)

@@ -393,12 +393,14 @@ def test_fused_finish_at_full_size_matches_the_merge_launch(capi, dev):
         assert (outs[0][:nb].float() - outs[1][:nb].float()).abs().max().item() <= 1e-3
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,t", [(9, 32, 32, 600), (36, 32, 8, 600), (5, 64, 64, 1100), (20, 16, 8, 1300)])
+@pytest.mark.parametrize("B,Hq,Hkv,t", [(9, 32, 32, 600), (36, 32, 8, 600), (5, 64, 64, 1100), (20, 16, 8, 1300), (72, 32, 8, 330),
+                                        (81, 16, 8, 290)])
 @pytest.mark.parametrize("zeroed", [False, True])
 def test_equal_lengths_on_an_uneven_grid(capi, ref, dev, B, Hq, Hkv, t, zeroed):
-    """Equal lengths with between one and two workgroups per compute unit (288, 320 units; 160 units cut in two): the
-    launcher hands every compute unit one equal share of the rows instead (balanced schedule, 256 workgroups), with
-    the merge launch or - on a zeroed workspace - the fused finish."""
+    """Equal lengths with a grid that does not fill the chip evenly (288, 320 units; 160 units cut in two; 576 and 648
+    grouped-query units on the matrix-core kernel, which holds two workgroups per compute unit): the launcher hands
+    the compute units equal shares of the rows instead (balanced schedule, 256 or 512 workgroups), with the merge
+    launch or - on a zeroed workspace - the fused finish."""
     announce("attn uneven grid", B, Hq, Hkv, t, zeroed)
     D, S = 128, t + 20
     qkv, bias, kc, vc = _case(np.float16, B, Hq, Hkv, D, S, 1, seed=B * 7 + t, std=0.5)
