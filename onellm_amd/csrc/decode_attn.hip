@@ -436,19 +436,22 @@ int item_rows_for(bool fp16, int D, int G)
 }
 
 // When the balanced schedule is the default (tuning knob attn_balanced = 1 / 0 forces it on / off): per-sequence
-// lengths on the matrix-core kernel with no more units than workgroups.  Measured on MI355X against the grid
-// schedule (us per step, lengths uniform in [S/8, S]): 32 q / 8 kv heads, batch 32, S 8192: 117 -> 102; 64 q / 8 kv,
-// batch 16: 81 -> 57; batch 8, S 16384: 97 -> 61; D = 256, batch 16, S 4096: 90 -> 74.  With equal lengths the grid
-// schedule needs no merge launch and is as fast or faster; with more units than workgroups (batch 128) and on the
-// vector-ALU kernel (which keeps four workgroups per compute unit resident) the hardware dispatcher balances the
-// grid schedule's chunks as well as the fixed shares do.  Nor for a small step (fewer than kBalancedMinItems items
+// lengths on the matrix-core kernels.  Measured on MI355X against the grid schedule (us per step, lengths uniform
+// in [S/8, S]): 32 q / 8 kv heads, batch 32, S 8192: 117 -> 98; 64 q / 8 kv, batch 16: 81 -> 57; batch 8, S 16384:
+// 97 -> 61; D = 256, batch 16, S 4096: 90 -> 64; and, since the shares are equal in cost, with more units than
+// workgroups too: batch 72, S 4096: 131 -> 118; batch 96, S 2048: 101 -> 87; batch 256, S 1024: 155 -> 118.  With
+// equal lengths a grid that fills the chip evenly needs no merge and is as fast or faster; on the vector-ALU kernel
+// (which keeps four workgroups per compute unit resident) the hardware dispatcher balances the grid schedule's
+// chunks about as well as the fixed shares do (batch 24 x 32 heads: 157.5 / 153.8; batch 16: 94.4 / 97.4).  Nor for
+// a small step (fewer than kBalancedMinItems items
 // if every length were the longest): the walk's set-up and its serial unit changes are then most of the time and
 // the grid schedule with the fused finish is faster (8 sequences of 256..2048 rows: 24.9 against 17.6 us; 4 of
 // 512..4096: 25.2 / 19.6; even at 3500..4100 items; the balanced schedule is ahead from ~7000: 16 sequences of
 // 1024..8192 rows 56.7 / 67.6).
 bool balanced_by_default(bool ragged, bool mfma, long units, long long max_items)
 {
-    return ragged && mfma && units <= kBalancedWorkgroups && max_items >= kBalancedMinItems;
+    (void)units;
+    return ragged && mfma && max_items >= kBalancedMinItems;
 }
 
 int max_splits(int max_t)
