@@ -348,6 +348,10 @@ def extras_section(capi, dev, args, with_cpu):
     ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, 8, 64, Hkv3, D, S3, S3, nsets=3, fp32=True)
     ex["decode_attn_gqa_fused_fp32_b8_q64_kv8_len8192"] = entry(ms_u, attn_bytes(8, 64, Hkv3, D, [S3] * 8, 4))
     torch.cuda.empty_cache()
+    # config 2's shape with fp32 caches at batch 8 (the same bytes as the headline): the reference's own element type
+    ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, 8, 32, 32, D, 4096, 4096, nsets=3, fp32=True)
+    ex["decode_attn_fp32_b8_h32_ctx4096"] = entry(ms_u, attn_bytes(8, 32, 32, D, [4096] * 8, 4))
+    torch.cuda.empty_cache()
     # the reference-style path on the same data: concat the new row, repeat KV to 32 heads, attend over 32 heads
     hist = (t_dev - 1).contiguous()
     ones = torch.ones(B3, dtype=torch.int32, device=dev)
