@@ -418,6 +418,27 @@ def test_equal_lengths_on_an_uneven_grid(capi, ref, dev, B, Hq, Hkv, t, zeroed):
         assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0, "the counter region must stay zero either way"
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,D,t", [(1, 32, 8, 128, 8192), (2, 32, 8, 128, 8192), (1, 64, 8, 128, 8192), (1, 32, 32, 128, 4096),
+                                          (1, 16, 2, 256, 6000), (1, 16, 16, 64, 8192)])
+def test_long_sequences_of_a_small_batch(capi, ref, dev, B, Hq, Hkv, D, t):
+    """One or two long sequences: every unit is cut into up to 64 pieces and finished inside the kernel by the piece
+    that arrives last (on a zeroed workspace) - with many pieces through the LDS-staged form of that merge - or by
+    the merge launch; both against the oracle."""
+    announce("attn long sequence, small batch", B, Hq, Hkv, D, t)
+    S = t
+    qkv, bias, kc, vc = _case(np.float16, B, Hq, Hkv, D, S, 1, seed=t + Hq, std=0.5)
+    d_qkv, d_bias = torch.from_numpy(qkv).to(dev), torch.from_numpy(bias).to(dev)
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    r_kc, r_vc = kc.copy(), vc.copy()
+    want = ref.decode_attn(qkv, bias, r_kc, r_vc, Hq, t, D, 10000.0)
+    for flags in (capi.ATTN_ZEROED_WORKSPACE, capi.ATTN_ZEROED_WORKSPACE, 0):
+        d_kc, d_vc = torch.from_numpy(kc).to(dev), torch.from_numpy(vc).to(dev)
+        out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+        capi.decode_attn(d_qkv, d_bias, d_kc, d_vc, out, Hq, t, D, 10000.0, workspace=ws, flags=flags)
+        _assert_parity((out.cpu().numpy(), want, d_kc.cpu().numpy(), d_vc.cpu().numpy(), r_kc, r_vc), np.float16)
+        assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0
+
+
 def test_random_shapes_sweep(capi, ref, dev):
     """Eighty seeded random (dtype, heads, group size, head size, lengths, split count, schedule) combinations, ragged lengths
     included: every kernel variant and padded head tile gets shapes nobody picked by hand."""
