@@ -439,6 +439,42 @@ def test_long_sequences_of_a_small_batch(capi, ref, dev, B, Hq, Hkv, D, t):
         assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0
 
 
+def test_default_dispatch_at_medium_sizes(capi, ref, dev):
+    """Sixteen seeded shapes of a few hundred units and a few thousand rows, equal and per-sequence lengths, with and
+    without a zeroed workspace, no tuning keys: whatever schedule the launcher picks by itself (grid with or without a
+    split, equal shares on an uneven grid, balanced walk, merge launch or fused finish) gives the oracle's result."""
+    rng = np.random.default_rng(20240)
+    for case in range(16):
+        dtype = [np.float16, np.float16, np.float32][int(rng.integers(0, 3))]
+        D = int(rng.choice([64, 128, 128, 256]))
+        if dtype == np.float32 and D == 256:
+            D = 128
+        Hkv = int(rng.choice([2, 4, 8, 8, 32, 40]))
+        G = int(rng.choice([1, 4, 8, 5])) if Hkv <= 8 else 1
+        Hq = Hkv * G
+        B = int(rng.integers(1, 17 if Hkv >= 32 else 41))
+        tmax = int(rng.integers(200, 1801))
+        S = tmax + int(rng.integers(0, 64))
+        ragged = bool(rng.integers(0, 2))
+        lens = rng.integers(max(1, tmax // 8), tmax + 1, size=B) if ragged else np.full(B, tmax)
+        lens[int(rng.integers(0, B))] = tmax
+        zeroed = bool(rng.integers(0, 2))
+        announce("attn default dispatch", case, dtype.__name__, "B", B, "Hq", Hq, "Hkv", Hkv, "D", D, "t", tmax, "ragged", ragged, "zeroed", zeroed)
+        qkv, bias, kc, vc = _case(dtype, B, Hq, Hkv, D, S, 1, seed=7000 + case, std=0.5)
+        d_qkv, d_bias = torch.from_numpy(qkv).to(dev), torch.from_numpy(bias).to(dev)
+        d_kc, d_vc = torch.from_numpy(kc).to(dev), torch.from_numpy(vc).to(dev)
+        out = torch.zeros(B, Hq * D, dtype=d_qkv.dtype, device=dev)
+        ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+        t_dev = torch.from_numpy(lens.astype(np.int32)).to(dev) if ragged else None
+        for _ in range(2):                                       # (twice on one workspace: the counters must come back to zero)
+            capi.decode_attn(d_qkv, d_bias, d_kc, d_vc, out, Hq, tmax, D, 10000.0, t_dev=t_dev, max_t=tmax,
+                             flags=capi.ATTN_ZEROED_WORKSPACE if zeroed else 0, workspace=ws)
+        r_kc, r_vc = kc.copy(), vc.copy()
+        want = ref.decode_attn(qkv, bias, r_kc, r_vc, Hq, lens if ragged else tmax, D, 10000.0)
+        _assert_parity((out.cpu().numpy(), want, d_kc.cpu().numpy(), d_vc.cpu().numpy(), r_kc, r_vc), dtype)
+        assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0
+
+
 def test_random_shapes_sweep(capi, ref, dev):
     """Eighty seeded random (dtype, heads, group size, head size, lengths, split count, schedule) combinations, ragged lengths
     included: every kernel variant and padded head tile gets shapes nobody picked by hand."""
