@@ -53,6 +53,16 @@ int onellm_hip_version(void);
 const char* onellm_error_string(int code);
 
 /*
+ * Sets a launch-selection key for benchmarks and sweeps (for instance "attn_nsplit", "attn_balanced",
+ * "attn_balanced_wgs", "attn_balanced_cost", "attn_fused_finish", "attn_turns", "attn_target_wgs",
+ * "attn_gqa_valu", "norm_tpr", "prefill_generic"); value -1 hands the choice back to the launcher.
+ * Process-wide, read at launch time.  The keys are not part of the stable interface: no caller
+ * needs them, results never depend on them beyond rounding, and an unknown key returns
+ * ONELLM_EINVAL.  No counterpart in the reference.
+ */
+int onellm_tune_set(const char* key, int value);
+
+/*
  * Fused masked decoder self-attention for ONE new token per sequence.
  * Replaces launchDecoderMaskedMHA + masked_MHA_kernel
  * (src/kernels/decoder_masked_attn.h:7-14, src/kernels/decoder_masked_attn.cu:136-327).

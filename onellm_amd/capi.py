@@ -22,6 +22,7 @@ _vp, _ci, _cf, _cu, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.
 SYMBOLS = {
     "onellm_hip_version": (_ci, []),
     "onellm_error_string": (ctypes.c_char_p, [_ci]),
+    "onellm_tune_set": (_ci, [ctypes.c_char_p, _ci]),
     "onellm_decode_attn": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp, _ci,
                                  _ci, _cf, _ci, _cu, _vp, _sz, _vp]),
     "onellm_decode_attn_workspace_bytes": (_sz, [_ci, _ci, _ci, _ci, _ci]),
@@ -65,8 +66,6 @@ def lib():
             fn = getattr(L, name)
             fn.restype = res
             fn.argtypes = args
-        L.onellm_tune_set.restype = _ci
-        L.onellm_tune_set.argtypes = [ctypes.c_char_p, _ci]
         _lib = L
     return _lib
 
