@@ -354,11 +354,13 @@ int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 constexpr bool mfma_head_size(int D) { return D == 64 || D == 128 || D == 256; }
 
 // shapes that run on the matrix cores: fp16 caches with two or more query heads per kv head at those head
-// sizes; fp32 caches at D = 64 or 128 with more than four (up to four the vector ALU keeps up with the stream)
+// sizes (three or more at D = 256, where the kernel has one register buffer and one wave per SIMD: with two heads
+// the vector ALU is 3-5 % faster - 16 q / 8 kv heads, batch 32, 4096 rows: 152.7 against 157.4 us; with four it
+// is 13 % slower); fp32 caches at D = 64 or 128 with more than four (up to four the vector ALU keeps up with the stream)
 bool on_matrix_cores(bool fp16, int D, int G)
 {
     if (tune_get("attn_gqa_valu") == 1) return false;
-    return fp16 ? (G > 1 && mfma_head_size(D)) : (G > 4 && (D == 128 || D == 64));
+    return fp16 ? (G > 1 && mfma_head_size(D) && !(D == 256 && G == 2)) : (G > 4 && (D == 128 || D == 64));
 }
 
 // query heads one workgroup serves (they share every K/V row it reads)
@@ -587,6 +589,9 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
         const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
         const int user_wgs = tune_get("attn_balanced_wgs");
         long long nwg = user_wgs > 0 ? user_wgs : (uneven_grid && bal != 1 && grid_wgs < 512 ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
+        // (the matrix-core kernel for D = 256 keeps one workgroup per compute unit resident: a second 256 would only
+        // queue behind the first - 16 sequences of 512..4096 rows x 4 kv heads: 65.7 -> 47.1 us)
+        if (user_wgs <= 0 && mfma_kernel && dtype == ONELLM_FP16 && D == 256 && nwg > kBalancedWorkgroups / 2) nwg = kBalancedWorkgroups / 2;
         if (nwg > kBalancedWorkgroups * 2) nwg = kBalancedWorkgroups * 2;
         // no workgroup for fewer than four items; between one and two workgroups per compute unit some units would
         // get two shares and the rest one, so one larger share each (6 sequences of 1024..4096 rows: 28.9 -> 25.3 us)
