@@ -353,21 +353,21 @@ int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 // head sizes the matrix-core kernel is built for (fp16 caches)
 constexpr bool mfma_head_size(int D) { return D == 64 || D == 128 || D == 256; }
 
-// shapes that run on the matrix cores: fp16 caches with two or more query heads per kv head at those head
-// sizes (three or more at D = 256, where the kernel has one register buffer and one wave per SIMD: with two heads
-// the vector ALU is 3-5 % faster - 16 q / 8 kv heads, batch 32, 4096 rows: 152.7 against 157.4 us; with four it
-// is 13 % slower); fp32 caches at D = 64 or 128 with more than four (up to four the vector ALU keeps up with the stream)
+// shapes that run on the matrix cores: fp16 caches with three or more query heads per kv head at those head
+// sizes (with two the vector ALU keeps up with the stream and is as fast or faster: 16 q / 8 kv heads, 8192 rows,
+// D = 128, batch 32: 152.8 against 154.4 us; D = 64: 78.9 against 86.8; D = 256, 4096 rows: 152.7 against 157.4 -
+// with four heads it is 13 % slower); fp32 caches at D = 64 or 128 with more than four
 bool on_matrix_cores(bool fp16, int D, int G)
 {
     if (tune_get("attn_gqa_valu") == 1) return false;
-    return fp16 ? (G > 1 && mfma_head_size(D) && !(D == 256 && G == 2)) : (G > 4 && (D == 128 || D == 64));
+    return fp16 ? (G > 2 && mfma_head_size(D)) : (G > 4 && (D == 128 || D == 64));
 }
 
 // query heads one workgroup serves (they share every K/V row it reads)
 int heads_per_tile(bool fp16, int D, int G)
 {
     if (G == 1) return 1;       // one head: memory-bound on either kernel (measured equal), keep the lighter one
-    // two or more query heads per kv head, fp16: both products on the matrix cores, where up to 16
+    // three or more query heads per kv head, fp16: both products on the matrix cores, where up to 16
     // heads cost the same as 4 (8 at D = 256: the per-wave states of 16 heads would not fit 64 KiB of LDS)
     if (on_matrix_cores(fp16, D, G)) {
         const int cap = D == 256 ? 8 : 16;
@@ -450,10 +450,10 @@ int item_rows_for(bool fp16, int D, int G)
 // the grid schedule with the fused finish is faster (8 sequences of 256..2048 rows: 24.9 against 17.6 us; 4 of
 // 512..4096: 25.2 / 19.6; even at 3500..4100 items; the balanced schedule is ahead from ~7000: 16 sequences of
 // 1024..8192 rows 56.7 / 67.6).
-bool balanced_by_default(bool ragged, bool mfma, long units, long long max_items)
+bool balanced_by_default(bool ragged, bool mfma, int G, long long max_items)
 {
-    (void)units;
-    return ragged && mfma && max_items >= kBalancedMinItems;
+    // (two heads per kv head on the vector-ALU kernel: 32 sequences of 1024..8192 rows 105.4 -> 98.1 us; one head: +-3 %)
+    return ragged && (mfma || G == 2) && max_items >= kBalancedMinItems;
 }
 
 int max_splits(int max_t)
@@ -530,7 +530,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     const long base_wgs = (long)B * Hkv * ngt;
     const int user_target = tune_get("attn_target_wgs");
     // (the matrix-core kernel at D = 64 has half the bytes in flight per workgroup: two per compute unit)
-    const bool mfma64 = dtype == ONELLM_FP16 && D == 64 && G > 1 && tune_get("attn_gqa_valu") != 1;
+    const bool mfma64 = D == 64 && on_matrix_cores(dtype == ONELLM_FP16, D, G) && dtype == ONELLM_FP16;
     const int target = user_target > 0 ? user_target : (t_dev ? 4096 : (mfma64 ? 512 : 256));
     int nsplit = (int)((target + base_wgs - 1) / base_wgs);
     int cap = max_splits(max_t);
@@ -580,7 +580,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // rounds ends with part of the chip idle: 576 units 227 -> 190 us, 640 units 265 -> 212, 768 units 284 -> 249)
     const bool uneven_grid = !t_dev && wmax >= 2048 && grid_wgs > 256
                              && (mfma_kernel ? (grid_wgs % 512 != 0 && grid_wgs < 4096) : grid_wgs < 384);
-    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && (uneven_grid || balanced_by_default(t_dev != nullptr, mfma_kernel, (long)B * nunits, wmax))))) {
+    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && (uneven_grid || balanced_by_default(t_dev != nullptr, mfma_kernel, G, wmax))))) {
         a.item_rows = item_rows;
         // (what a change of unit costs a workgroup, in items: measured on the matrix-core kernel, where workgroups whose
         // equal-row shares held one / two / three units finished at 82 / 90 / 94 us of a 101 us step)
