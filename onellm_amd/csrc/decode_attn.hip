@@ -452,8 +452,12 @@ int item_rows_for(bool fp16, int D, int G)
 // 1024..8192 rows 56.7 / 67.6).
 bool balanced_by_default(bool ragged, bool mfma, int G, long long max_items)
 {
-    // (two heads per kv head on the vector-ALU kernel: 32 sequences of 1024..8192 rows 105.4 -> 98.1 us; one head: +-3 %)
-    return ragged && (mfma || G == 2) && max_items >= kBalancedMinItems;
+    // (two heads per kv head on the vector-ALU kernel: 32 sequences of 1024..8192 rows 105.4 -> 98.1 us.  One head,
+    // where the dispatcher keeps four workgroups per compute unit busy with the grid schedule's chunks: a tie up to
+    // ~16000 items, then 3-6 % - 16 sequences x 32 heads of 512..4096 rows 105 -> 100 us, 64 of 128..2048: 184 -> 174)
+    if (!ragged) return false;
+    if (mfma || G == 2) return max_items >= kBalancedMinItems;
+    return max_items >= 16384;
 }
 
 int max_splits(int max_t)
