@@ -32,6 +32,7 @@ extern "C" {
 #define ONELLM_EINVAL      (-1)  /* null pointer, non-positive size, bad enum  */
 #define ONELLM_EUNSUPPORTED (-2) /* shape outside what the kernels are built for */
 #define ONELLM_EWORKSPACE  (-3)  /* workspace missing or too small              */
+#define ONELLM_ESCRATCH    (-4)  /* onellm_decode_attn_static: the step needs more than the built-in scratch */
 
 /* flags for onellm_decode_attn */
 #define ONELLM_ATTN_NO_V_BIAS     0x1u /* skip the v-bias add (reference decode kernel behaviour,
@@ -108,6 +109,28 @@ int onellm_decode_attn(int dtype,
 
 /* Bytes of workspace onellm_decode_attn needs for these sizes (0 never; at least 256). */
 size_t onellm_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int max_t);
+
+/*
+ * onellm_decode_attn for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, results and kernels as onellm_decode_attn, minus the workspace: split partials and
+ * arrival counters live in a fixed device array inside the library,
+ * ONELLM_DECODE_ATTN_STATIC_SCRATCH_BYTES (16 MiB) per GPU, held from library load to process exit.
+ * The call allocates, frees and synchronises nothing.  The first call on a GPU also queues one small
+ * kernel on `stream` that clears the counter region.  A step whose partials do not fit returns
+ * ONELLM_ESCRATCH before anything is launched (onellm_decode_attn_workspace_bytes() is an upper bound
+ * of what a step may need; steps that are not split need nothing).  All calls on one GPU share the
+ * array, so calls that overlap in time on one GPU (two streams, two threads) race: serialise them.
+ */
+#define ONELLM_DECODE_ATTN_STATIC_SCRATCH_BYTES (16u << 20)
+int onellm_decode_attn_static(int dtype,
+                              const void* qkv, const void* qkv_bias,
+                              void* k_cache, void* v_cache, void* out,
+                              int B, int Hq, int Hkv, int D, int S,
+                              int layer, int num_layers,
+                              int t_host, const int* t_dev, int max_t,
+                              int rotary_dim, float rope_base, int rope_pos_offset,
+                              unsigned flags, onellm_stream_t stream);
 
 /*
  * In-place RMSNorm over rows: x <- gamma * x * rsqrt(mean(x^2) + eps).

@@ -11,7 +11,8 @@ LIB_PATH = os.path.join(_HERE, "libonellm_hip.so")
 LAUNCHERS_PATH = os.path.join(_HERE, "libonellm_launchers.so")
 
 FP32, FP16 = 0, 1
-EINVAL, EUNSUPPORTED, EWORKSPACE = -1, -2, -3
+EINVAL, EUNSUPPORTED, EWORKSPACE, ESCRATCH = -1, -2, -3, -4
+DECODE_ATTN_STATIC_SCRATCH_BYTES = 16 << 20
 ATTN_NO_V_BIAS = 0x1
 ATTN_NO_CACHE_WRITE = 0x2
 ATTN_ZEROED_WORKSPACE = 0x4
@@ -26,6 +27,8 @@ SYMBOLS = {
     "onellm_decode_attn": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp, _ci,
                                  _ci, _cf, _ci, _cu, _vp, _sz, _vp]),
     "onellm_decode_attn_workspace_bytes": (_sz, [_ci, _ci, _ci, _ci, _ci]),
+    "onellm_decode_attn_static": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp, _ci,
+                                        _ci, _cf, _ci, _cu, _vp]),
     "onellm_rmsnorm": (_ci, [_ci, _vp, _vp, _cf, _ci, _ci, _vp]),
     "onellm_fused_add_bias_residual_rmsnorm": (_ci, [_ci, _vp, _vp, _vp, _vp, _cf, _ci, _ci, _vp]),
     "onellm_kv_append": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp]),
@@ -124,6 +127,21 @@ def decode_attn(qkv, bias, k_cache, v_cache, out, Hq, t, rotary_dim, rope_base, 
                                   rotary_dim, rope_base, rope_pos_offset, flags,
                                   _ptr(workspace), workspace.numel(), _stream())
     _check(rc, "onellm_decode_attn")
+    return out
+
+
+def decode_attn_static(qkv, bias, k_cache, v_cache, out, Hq, t, rotary_dim, rope_base, layer=0, t_dev=None,
+                       max_t=None, rope_pos_offset=0, flags=0):
+    """decode_attn through the entry point that uses the library's built-in scratch (allocates nothing)."""
+    B, QKVH, D = qkv.shape
+    L, _, Hkv, S, _ = k_cache.shape
+    assert QKVH == Hq + 2 * Hkv
+    if max_t is None:
+        max_t = t
+    rc = lib().onellm_decode_attn_static(_dt(qkv), _ptr(qkv), _ptr(bias), _ptr(k_cache), _ptr(v_cache), _ptr(out),
+                                         B, Hq, Hkv, D, S, layer, L, int(t), _ptr(t_dev), int(max_t),
+                                         rotary_dim, rope_base, rope_pos_offset, flags, _stream())
+    _check(rc, "onellm_decode_attn_static")
     return out
 
 

@@ -36,7 +36,8 @@ int tune_get(const char* key)
 }  // namespace onellm
 
 // 1.1: ONELLM_ATTN_ZEROED_WORKSPACE, 64 KiB of arrival counters at the front of the attention workspace
-extern "C" int onellm_hip_version(void) { return 1001; }
+// 1.2: onellm_decode_attn_static
+extern "C" int onellm_hip_version(void) { return 1002; }
 
 extern "C" int onellm_tune_set(const char* key, int value)
 {
@@ -56,6 +57,8 @@ extern "C" const char* onellm_error_string(int code)
         case ONELLM_EINVAL: return "onellm: invalid argument (null pointer, non-positive size or unknown enum)";
         case ONELLM_EUNSUPPORTED: return "onellm: shape or alignment not supported by the gfx950 kernels";
         case ONELLM_EWORKSPACE: return "onellm: workspace missing or too small";
+        case ONELLM_ESCRATCH: return "onellm: the step's split partials exceed the library's built-in scratch "
+                                     "(ONELLM_DECODE_ATTN_STATIC_SCRATCH_BYTES); use onellm_decode_attn with a workspace";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));

@@ -20,7 +20,8 @@ def test_header_declares_the_expected_entry_points():
     for must in ["onellm_decode_attn", "onellm_decode_attn_workspace_bytes", "onellm_rmsnorm",
                  "onellm_fused_add_bias_residual_rmsnorm", "onellm_kv_append", "onellm_kv_repeat",
                  "onellm_beam_topk", "onellm_beam_topk_workspace_bytes", "onellm_error_string", "onellm_hip_version",
-                 "onellm_qkv_bias_rope_transpose", "onellm_silu_and_mul", "onellm_topk_sample"]:
+                 "onellm_qkv_bias_rope_transpose", "onellm_silu_and_mul", "onellm_topk_sample",
+                 "onellm_decode_attn_static"]:
         assert must in names
 
 
@@ -53,6 +54,7 @@ def test_version_and_error_strings(capi):
     assert L.onellm_hip_version() >= 1000
     assert b"invalid argument" in L.onellm_error_string(capi.EINVAL)
     assert b"workspace" in L.onellm_error_string(capi.EWORKSPACE)
+    assert b"built-in scratch" in L.onellm_error_string(capi.ESCRATCH)
     assert L.onellm_error_string(0) == b"success"
     assert L.onellm_error_string(-99)
 
