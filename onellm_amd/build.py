@@ -41,6 +41,12 @@ LAYER_SOURCES = ["layers.cpp", "layers_capi.cpp"]
 # what the kernels are written in)
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC, "-Wall", "-Wno-unused-function"]
 DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# Kernels whose workgroups live a few microseconds get their first kernel arguments handed over in scalar
+# registers at wave launch instead of fetching them first (gfx950 kernel-argument preload, up to 16 dwords;
+# the code object keeps the ordinary fetch as its entry for a loader that does not preload).  Measured on
+# MI355X: RMSNorm 8192 x 4096 fp16 22.2 -> 21.7 us.
+PRELOAD_KERNARGS = ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
+PRELOAD_SOURCES = {"norms.hip", "activation.hip", "kv_cache.hip", "prefill_rope.hip"}
 
 
 def _newer(target, deps):
@@ -67,6 +73,8 @@ def _compile(src, force):
         # (the compiler's per-kernel register / occupancy / scratch remarks are kept next to the object:
         # tests/test_kernel_resources.py holds the kernels to their budgets)
         cmd += DEVICE + ["-Rpass-analysis=kernel-resource-usage"]
+        if src in PRELOAD_SOURCES and os.environ.get("ONELLM_NO_KERNARG_PRELOAD") != "1":
+            cmd += PRELOAD_KERNARGS
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr[-4000:]))

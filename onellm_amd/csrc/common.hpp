@@ -104,6 +104,18 @@ __device__ __forceinline__ void store16_stream(T* p, const Vec16<T>& v)
 {
     __builtin_nontemporal_store(v.raw, reinterpret_cast<decltype(v.raw)*>(p));
 }
+// 16 bytes written through to memory (the sc1 bit), with or without the non-temporal hint.  Pays where stores
+// dominate - measured on MI355X against the non-temporal hint alone: the KV repeat (one load, G stores) 8 % faster
+// with sc1 + nt (sc1 alone: 2 %), a prefill-sized KV append 12 % faster with sc1 alone (sc1 + nt: 7 %), an in-place
+// read-modify-write stream 2 % with sc1 + nt.  Kernels that read two streams per stream written (SwiGLU, the
+// prefill transpose) are 0.5-2 % slower with either and keep the plain non-temporal store.
+typedef float stream_f32x4 __attribute__((ext_vector_type(4)));
+template <bool NT>
+__device__ __forceinline__ void store16_write_through(void* p, stream_f32x4 v)
+{
+    if constexpr (NT) asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(p), "v"(v) : "memory");
+    else asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
 
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(__half v) { return __half2float(v); }

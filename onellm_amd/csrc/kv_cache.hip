@@ -11,6 +11,14 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // COPY is the access type: 16 bytes on the normal path, the element itself otherwise.
+// a piece stored for a reader that comes much later: 16-byte pieces written through, smaller ones non-temporal
+template <bool NT, typename COPY>
+__device__ __forceinline__ void store_piece(COPY* p, const COPY& v)
+{
+    if constexpr (sizeof(COPY) == 16) store16_write_through<NT>(p, __builtin_bit_cast(stream_f32x4, v));
+    else __builtin_nontemporal_store(v, p);
+}
+
 template <typename COPY>
 __global__ __launch_bounds__(256)
 void kv_append_kernel(const COPY* __restrict__ k_src, const COPY* __restrict__ v_src,
@@ -29,8 +37,8 @@ void kv_append_kernel(const COPY* __restrict__ k_src, const COPY* __restrict__ v
     const COPY* src = blockIdx.z ? v_src : k_src;
     COPY* dst = blockIdx.z ? v_cache : k_cache;
     // streamed once in, once out: keep it out of the way of reusable cache lines
-    __builtin_nontemporal_store(__builtin_nontemporal_load(&src[((size_t)bh * max_q_len + tau) * rowv + c]),
-                                &dst[slab + ((size_t)bh * S + (size_t)drow) * rowv + c]);
+    store_piece<false>(&dst[slab + ((size_t)bh * S + (size_t)drow) * rowv + c],
+                __builtin_nontemporal_load(&src[((size_t)bh * max_q_len + tau) * rowv + c]));
 }
 
 template <typename COPY>
@@ -54,7 +62,7 @@ void kv_repeat_kernel(const COPY* __restrict__ k_cache, const COPY* __restrict__
     const COPY val = __builtin_nontemporal_load(&src[slab + ((size_t)bh * S + s) * rowv + c]);
     const size_t Hq = (size_t)Hkv * G;
     size_t o = (((size_t)b * Hq + (size_t)kvh * G) * max_k_len + s) * rowv + c;
-    for (int g = 0; g < G; ++g, o += (size_t)max_k_len * rowv) __builtin_nontemporal_store(val, &dst[o]);
+    for (int g = 0; g < G; ++g, o += (size_t)max_k_len * rowv) store_piece<true>(&dst[o], val);
 }
 
 struct CopyPlan {

@@ -1,173 +1,184 @@
 // RMSNorm and fused add-bias-residual-RMSNorm for gfx950.
 //
-// Both are one-pass row kernels: a row is read from HBM once with 16-byte loads, kept in
-// registers, reduced with DPP (plus one LDS hop when more than one wave shares a row), scaled
-// and written back.  Algorithmic traffic: RMSNorm 2*N*H*e + H*e bytes, fused 4*N*H*e + 2*H*e.
-// A row is owned by TPR threads (64 = one wave per row, no barrier at all; 256 or 1024 = one
-// workgroup per row) holding NV 16-byte vectors each.
+// Both are one-pass row kernels: a row is read from HBM once with 16-byte loads, kept in registers, reduced with
+// DPP (plus one LDS hop when more than one wave shares a row), scaled and written back.  Algorithmic traffic:
+// RMSNorm 2*N*H*e + H*e bytes, fused 4*N*H*e + 2*H*e.  A row is owned by a team of TPR threads holding NV 16-byte
+// vectors each: one wave (no barrier at all) or two waves for short rows, several teams to a 256-thread workgroup;
+// a whole workgroup of 256, 512 or 1024 threads for rows of more than 128 vectors.
 #include "common.hpp"
 
 namespace onellm {
 namespace {
 
-// Sums over the TPR threads that share a row, for RPT rows at once; smem holds RPT floats per
-// wave of the block.  Teams of a block reach the barrier together (callers keep whole blocks alive).
-template <int TPR, int RPT>
-__device__ __forceinline__ void row_sums(float (&v)[RPT], float* smem, int tid)
+// ---------------------------------------------------------------- buffer accesses
+//
+// A team of TPR threads per row, NV vectors per thread.  Loads and stores are raw buffer accesses whose
+// descriptor covers exactly the row, so a lane past the row's end reads zeros and stores nothing - there is no
+// branch anywhere - and the cache policy is chosen per access: the row is read non-temporally and written
+// non-temporally + write-through (measured on MI355X with a read-reduce-write kernel of this shape over 64 MiB:
+// 24.6 us with plain accesses, 21.5 us non-temporal both ways, 21.1 us with the write-through bit on the store).
+// The arithmetic is kept to what the memory pipeline leaves room for: the sum of squares of fp16 pairs is one
+// dot instruction per pair (exact products, fp32 accumulation), gamma is folded into the row's scale once
+// (gamma * inv as a mixed-precision fma on the stored fp16 value), and the result is one mixed-precision fma and
+// half a packed conversion per element.
+
+constexpr int kAuxPlain = 0;
+constexpr int kAuxStreamLoad = 2;        // nt
+constexpr int kAuxStreamStore = 2 | 16;  // nt + sc1
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_descriptor(const void* base, unsigned bytes)
 {
-#pragma unroll
-    for (int k = 0; k < RPT; ++k) v[k] = wave_sum(v[k]);
-    if constexpr (TPR > kWave) {
-        constexpr int NWAVE = TPR / kWave;
-        const int wave = tid / kWave;
-        if ((tid & (kWave - 1)) == 0) {
-#pragma unroll
-            for (int k = 0; k < RPT; ++k) smem[wave * RPT + k] = v[k];
-        }
-        __syncthreads();
-        const int first = wave / NWAVE * NWAVE;
-#pragma unroll
-        for (int k = 0; k < RPT; ++k) {
-            float s = 0.f;
-#pragma unroll
-            for (int w = 0; w < NWAVE; ++w) s += smem[(first + w) * RPT + k];
-            v[k] = s;
-        }
-    }
+    // raw buffer (stride 0): an access is dropped when offset + size exceeds `bytes`
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
-// A team of TPR threads owns RPT rows at a time and each thread holds NV 16-byte vectors of each:
-// all RPT*NV loads (twice that when FUSED) are issued before anything is consumed, so a thread
-// keeps up to 8 KiB-per-wave-sized bursts in flight; then one reduction serves the RPT rows.
-// FUSED selects the add-bias-residual form at compile time.
-template <typename T, int NV, int TPR, int RPT, bool FUSED>
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T, int AUX>
+__device__ __forceinline__ Vec16<T> buffer_load16(__amdgpu_buffer_rsrc_t r, unsigned byte_offset)
+{
+    Vec16<T> v;
+    v.raw = __builtin_bit_cast(decltype(v.raw), __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_offset, 0, AUX));
+    return v;
+}
+template <typename T, int AUX>
+__device__ __forceinline__ void buffer_store16(__amdgpu_buffer_rsrc_t r, unsigned byte_offset, const Vec16<T>& v)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v.raw), r, (int)byte_offset, 0, AUX);
+}
+
+// sum of the squares of the 16 bytes' elements, added to acc
+__device__ __forceinline__ float sum_squares(const Vec16<float>& v, float acc)
+{
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = fmaf(v.raw[e], v.raw[e], acc);
+    return acc;
+}
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float sum_squares(const Vec16<__half>& v, float acc)
+{
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+        const f16x2 pr = {v.raw[e], v.raw[e + 1]};
+        acc = __builtin_amdgcn_fdot2(pr, pr, acc, false);
+    }
+    return acc;
+}
+
+// Total over the wave, valid in lane 63 only: row sums by DPP, then the two row broadcasts.
+__device__ __forceinline__ float wave_sum_in_last_lane(float v)
+{
+    v += dpp_f32<kDppQuadXor1>(v);
+    v += dpp_f32<kDppQuadXor2>(v);
+    v += dpp_f32<kDppRowHalfMirror>(v);
+    v += dpp_f32<kDppRowMirror>(v);
+    // row_bcast:15 into rows 1 and 3, row_bcast:31 into rows 2 and 3 (lanes of the other rows keep their value)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));
+    return v;
+}
+
+template <typename T, int NV, int TPR, bool FUSED>
 __global__ __launch_bounds__(TPR > 256 ? TPR : 256)
-void norm_rows_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __restrict__ bias,
-                      const T* __restrict__ gamma, float eps, int N, int H)
+void norm_row_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __restrict__ bias,
+                     const T* __restrict__ gamma, float eps, int N, int H)
 {
     constexpr int VEC = Elt<T>::kVec;
     constexpr int BLOCK = TPR > 256 ? TPR : 256;
-    constexpr int TPB = BLOCK / TPR;             // teams per block
-    __shared__ float smem[BLOCK / kWave * RPT];
+    constexpr int TPB = BLOCK / TPR;              // teams (rows) per workgroup
+    constexpr int NWAVE = TPR / kWave;            // waves per team
+    __shared__ float smem[BLOCK / kWave];
     const int tid = threadIdx.x;
     const int lane = tid % TPR;
-    const int row0 = (blockIdx.x * TPB + tid / TPR) * RPT;
-    // one wave per team: a wave past the end simply leaves (no barrier is ever used);
-    // several waves per team: every team stays for the barrier, rows past the end are empty
-    if (TPR <= kWave && row0 >= N) return;
-    const int nvec = H / VEC;
-
-    // mean = sum * (1/H) instead of a division (ten instructions per thread); a zero the compiler cannot see through
-    // keeps gamma * x a mixed-precision fma on the fp16 values themselves (v_fma_mix_f32: no widening instructions)
+    // the row a wave works on is the same for all its lanes: say so, the descriptors live in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int row_id = blockIdx.x * TPB + wave / NWAVE;
+    // a team past the last row keeps running with empty descriptors (every load gives zeros, every store is
+    // dropped), so that all waves of the workgroup reach the barrier
+    const unsigned row_bytes = row_id < N ? (unsigned)H * (unsigned)sizeof(T) : 0u;
+    const size_t row = (size_t)(row_id < N ? row_id : 0) * H;
+    const __amdgpu_buffer_rsrc_t d_out = row_descriptor(out + row, row_bytes);
+    const __amdgpu_buffer_rsrc_t d_gamma = row_descriptor(gamma, row_bytes);
     const float inv_h = 1.0f / (float)H;
-    const float zero = eps * 0.0f;
-    const float one = 1.0f + zero;
-    Vec16<T> x[RPT][NV];
-    float ss[RPT];
-    // gamma is requested with the row, not after the reduction: by then it has arrived, instead of
-    // costing every workgroup a second memory round trip between its barrier and its stores
-    Vec16<T> g[NV];
+    const float zero = eps * 0.0f;          // a zero and a one the compiler cannot see through keep the fp16
+    const float one = 1.0f + zero;          // operands inside mixed-precision fmas (no widening instructions)
+
+    // gamma is requested right behind the row, so that it has arrived when the reduction is done - except in the
+    // one form whose registers that would overflow (fused, fp16, eight vectors per thread: rows beyond 32 Ki elements)
+    constexpr bool kLateGamma = FUSED && NV >= 8 && sizeof(T) == 2;
+    Vec16<T> g[NV], x[NV];
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        const int idx = lane + j * TPR;
-        if (idx < nvec) g[j] = load16(gamma + idx * VEC);
+    for (int j = 0; j < NV; ++j) x[j] = buffer_load16<T, kAuxStreamLoad>(d_out, (unsigned)(lane + j * TPR) * 16u);
+    if constexpr (!kLateGamma) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) g[j] = buffer_load16<T, kAuxPlain>(d_gamma, (unsigned)(lane + j * TPR) * 16u);
     }
-#pragma unroll
-    for (int k = 0; k < RPT; ++k) {
-        ss[k] = 0.f;
-        const bool live = row0 + k < N;
-        const T* orow = out + (size_t)(live ? row0 + k : 0) * H;
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const int idx = lane + j * TPR;
-            if (live && idx < nvec) x[k][j] = load16_stream(orow + idx * VEC);
-        }
-    }
+    float ss = 0.f;
+    float r[FUSED ? NV : 1][VEC];
     if constexpr (FUSED) {
-        // r = (out + residual) + bias is kept in fp32 in place of the raw inputs
-        float r[RPT][NV][VEC];
-        {
-            Vec16<T> y[RPT][NV];
-#pragma unroll
-            for (int k = 0; k < RPT; ++k) {
-                const bool live = row0 + k < N;
-                const T* rrow = residual + (size_t)(live ? row0 + k : 0) * H;
-#pragma unroll
-                for (int j = 0; j < NV; ++j) {
-                    const int idx = lane + j * TPR;
-                    if (live && idx < nvec) y[k][j] = load16_stream(rrow + idx * VEC);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < NV; ++j) {
-                const int idx = lane + j * TPR;
-                Vec16<T> b;
-                if (bias && idx < nvec) b = load16(bias + idx * VEC);
-#pragma unroll
-                for (int k = 0; k < RPT; ++k) {
-                    if (row0 + k < N && idx < nvec) {
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) {
-                            // (out + residual) + bias, in this order; the multiplications by a one the compiler
-                            // cannot see through keep the additions mixed-precision fmas on the stored values
-                            float v = __builtin_fmaf(x[k][j].get(e), one, y[k][j].get(e));
-                            if (bias) v = __builtin_fmaf(b.get(e), one, v);
-                            r[k][j][e] = v;
-                            y[k][j].set(e, v);
-                            ss[k] = fmaf(v, v, ss[k]);
-                        }
-                        store16_stream(residual + (size_t)(row0 + k) * H + idx * VEC, y[k][j]);
-                    }
-                }
-            }
-        }
-        row_sums<TPR, RPT>(ss, smem, tid);
+        const __amdgpu_buffer_rsrc_t d_res = row_descriptor(residual + row, row_bytes);
+        const __amdgpu_buffer_rsrc_t d_bias = row_descriptor(bias, bias ? row_bytes : 0u);   // no bias: zeros
+        Vec16<T> y[NV], b[NV];
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
-            const int idx = lane + j * TPR;
-            if (idx < nvec) {
+            const unsigned off = (unsigned)(lane + j * TPR) * 16u;
+            y[j] = buffer_load16<T, kAuxStreamLoad>(d_res, off);
+            b[j] = buffer_load16<T, kAuxPlain>(d_bias, off);
+        }
 #pragma unroll
-                for (int k = 0; k < RPT; ++k) {
-                    if (row0 + k < N) {
-                        const float inv = rsqrtf(__builtin_fmaf(ss[k], inv_h, eps));
+        for (int j = 0; j < NV; ++j) {
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) x[k][j].set(e, g[j].get(e) * r[k][j][e] * inv);
-                        store16_stream(out + (size_t)(row0 + k) * H + idx * VEC, x[k][j]);
-                    }
-                }
+            for (int e = 0; e < VEC; ++e) {
+                // (out + residual) + bias in fp32, in this order
+                float v = __builtin_fmaf(x[j].get(e), one, y[j].get(e));
+                v = __builtin_fmaf(b[j].get(e), one, v);
+                r[j][e] = v;
+                y[j].set(e, v);
+                ss = fmaf(v, v, ss);
             }
+            buffer_store16<T, kAuxStreamStore>(d_res, (unsigned)(lane + j * TPR) * 16u, y[j]);
         }
     } else {
 #pragma unroll
-        for (int k = 0; k < RPT; ++k)
-#pragma unroll
-            for (int j = 0; j < NV; ++j) {
-                const int idx = lane + j * TPR;
-                if (row0 + k < N && idx < nvec) {
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        const float v = x[k][j].get(e);
-                        ss[k] = fmaf(v, v, ss[k]);
-                    }
-                }
-            }
-        row_sums<TPR, RPT>(ss, smem, tid);
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const int idx = lane + j * TPR;
-            if (idx < nvec) {
-#pragma unroll
-                for (int k = 0; k < RPT; ++k) {
-                    if (row0 + k < N) {
-                        const float inv = rsqrtf(__builtin_fmaf(ss[k], inv_h, eps));
-#pragma unroll
-                        for (int e = 0; e < VEC; ++e) x[k][j].set(e, __builtin_fmaf(g[j].get(e), x[k][j].get(e), zero) * inv);
-                        store16_stream(out + (size_t)(row0 + k) * H + idx * VEC, x[k][j]);
-                    }
-                }
-            }
-        }
+        for (int j = 0; j < NV; ++j) ss = sum_squares(x[j], ss);
     }
+    float total;
+    if constexpr (NWAVE == 1) {
+        total = wave_sum(ss);
+    } else {
+        ss = wave_sum_in_last_lane(ss);
+        if ((tid & (kWave - 1)) == kWave - 1) smem[wave] = ss;
+        __syncthreads();
+        total = 0.f;
+        const int first = wave / NWAVE * NWAVE;
+#pragma unroll
+        for (int w = 0; w < NWAVE; ++w) total += smem[first + w];
+    }
+    const float inv = rsqrtf(__builtin_fmaf(total, inv_h, eps));
+    if constexpr (kLateGamma) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) g[j] = buffer_load16<T, kAuxPlain>(d_gamma, (unsigned)(lane + j * TPR) * 16u);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float gs = __builtin_fmaf(g[j].get(e), inv, zero);
+            if constexpr (FUSED) x[j].set(e, r[j][e] * gs);
+            else x[j].set(e, __builtin_fmaf(x[j].get(e), gs, zero));
+        }
+        buffer_store16<T, kAuxStreamStore>(d_out, (unsigned)(lane + j * TPR) * 16u, x[j]);
+    }
+}
+
+template <typename T, int NV, int TPR, bool FUSED>
+int launch_row(T* out, T* residual, const T* bias, const T* gamma, float eps, int N, int H, hipStream_t st)
+{
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int TPB = BLOCK / TPR;
+    hipLaunchKernelGGL((norm_row_kernel<T, NV, TPR, FUSED>), dim3((N + TPB - 1) / TPB), dim3(BLOCK), 0, st,
+                       out, residual, bias, gamma, eps, N, H);
+    return launch_status();
 }
 
 // Any H, any alignment: scalar accesses, the row is read twice.  Not a performance path.
@@ -189,9 +200,10 @@ void norm_rows_generic_kernel(T* __restrict__ out, T* __restrict__ residual, con
         }
         ss = fmaf(v, v, ss);
     }
-    float sv[1] = {ss};
-    row_sums<256, 1>(sv, smem, tid);
-    const float inv = rsqrtf(sv[0] / (float)H + eps);
+    ss = wave_sum(ss);
+    if ((tid & (kWave - 1)) == 0) smem[tid / kWave] = ss;
+    __syncthreads();
+    const float inv = rsqrtf((smem[0] + smem[1] + smem[2] + smem[3]) / (float)H + eps);
     for (int i = tid; i < H; i += 256) {
         float v = to_f32(orow[i]);
         if constexpr (FUSED) {
@@ -203,61 +215,47 @@ void norm_rows_generic_kernel(T* __restrict__ out, T* __restrict__ residual, con
     }
 }
 
-template <typename T, int TPR, int RPT, bool FUSED>
-int launch_team(T* out, T* residual, const T* bias, const T* gamma, float eps, int N, int H, hipStream_t st)
-{
-    constexpr int VEC = Elt<T>::kVec;
-    constexpr int BLOCK = TPR > 256 ? TPR : 256;
-    constexpr int RPB = BLOCK / TPR * RPT;       // rows per block
-    const int nvec = H / VEC;
-    const int need = (nvec + TPR - 1) / TPR;
-    const dim3 grid((N + RPB - 1) / RPB), block(BLOCK);
-#define ONELLM_NORM_CASE(nv)                                                                                          \
-    hipLaunchKernelGGL((norm_rows_kernel<T, nv, TPR, RPT, FUSED>), grid, block, 0, st, out, residual, bias, gamma, eps, N, H)
-    if (need <= 1) ONELLM_NORM_CASE(1);
-    else if (need <= 2) ONELLM_NORM_CASE(2);
-    else if (need <= 4) ONELLM_NORM_CASE(4);
-    else if (need <= 8) ONELLM_NORM_CASE(8);
-    else if (need <= 16) ONELLM_NORM_CASE(16);
-    else return ONELLM_EUNSUPPORTED;
-#undef ONELLM_NORM_CASE
-    return launch_status();
-}
-
-template <typename T, int RPT, bool FUSED>
-int launch_tpr(int tpr, T* out, T* residual, const T* bias, const T* gamma, float eps, int N, int H, hipStream_t st)
-{
-    if (tpr == 64) return launch_team<T, 64, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
-    if (tpr == 128) return launch_team<T, 128, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
-    if (tpr == 256) return launch_team<T, 256, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
-    if (tpr == 512) return launch_team<T, 512, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
-    return launch_team<T, 1024, RPT, FUSED>(out, residual, bias, gamma, eps, N, H, st);
-}
-
+// Team size and vectors per thread: a wave or two for short rows; 256 threads up to 256 vectors, 512 threads up
+// to 2048 (one, two or four vectors each: measured best on MI355X at 8 KiB and 16 KiB rows - 256 threads x 2 and
+// 1024 x 1 are 0.5-45 % slower), 1024 threads with four or eight beyond.  `forced` (a tuning knob) picks the
+// team size where the row fits it.
 template <typename T, bool FUSED>
 int launch_norm(T* out, T* residual, const T* bias, const T* gamma, float eps, int N, int H, hipStream_t st)
 {
     constexpr int VEC = Elt<T>::kVec;
     if (N == 0) return 0;
+    const int nvec = H / VEC;
     const bool vec_ok = (H % VEC == 0) && aligned16(out) && aligned16(gamma) && (!FUSED || aligned16(residual))
-                        && (!bias || aligned16(bias)) && (H / VEC) <= 1024 * 16;
+                        && (!bias || aligned16(bias)) && nvec <= 1024 * 8;
     if (!vec_ok) {
         hipLaunchKernelGGL((norm_rows_generic_kernel<T, FUSED>), dim3(N), dim3(256), 0, st, out, residual, bias, gamma, eps, N, H);
         return launch_status();
     }
-    const int nvec = H / VEC;
-    // team size: one 16-byte vector per thread and row up to 512 threads, then more vectors per thread
-    // (8 KiB fp16 rows -> 512 threads x 1: 23.3 / 44.4 us plain / fused at 8192 rows against 23.5 / 45.6 with
-    // 256 x 2; 16 KiB rows -> 512 x 2: 44.7 / 90.8 against 47.2 / 90.4 with 1024 x 1)
-    int tpr = tune_get("norm_tpr");
-    if (tpr != 64 && tpr != 128 && tpr != 256 && tpr != 512 && tpr != 1024) {
-        tpr = 64;
-        while (tpr < 512 && nvec > tpr) tpr *= 2;
+    int tpr = nvec <= 64 ? 64 : nvec <= 128 ? 128 : nvec <= 256 ? 256 : nvec <= 2048 ? 512 : 1024;
+    const int forced = tune_get("norm_tpr");
+    if ((forced == 64 || forced == 128 || forced == 256 || forced == 512 || forced == 1024)
+        && nvec <= forced * (forced >= 1024 ? 8 : forced >= 256 ? 4 : 1))
+        tpr = forced;
+    const int nv = (nvec + tpr - 1) / tpr;
+#define ONELLM_NORM_CASE(NV, TPR) return launch_row<T, NV, TPR, FUSED>(out, residual, bias, gamma, eps, N, H, st)
+    switch (tpr) {
+        case 64: ONELLM_NORM_CASE(1, 64);
+        case 128: ONELLM_NORM_CASE(1, 128);
+        case 256:
+            if (nv <= 1) ONELLM_NORM_CASE(1, 256);
+            if (nv <= 2) ONELLM_NORM_CASE(2, 256);
+            ONELLM_NORM_CASE(4, 256);
+        case 512:
+            if (nv <= 1) ONELLM_NORM_CASE(1, 512);
+            if (nv <= 2) ONELLM_NORM_CASE(2, 512);
+            ONELLM_NORM_CASE(4, 512);
+        default:
+            if (nv <= 1) ONELLM_NORM_CASE(1, 1024);
+            if (nv <= 2) ONELLM_NORM_CASE(2, 1024);
+            if (nv <= 4) ONELLM_NORM_CASE(4, 1024);
+            ONELLM_NORM_CASE(8, 1024);
     }
-    while (tpr < 1024 && nvec > tpr * 16) tpr *= 2;
-    // several rows per team (2 or 4, all loads issued up front) were measured too and gave nothing
-    // over one row per team on MI355X: the plateau is the read/write mix at the memory, not latency
-    return launch_tpr<T, 1, FUSED>(tpr, out, residual, bias, gamma, eps, N, H, st);
+#undef ONELLM_NORM_CASE
 }
 
 }  // namespace

@@ -41,7 +41,8 @@ def test_fused_reference_unit_vector(capi, dev):
 
 
 SHAPES = [(16, 4096), (512, 4096), (8192, 4096), (8192, 8192),      # BASELINE config 4
-          (3, 32), (5, 100), (7, 4100), (2, 16384), (1, 40960), (2050, 1024), (4, 70000)]
+          (3, 32), (5, 100), (7, 4100), (2, 16384), (1, 40960), (2050, 1024), (4, 70000),
+          (9, 512), (300, 1000), (5, 1032), (3, 2056), (2, 32768), (3, 65536)]     # every team size and vector count
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
@@ -76,7 +77,7 @@ def test_fused_norm_matches_oracle(capi, ref, dev, dtype, with_bias, N, H):
     np.testing.assert_allclose(d_out.cpu().numpy().astype(np.float64), w_out.astype(np.float64), **TOL[dtype])
 
 
-@pytest.mark.parametrize("tpr", [64, 256, 1024])
+@pytest.mark.parametrize("tpr", [256, 512, 1024])
 def test_every_row_team_size_gives_the_same_answer(capi, ref, dev, tpr):
     announce("norm team size", tpr)
     x, res, bias, gamma = _inputs(33, 4096, np.float16, seed=9)
