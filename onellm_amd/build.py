@@ -27,6 +27,9 @@ LIB_LAYERS = os.path.join(HERE, "libonellm_layers.so")
 # test-only: a C wrapper that drives the launcher shims with oneLLM-style Tensor objects
 HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "launcher_harness.cpp")
 LIB_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
+# test-only: bare access-pattern kernels (what the memory system gives each kernel's access mix); timed by bench.py
+CEILINGS_SRC = os.path.join(ROOT, "tests", "cpp", "access_ceilings.hip")
+LIB_CEILINGS = os.path.join(ROOT, "tests", "cpp", "libaccess_ceilings.so")
 # test-only: a stand-alone C++ program that runs one decode step through the layers, like the reference's example driver
 DRIVER_SRC = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver.cpp")
 DRIVER_BIN = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver")
@@ -127,6 +130,11 @@ def build(force=False, verbose=False):
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("hipcc failed for the launcher harness:\n" + r.stderr[-4000:])
+    if os.path.exists(CEILINGS_SRC) and (force or _newer(LIB_CEILINGS, [CEILINGS_SRC])):
+        cmd = [HIPCC, "-shared", "-fPIC", "-O3", "-std=c++17", CEILINGS_SRC, "-o", LIB_CEILINGS] + DEVICE + PRELOAD_KERNARGS
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for the access-ceiling kernels:\n" + r.stderr[-4000:])
     if force or _newer(LIB_GEMM, gobjs + [LIB_HIP]):
         cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_GEMM] + gobjs + \
               ["-L" + HERE, "-lonellm_hip", "-L/opt/rocm/lib", "-lhipblaslt", "-Wl,-rpath,$ORIGIN"]

@@ -123,10 +123,12 @@ void norm_row_kernel(T* __restrict__ out, T* __restrict__ residual, const T* __r
         for (int j = 0; j < NV; ++j) {
             const unsigned off = (unsigned)(lane + j * TPR) * 16u;
             y[j] = buffer_load16<T, kAuxStreamLoad>(d_res, off);
-            b[j] = buffer_load16<T, kAuxPlain>(d_bias, off);
+            if constexpr (!kLateGamma) b[j] = buffer_load16<T, kAuxPlain>(d_bias, off);
         }
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
+            // (the register-bound form fetches its bias vector by vector, a cache hit each)
+            if constexpr (kLateGamma) b[j] = buffer_load16<T, kAuxPlain>(d_bias, (unsigned)(lane + j * TPR) * 16u);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 // (out + residual) + bias in fp32, in this order
