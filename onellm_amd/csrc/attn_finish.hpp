@@ -307,21 +307,40 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, fl
     }
     if (u.direct || !a.counters) return;
 
-    // ---- fused finish.  Every piece of the unit has written its state with device-scope stores
-    // (written through to memory, not left in this chip quarter's L2) and then, once all of its
-    // threads' stores have completed, adds one to the unit's counter.  The piece whose add finds
-    // all the others there reads their states back with device-scope loads and merges them.  No
-    // cache write-back or invalidation is involved: the only data that crosses between workgroups
-    // moves through these scoped accesses, and nobody waits on anybody.
+    // ---- fused finish.  Every piece of the unit has written its state with agent-scope stores and then, once all
+    // of its threads' stores have completed, adds one to the unit's counter.  The piece whose add finds all the
+    // others there reads their states back with agent-scope loads and merges them.  Nobody waits on anybody.
+    //
+    // What orders the hand-over.  By default nothing in the source language does: the stores, the add and the loads
+    // are relaxed, so the ordering between a piece's state and its counter add rests on what these instructions do
+    // on gfx950, which is this.  (1) An agent-scope store is `global_store ... sc1`: it is written through this chip
+    // quarter's L2 to memory, and the wave's vmcnt drops only when that write has been acknowledged; the explicit
+    // `s_waitcnt vmcnt(0)` + barrier below therefore mean every thread's state is in memory before thread 0 issues
+    // the add.  That wait is exactly the instruction sequence the compiler emits for an agent-scope release, minus
+    // `buffer_wbl2 sc1` - the write-back of lines that ordinary stores left dirty in L2, of which the state has
+    // none.  (2) The add is an L2-bypassing device atomic executed at memory, so the piece that reads
+    // `npieces - 1` issues its loads after all the other pieces' adds, hence after their acknowledged writes.
+    // (3) An agent-scope load is `global_load ... sc1`: it is served from memory, not from a line another chip
+    // quarter's write could have left stale in this quarter's L2 or this unit's L1 - which is all that the
+    // `buffer_inv sc1` of an acquire would add, for ordinary loads.  The formally ordered form (release on the add,
+    // an acquire fence in the merging piece: `a.ordered`, tuning key attn_ordered_finish) is kept and tested; its two
+    // cache-maintenance instructions cost 8 % on a one-sequence step and 34 % on a 32-sequence ragged step on
+    // MI355X (17.2 -> 18.5 us, 96 -> 129 us), which is why it is not the default.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                                            // all stores done; st_ml no longer read
     int* arrived = reinterpret_cast<int*>(st_ml);                  // the merged states are no longer needed: reuse a word
     const int tid = lane_id_per_unit();
-    if (tid == 0)
-        *arrived = __hip_atomic_fetch_add(a.counters + u.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) {
+        if (a.ordered) *arrived = __hip_atomic_fetch_add(a.counters + u.counter, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        else *arrived = __hip_atomic_fetch_add(a.counters + u.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     __syncthreads();
     if (*arrived != u.npieces - 1) return;
     if (tid == 0) __hip_atomic_store(a.counters + u.counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
+    if (a.ordered) {
+        if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        __syncthreads();
+    }
     // (pieces whose loads are in flight together: 16 at most, no more than the unit has - most have two or three -
     // rounded up to a power of two; the surplus slots of a batch repeat the last piece's loads)
     if (u.npieces <= 2) merge_pieces<T, D, GT, NTHR, 2>(a, u, tid);

@@ -39,6 +39,7 @@ struct AttnArgs {
     // fused finish (counters != NULL): one arrival counter per unit, zero between calls; the piece
     // that arrives last merges the unit's partial states itself and no merge kernel is launched
     int* counters;
+    int ordered;          // 1: the counter add is a release and the merging piece takes an acquire fence (agent scope)
 };
 
 // What one workgroup works on: a chunk of the history of one (sequence, kv-head) for up to GT query heads.

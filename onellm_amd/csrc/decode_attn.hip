@@ -562,6 +562,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.G = Hq / Hkv; a.S = S;
     a.rotary_dim = rotary_dim; a.pos_offset = rope_pos_offset; a.flags = flags;
     a.turns = tune_get("attn_turns") != 0;
+    a.ordered = tune_get("attn_ordered_finish") == 1;
     a.qscale = (1.0f / sqrtf((float)D)) * 1.4426950408889634f;
     a.slab = (size_t)layer * B * Hkv * (size_t)S * D;
 

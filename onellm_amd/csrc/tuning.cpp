@@ -22,6 +22,7 @@ Knob g_knobs[] = {
     {"attn_fused_finish", {-1}}, // 0: keep the separate merge launch even when the workspace is declared zeroed
     {"prefill_generic", {-1}},   // 1: the index-walking prefill kernel also where the row-walking one applies
     {"attn_gqa_valu", {-1}},     // 1: grouped-query heads on the vector ALU kernel instead of the MFMA one
+    {"attn_ordered_finish", {-1}}, // 1: release on the fused finish's counter add + acquire fence in the merging piece
     {"attn_turns", {-1}},        // 0: co-resident attention workgroups do not take turns at wave priority
 };
 }  // namespace

@@ -393,6 +393,59 @@ def test_fused_finish_at_full_size_matches_the_merge_launch(capi, dev):
         assert (outs[0][:nb].float() - outs[1][:nb].float()).abs().max().item() <= 1e-3
 
 
+def test_fused_finish_soak_on_one_workspace(capi, dev):
+    """200 calls of mixed shapes, schedules and lengths on ONE zero-filled workspace, each compared with the same call
+    finished by the merge launch (same pieces, merged in piece order either way) and stopped at the first mismatch.
+    The fused finish hands partial states between workgroups through agent-scope accesses and an arrival counter; a
+    piece that read a stale state, or a counter that was not back at zero, shows up here as a wrong output."""
+    torch.manual_seed(5)
+    B, Hq, Hkv, D, S = 32, 32, 8, 128, 4096
+    kc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+    vc = torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half()
+    qkv = torch.randn(B, Hq + 2 * Hkv, D, device=dev).mul_(0.5).half()
+    bias = torch.randn((Hq + 2 * Hkv) * D, device=dev).mul_(0.5).half()
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    ws_merge = torch.empty_like(ws)
+    small = {nb: (kc[:, :nb].contiguous(), vc[:, :nb].contiguous()) for nb in (1, 2, 4, 8, 16)}
+    small[32] = (kc, vc)
+    rng = np.random.default_rng(5)
+    o_merge = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+    o_fused = torch.zeros_like(o_merge)
+    try:
+        for rep in range(200):
+            mode = rep % 5
+            nb = int(rng.choice([1, 2, 4, 8, 16, 32]))
+            if mode == 0:
+                t, t_dev = int(rng.integers(1, S + 1)), None
+            else:
+                lens = rng.integers(1, S + 1, size=nb).astype(np.int32)
+                if mode == 2:
+                    lens[:] = np.minimum(lens, 300)
+                t, t_dev = int(lens.max()), torch.from_numpy(lens).to(dev)
+            if mode == 3:
+                capi.tune_set("attn_balanced", 1)
+                capi.tune_set("attn_balanced_wgs", int(rng.choice([7, 100, 512, 1024])))
+            if mode == 4:
+                capi.tune_set("attn_ordered_finish", 1)      # the formally ordered hand-over (release / acquire fence)
+            if rep % 20 == 0:
+                announce("attn fused soak, rep", rep)
+            k, v = small[nb]
+            capi.decode_attn(qkv[:nb], bias, k, v, o_merge[:nb], Hq, t, D, 10000.0, t_dev=t_dev, max_t=t, workspace=ws_merge,
+                             flags=capi.ATTN_NO_CACHE_WRITE)
+            capi.decode_attn(qkv[:nb], bias, k, v, o_fused[:nb], Hq, t, D, 10000.0, t_dev=t_dev, max_t=t, workspace=ws,
+                             flags=capi.ATTN_NO_CACHE_WRITE | capi.ATTN_ZEROED_WORKSPACE)
+            capi.tune_set("attn_balanced", -1)
+            capi.tune_set("attn_balanced_wgs", -1)
+            capi.tune_set("attn_ordered_finish", -1)
+            diff = (o_merge[:nb].float() - o_fused[:nb].float()).abs().max().item()
+            assert diff <= 1e-3, "call %d (mode %d, batch %d, t %d): fused finish differs from the merge launch by %g" % (rep, mode, nb, t, diff)
+        assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0, "arrival counters not back at zero"
+    finally:
+        capi.tune_set("attn_balanced", -1)
+        capi.tune_set("attn_balanced_wgs", -1)
+        capi.tune_set("attn_ordered_finish", -1)
+
+
 @pytest.mark.parametrize("B,Hq,Hkv,t", [(9, 32, 32, 600), (36, 32, 8, 600), (5, 64, 64, 1100), (20, 16, 8, 1300), (72, 32, 8, 330),
                                         (81, 16, 8, 290)])
 @pytest.mark.parametrize("zeroed", [False, True])
