@@ -30,6 +30,7 @@
 //     layer) needs; setRopePositionOffset(0) restores the kernel's own convention;
 //   * no device synchronisation after each launch (src/layers/decoder/self_decoder.cpp:22,50,67).
 #pragma once
+#include <cstddef>
 #include <vector>
 #include "onellm/allocator.h"
 #include "onellm/kernels.h"
@@ -51,6 +52,11 @@ void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool tr
 // that first call synchronises the null stream.  Switch it off to keep every call asynchronous (for example before
 // capturing a step into a graph; shapes tuned earlier stay tuned).
 void setLinearGemmAutotune(bool on);
+// A projection the GEMM library has no kernel for throws unless it is tiny (unit-test and example-driver sizes) or
+// the plain kernel - about a hundred times slower - has been allowed here.
+void setLinearGemmPlainFallback(bool allow);
+// Number of GEMM workspaces alive: one per (device, launch stream) that has run a projection.
+size_t linearGemmWorkspaceCount();
 
 class LLaMASelfAttentionLayer {
 public:

@@ -21,6 +21,20 @@ do {                                                                    \
     }                                                                   \
 } while (0)
 
+// src/utils/macro.h:59-70: status check of a BLAS-library call.  The layers here call the GEMM through
+// onellm_linear (which reports through its return code), so nothing in this backend uses it; it is kept so that layer
+// sources written against the reference (`CHECK_CUBLAS(cublasXxx(...))`) compile unchanged when the call they wrap
+// returns a hipblasStatus_t / hipError_t-like integer: non-zero throws, as in the reference.
+template<typename T>
+void check(T result, char const* const func, const char* const file, int const line)
+{
+    if (result) {
+        throw std::runtime_error(std::string("[TM][ERROR] HIP runtime error: status ") + std::to_string((long long)result)
+                                 + " from " + func + " " + file + ":" + std::to_string(line) + " \n");
+    }
+}
+#define CHECK_CUBLAS(val) check((val), #val, __FILE__, __LINE__)
+
 // src/utils/macro.h:74-84
 inline void syncAndCheck(const char* const file, int const line)
 {

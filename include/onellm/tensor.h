@@ -102,4 +102,20 @@ struct Tensor {
         s += ")]";
         return s;
     }
+
+    friend bool operator==(Tensor& t1, Tensor& t2);
 };
+
+// src/utils/tensor.h:86,146-160: element-wise comparison of two host-readable FP32 tensors of equal size (the
+// reference dereferences `data` as float on the host whatever the element type or location are; so does this).
+// Sizes that differ, or an empty tensor on either side with a non-empty one on the other, compare unequal.
+inline bool operator==(Tensor& t1, Tensor& t2)
+{
+    if (t1.size() != t2.size()) return false;
+    const float* a = static_cast<const float*>(t1.data);
+    const float* b = static_cast<const float*>(t2.data);
+    for (int i = 0; i < t1.size(); ++i) {
+        if (a[i] != b[i]) return false;
+    }
+    return true;
+}

@@ -3,8 +3,9 @@
  * Replaces launchLinearGemm (src/kernels/qkv_linear.cu:8-66, declared src/kernels/qkv_linear.h:9-14) and the
  * cublasWrapper::Gemm call under it (src/kernels/cublas_wrapper.cc:33-85).  The multiplication itself is a library
  * GEMM (hipBLASLt, fp32 accumulation); this entry point adds what the reference re-creates on every call: a handle
- * per device and a cached plan per (dtype, M, K, N, layout).  Shapes the library has no kernel for fall back to a
- * plain kernel in this library, so every shape returns a result.
+ * per device and a cached plan per (dtype, M, K, N, layout).  Small shapes the library has no kernel for (unit-test
+ * and example-driver sizes, up to 2^24 multiply-adds) run a plain kernel in this library; a larger one returns
+ * ONELLM_ENOGEMMKERNEL unless the caller has allowed the plain kernel, which is about a hundred times slower.
  *
  * Kept out of libonellm_hip.so so that the decode-path kernels do not pull in the BLAS library.
  */
@@ -41,6 +42,11 @@ size_t onellm_linear_workspace_bytes(void);
 
 /* 1 if the last onellm_linear call on this thread ran the library GEMM, 0 if it ran the plain fallback kernel */
 int onellm_linear_last_path(void);
+
+/* allow != 0: problems of any size may run the plain kernel when the library declines them (process-wide; off by
+ * default, so that a projection of a real model never becomes a hundred times slower without an error).  Returns
+ * the previous setting. */
+int onellm_linear_allow_plain(int allow);
 
 #ifdef __cplusplus
 }

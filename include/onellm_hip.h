@@ -33,6 +33,9 @@ extern "C" {
 #define ONELLM_EUNSUPPORTED (-2) /* shape outside what the kernels are built for */
 #define ONELLM_EWORKSPACE  (-3)  /* workspace missing or too small              */
 #define ONELLM_ESCRATCH    (-4)  /* onellm_decode_attn_static: the step needs more than the built-in scratch */
+#define ONELLM_ENOGEMMKERNEL (-5) /* onellm_linear (onellm_gemm.h): the GEMM library has no kernel for this problem and
+                                     the plain kernel was not allowed                                          */
+#define ONELLM_ECAPTURING  (-6)  /* the call would have to allocate or synchronise, and its stream is being captured */
 
 /* flags for onellm_decode_attn */
 #define ONELLM_ATTN_NO_V_BIAS     0x1u /* skip the v-bias add (reference decode kernel behaviour,

@@ -19,6 +19,12 @@ const char* onellm_layers_last_error(void);
  * pair: y is the {2, M, N} gate/up buffer of the FFN (rows interleaved as [M, 2, N]); second: write its second slot. */
 int onellm_layers_linear(int dtype, void* x, void* w, void* y, int M, int K, int N, int trans_b, int pair, int second);
 
+/* setLinearGemmPlainFallback / linearGemmWorkspaceCount of onellm/layers.h: whether a projection the GEMM library
+ * declines may run the plain kernel whatever its size (off by default: a large one throws); how many GEMM workspaces
+ * exist (one per device and launch stream that has run a projection). */
+int onellm_layers_allow_plain_gemm(int allow);
+int onellm_layers_gemm_workspace_count(void);
+
 /* A LlamaSelfDecoder (src/layers/decoder/self_decoder.h:10-74) with its layer weights and an allocator.
  * The ten `void**` are host arrays of L device pointers, in the order of LlamaLayerWeight::loadWeights
  * (src/weights/llama/layer_weights.h:32-41); with attn_bias == 0 the qkv / output biases are ignored; bdown[l] may be

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(_HERE, "libonellm_hip.so")
 LAUNCHERS_PATH = os.path.join(_HERE, "libonellm_launchers.so")
 
 FP32, FP16 = 0, 1
-EINVAL, EUNSUPPORTED, EWORKSPACE, ESCRATCH = -1, -2, -3, -4
+EINVAL, EUNSUPPORTED, EWORKSPACE, ESCRATCH, ENOGEMMKERNEL, ECAPTURING = -1, -2, -3, -4, -5, -6
 DECODE_ATTN_STATIC_SCRATCH_BYTES = 16 << 20
 ATTN_NO_V_BIAS = 0x1
 ATTN_NO_CACHE_WRITE = 0x2
@@ -228,6 +228,7 @@ GEMM_SYMBOLS = {
     "onellm_linear_tune": (_ci, [_ci, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp, ctypes.POINTER(_cf), ctypes.POINTER(_cf)]),
     "onellm_linear_workspace_bytes": (_sz, []),
     "onellm_linear_last_path": (_ci, []),
+    "onellm_linear_allow_plain": (_ci, [_ci]),
 }
 _gemm = None
 

@@ -53,6 +53,14 @@ struct Workspace {
         std::lock_guard<std::mutex> g(mu);
         Buffer& b = buffers[std::make_pair(device, stream)];
         if (need > b.bytes) {
+            // creating (or growing) the buffer synchronises, allocates and clears: none of that may be recorded
+            // into a graph, so a stream that is being captured is refused - run one ordinary step first
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+            if (capturing != hipStreamCaptureStatusNone)
+                throw std::runtime_error("[oneLLM][ERROR] launchDecoderMaskedMHA: this step needs the attention workspace to be "
+                                         "created or grown, which cannot be done while the launch stream is being captured; "
+                                         "run one ordinary step on this stream first \n");
             // the old buffer may still be in use by work queued earlier on its stream
             if (b.ptr) {
                 throw_on_error((int)hipStreamSynchronize(stream), "workspace sync");

@@ -4,6 +4,7 @@
 #include <mutex>
 #include <set>
 #include <tuple>
+#include <utility>
 #include <stdexcept>
 #include <string>
 #include <hip/hip_runtime_api.h>
@@ -33,27 +34,47 @@ int cols_of(const Tensor* t)
     return n;
 }
 
-// scratch for the GEMM library's split-K algorithms: one per device, created on first use there
+bool stream_is_capturing(hipStream_t stream)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
+// Scratch for the GEMM library's split-K algorithms: one buffer per (device, launch stream), created on first use
+// there - steps queued on different streams of one GPU (two decoders, two threads) must not share split-K
+// partials.  Creating one allocates, so a stream that is being captured is refused.
 struct GemmWorkspace {
     struct Buffer {
         void* ptr = nullptr;
         size_t bytes = 0;
     };
     std::mutex mu;
-    std::map<int, Buffer> buffers;
-    Buffer get()
+    std::map<std::pair<int, hipStream_t>, Buffer> buffers;
+    Buffer get(hipStream_t stream)
     {
         int device = 0;
         hip_ok(hipGetDevice(&device), "gemm workspace device");
         std::lock_guard<std::mutex> g(mu);
-        auto it = buffers.find(device);
+        const auto key = std::make_pair(device, stream);
+        auto it = buffers.find(key);
         if (it != buffers.end()) return it->second;
+        require(!stream_is_capturing(stream), "launchLinearGemm: the first call on a stream creates its GEMM workspace, which "
+                                              "cannot be done while the stream is being captured; run one ordinary step first");
         Buffer b;
         const size_t want = onellm_linear_workspace_bytes();
         if (hipMalloc(&b.ptr, want) == hipSuccess) b.bytes = want;
         else { b.ptr = nullptr; (void)hipGetLastError(); }      // the library then keeps to algorithms that need none
-        buffers[device] = b;
+        buffers[key] = b;
         return b;
+    }
+    size_t count()
+    {
+        std::lock_guard<std::mutex> g(mu);
+        return buffers.size();
     }
 };
 GemmWorkspace g_gemm_ws;
@@ -69,7 +90,11 @@ void tune_once(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* ws, s
 {
     {
         std::lock_guard<std::mutex> g(g_tuned_mu);
-        if (!g_autotune || !g_tuned.insert(std::make_tuple(dtype, M, K, N, ldy, w_is_nk)).second) return;
+        if (!g_autotune || g_tuned.count(std::make_tuple(dtype, M, K, N, ldy, w_is_nk))) return;
+        // a shape first seen under capture is not timed now (that would allocate and synchronise) and stays
+        // unmarked, so that the next ordinary call tunes it; the captured call uses the library's first suggestion
+        if (stream_is_capturing(onellmGetLaunchStream())) return;
+        g_tuned.insert(std::make_tuple(dtype, M, K, N, ldy, w_is_nk));
     }
     (void)onellm_linear_tune(dtype, M, K, N, ldy, w_is_nk, ws, ws_bytes, onellmGetLaunchStream(), nullptr, nullptr);   // best effort
 }
@@ -98,6 +123,10 @@ void setLinearGemmAutotune(bool on)
     g_autotune = on;
 }
 
+void setLinearGemmPlainFallback(bool allow) { (void)onellm_linear_allow_plain(allow ? 1 : 0); }
+
+size_t linearGemmWorkspaceCount() { return g_gemm_ws.count(); }
+
 // src/kernels/qkv_linear.cu:8-66
 void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool trans_a, bool trans_b, bool shared_out_buf)
 {
@@ -124,7 +153,7 @@ void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool tr
         require(!shared_out_buf, "launchLinearGemm: shared_out_buf needs a {2, M, N} output");
         require(rows_of(output) == M && cols_of(output) == N, "launchLinearGemm: output shape");
     }
-    const GemmWorkspace::Buffer ws = g_gemm_ws.get();
+    const GemmWorkspace::Buffer ws = g_gemm_ws.get(onellmGetLaunchStream());
     const int dtype_code = input->dtype == FP32 ? ONELLM_FP32 : ONELLM_FP16;
     tune_once(dtype_code, M, K, N, ldy, trans_b ? 1 : 0, ws.ptr, ws.bytes);
     const int rc = onellm_linear(dtype_code, input->data, weight.data, y, M, K, N, ldy, trans_b ? 1 : 0, ws.ptr, ws.bytes,

@@ -56,6 +56,14 @@ int onellm_layers_linear(int dtype, void* x, void* w, void* y, int M, int K, int
     });
 }
 
+int onellm_layers_allow_plain_gemm(int allow)
+{
+    setLinearGemmPlainFallback(allow != 0);
+    return 0;
+}
+
+int onellm_layers_gemm_workspace_count(void) { return (int)linearGemmWorkspaceCount(); }
+
 // per-layer pointer arrays of length L, in the argument order of LlamaLayerWeight::loadWeights
 void* onellm_decoder_create(int dtype, int B, int Hq, int Hkv, int D, int I, int L, int S, int rotary_dim, float rope_base,
                         float eps, int attn_bias, void** attn_norm, void** ffn_norm, void** wqkv, void** bqkv, void** wo,

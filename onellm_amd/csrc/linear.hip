@@ -1,5 +1,6 @@
 // y = x . W for the projections around the decode path: hipBLASLt with a per-device handle and cached
 // plans, plus a plain kernel for shapes the library declines.
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -9,9 +10,16 @@
 #include "onellm_gemm.h"
 
 namespace onellm {
+int tune_get(const char* key);     // libonellm_hip.so's tuning table
 namespace {
 
 constexpr size_t kWorkspaceBytes = 32u << 20;
+// The plain kernel runs one thread per output element: fine for the tiny matrices of unit tests and example
+// drivers, about a hundred times slower than the library on a projection of a real model.  Up to this many
+// multiply-adds it is used without asking; a larger problem the library declines is an error unless the caller
+// has allowed the plain kernel (onellm_linear_allow_plain).
+constexpr unsigned long long kPlainQuietMacs = 1ull << 24;
+std::atomic<int> g_allow_plain{0};
 
 template <typename T> __device__ __forceinline__ float ld(const T* p, size_t i);
 template <> __device__ __forceinline__ float ld<float>(const float* p, size_t i) { return p[i]; }
@@ -46,6 +54,16 @@ struct Plan {
     hipblasLtMatmulHeuristicResult_t heur{};
 };
 
+// gives the library's objects of a plan back (a plan that is replaced, or one whose set-up failed half way)
+void destroy_plan(Plan& p)
+{
+    if (p.desc) (void)hipblasLtMatmulDescDestroy(p.desc);
+    if (p.la) (void)hipblasLtMatrixLayoutDestroy(p.la);
+    if (p.lb) (void)hipblasLtMatrixLayoutDestroy(p.lb);
+    if (p.lc) (void)hipblasLtMatrixLayoutDestroy(p.lc);
+    p = Plan{};
+}
+
 struct DeviceState {
     hipblasLtHandle_t handle = nullptr;
     bool handle_failed = false;
@@ -73,7 +91,8 @@ Plan make_problem(int dtype, int M, int K, int N, int ldy, int w_is_nk)
     else ok &= hipblasLtMatrixLayoutCreate(&p.la, dt, N, K, N) == HIPBLAS_STATUS_SUCCESS;
     ok &= hipblasLtMatrixLayoutCreate(&p.lb, dt, K, M, K) == HIPBLAS_STATUS_SUCCESS;
     ok &= hipblasLtMatrixLayoutCreate(&p.lc, dt, N, M, ldy) == HIPBLAS_STATUS_SUCCESS;
-    p.usable = ok;
+    if (!ok) destroy_plan(p);
+    else p.usable = true;
     return p;
 }
 
@@ -99,7 +118,7 @@ Plan make_plan(hipblasLtHandle_t h, int dtype, int M, int K, int N, int ldy, int
 {
     Plan p = make_problem(dtype, M, K, N, ldy, w_is_nk);
     if (!p.usable) return p;
-    p.usable = candidates(h, p, ws_bytes, &p.heur, 1) == 1;
+    if (candidates(h, p, ws_bytes, &p.heur, 1) != 1) destroy_plan(p);       // (an unusable plan holds nothing)
     return p;
 }
 
@@ -159,7 +178,17 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
     constexpr int kWant = 32;
     hipblasLtMatmulHeuristicResult_t cand[kWant];
     const int n = candidates(handle, p, workspace_bytes, cand, kWant);
-    if (n == 0) return ONELLM_EUNSUPPORTED;
+    if (n == 0) {
+        destroy_plan(p);
+        return ONELLM_EUNSUPPORTED;
+    }
+    // the timing runs allocate, synchronise and launch: none of that may happen on a stream that is being captured
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) (void)hipGetLastError();
+    if (capturing != hipStreamCaptureStatusNone) {
+        destroy_plan(p);
+        return ONELLM_ECAPTURING;
+    }
 
     // stand-in operands of the right size (values do not matter for the timing; 0x3c3c.. is ~1.06 in fp16 and a
     // small normal number in fp32)
@@ -178,6 +207,7 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
         (e = hipMalloc(&y, (size_t)M * ldy * esz)) != hipSuccess || (e = hipEventCreate(&t0)) != hipSuccess ||
         (e = hipEventCreate(&t1)) != hipSuccess) {
         cleanup();
+        destroy_plan(p);
         return (int)e;
     }
     (void)hipMemsetAsync(x, 0x3c, (size_t)M * K * esz, st);
@@ -209,12 +239,18 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
         }
     }
     cleanup();
-    if (rc != 0) return rc;
-    if (best < 0) return ONELLM_EUNSUPPORTED;
+    if (rc != 0 || best < 0) {
+        destroy_plan(p);
+        return rc != 0 ? rc : ONELLM_EUNSUPPORTED;
+    }
     p.heur = cand[best];
     {
+        // (a plan in the table is only ever used under this lock or as a copy taken under it by a call that was
+        // queued before this one returns: the stream was synchronised above, so the old objects are idle)
         std::lock_guard<std::mutex> g(g_mu);
-        g_devices[dev].plans[std::make_tuple(dtype, M, K, N, ldy, w_is_nk, workspace_bytes ? 1 : 0)] = p;
+        Plan& slot = g_devices[dev].plans[std::make_tuple(dtype, M, K, N, ldy, w_is_nk, workspace_bytes ? 1 : 0)];
+        destroy_plan(slot);
+        slot = p;
     }
     if (best_us) *best_us = best_ms * 1e3f;
     if (first_us) *first_us = first_ms * 1e3f;
@@ -224,6 +260,8 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
 extern "C" size_t onellm_linear_workspace_bytes(void) { return onellm::kWorkspaceBytes; }
 
 extern "C" int onellm_linear_last_path(void) { return onellm::t_last_path; }
+
+extern "C" int onellm_linear_allow_plain(int allow) { return onellm::g_allow_plain.exchange(allow ? 1 : 0); }
 
 extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, int M, int K, int N, int ldy, int w_is_nk,
                              void* workspace, size_t workspace_bytes, onellm_stream_t stream)
@@ -260,6 +298,7 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
             if (plan.usable && plan.heur.workspaceSize > workspace_bytes) plan.usable = false;
         }
     }
+    if (tune_get("gemm_no_library") == 1) plan.usable = false;
     if (plan.usable) {
         const float alpha = 1.f, beta = 0.f;
         const hipblasStatus_t s = hipblasLtMatmul(handle, plan.desc, &alpha, w, plan.la, x, plan.lb, &beta, y, plan.lc, y,
@@ -269,6 +308,10 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
             return 0;
         }
     }
+    // no library kernel (or the library refused at run time): the plain kernel, unless that would be a silent
+    // hundredfold slowdown
+    if ((unsigned long long)M * (unsigned long long)K * (unsigned long long)N > kPlainQuietMacs && !g_allow_plain.load())
+        return ONELLM_ENOGEMMKERNEL;
     t_last_path = 0;
     return dtype == ONELLM_FP16 ? run_plain<__half>(x, w, y, M, K, N, ldy, w_is_nk, st)
                                 : run_plain<float>(x, w, y, M, K, N, ldy, w_is_nk, st);

@@ -22,6 +22,7 @@ Knob g_knobs[] = {
     {"attn_fused_finish", {-1}}, // 0: keep the separate merge launch even when the workspace is declared zeroed
     {"prefill_generic", {-1}},   // 1: the index-walking prefill kernel also where the row-walking one applies
     {"attn_gqa_valu", {-1}},     // 1: grouped-query heads on the vector ALU kernel instead of the MFMA one
+    {"gemm_no_library", {-1}},   // 1: onellm_linear behaves as if the GEMM library had declined the problem (tests)
     {"attn_ordered_finish", {-1}}, // 1: release on the fused finish's counter add + acquire fence in the merging piece
     {"attn_turns", {-1}},        // 0: co-resident attention workgroups do not take turns at wave priority
 };
@@ -60,6 +61,10 @@ extern "C" const char* onellm_error_string(int code)
         case ONELLM_EWORKSPACE: return "onellm: workspace missing or too small";
         case ONELLM_ESCRATCH: return "onellm: the step's split partials exceed the library's built-in scratch "
                                      "(ONELLM_DECODE_ATTN_STATIC_SCRATCH_BYTES); use onellm_decode_attn with a workspace";
+        case ONELLM_ENOGEMMKERNEL: return "onellm: the GEMM library has no kernel for this problem; onellm_linear_allow_plain(1) permits the "
+                        "plain kernel (about a hundred times slower)";
+        case ONELLM_ECAPTURING: return "onellm: the call has to allocate or synchronise and its stream is being captured; run one "
+                        "ordinary step on this stream first";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));

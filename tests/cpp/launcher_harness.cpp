@@ -182,6 +182,22 @@ int h_type_tags()
            + 32 * (getBitNum(WeightType::INT8_W) == 8);
 }
 
+// Tensor == Tensor (src/utils/tensor.h:146-160) and CHECK_CUBLAS (src/utils/macro.h:59-70): a bit per check that holds
+int h_equality_and_status_checks()
+{
+    float a[4] = {1.f, 2.f, 3.f, 4.f}, b[4] = {1.f, 2.f, 3.f, 4.f}, c[4] = {1.f, 2.f, 3.f, 5.f}, d[2] = {1.f, 2.f};
+    Tensor ta(CPU, FP32, {2, 2}, a), tb(CPU, FP32, {4}, b), tc(CPU, FP32, {2, 2}, c), td(CPU, FP32, {2}, d), empty(CPU, FP32, {2, 2});
+    int ok = 0;
+    ok |= (ta == tb) << 0;                        // same count, same values (shapes are not compared, as in the reference)
+    ok |= (!(ta == tc)) << 1;
+    ok |= (!(ta == td)) << 2;
+    ok |= (!(ta == empty)) << 3;
+    const int fine = guarded([] { CHECK_CUBLAS(0); });
+    const int threw = guarded([] { CHECK_CUBLAS(3); });
+    ok |= (fine == 0 && threw == 1 && g_last_error.find("[TM][ERROR]") != std::string::npos) << 4;
+    return ok;
+}
+
 // TensorMap as the layers use it (src/utils/tensor.h:160-296): returns a bit per check that holds
 int h_tensor_map_checks()
 {

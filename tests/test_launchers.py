@@ -43,6 +43,7 @@ def test_carrier_types(H):
     assert H.h_tensor_size(2, 3, 4) == 24
     assert H.h_getval_requires_cpu_tensor() == 1          # getVal on a GPU tensor throws
     assert b"[oneLLM][ERROR]" in H.h_last_error()
+    assert H.h_equality_and_status_checks() == 31         # Tensor == Tensor and CHECK_CUBLAS as the reference's
 
 
 def test_tensor_map_and_layer_weight_views(H):
@@ -331,5 +332,37 @@ def test_every_launcher_queues_on_the_launch_stream(H, dev):
             torch.cuda.synchronize()
             for i, (a, b) in enumerate(zip(state, want)):
                 assert torch.equal(a, b), f"replay {replay}: buffer {i} differs from the eager result"
+    finally:
+        H.h_set_launch_stream(None)
+
+
+@pytest.mark.gpu
+def test_first_split_step_on_a_capturing_stream_is_refused(H, dev):
+    """The attention launcher owns a workspace per launch stream and creates it (allocation, clear) when a step first
+    needs one.  That must not happen while the stream is being captured: the launcher throws, nothing is recorded or
+    launched, and the same step runs normally once the capture is over."""
+    import torch
+    announce("launchDecoderMaskedMHA first split step under capture")
+    torch.manual_seed(8)
+    B, Hq, Hkv, D, S, t = 1, 8, 2, 128, 2048, 2000            # one sequence, two kv heads: split into pieces
+    h = lambda *s: torch.randn(*s, device=dev).mul(0.5).half()
+    qkv, bias, kc, vc = h(B, Hq + 2 * Hkv, D), h((Hq + 2 * Hkv) * D), h(1, B, Hkv, S, D), h(1, B, Hkv, S, D)
+    out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+    p = lambda a: a.data_ptr()
+    call = lambda: H.h_decode_mha(1, p(qkv), p(bias), p(kc), p(vc), p(out), B, Hq, Hkv, D, S, 1, t, 0, D, 10000.0)
+    side = torch.cuda.Stream()                                 # a stream no launcher has seen
+    H.h_set_launch_stream(side.cuda_stream)
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            qkv.add_(0)                                        # (something for the graph to hold)
+            rc = call()
+            msg = H.h_last_error()
+        assert rc == 1 and b"captured" in msg, msg
+        torch.cuda.synchronize()
+        assert not out.any()
+        assert call() == 0, H.h_last_error()                   # outside a capture the workspace is created
+        torch.cuda.synchronize()
+        assert out.any()
     finally:
         H.h_set_launch_stream(None)

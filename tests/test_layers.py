@@ -51,7 +51,8 @@ def test_gemm_library_exports_what_its_header_declares(G):
     text = open(os.path.join(ROOT, "include", "onellm_gemm.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = sorted(set(re.findall(r"\b(onellm_[a-z0-9_]+)\s*\(", text)))
-    assert names == ["onellm_linear", "onellm_linear_last_path", "onellm_linear_tune", "onellm_linear_workspace_bytes"]
+    assert names == ["onellm_linear", "onellm_linear_allow_plain", "onellm_linear_last_path", "onellm_linear_tune",
+                     "onellm_linear_workspace_bytes"]
     for n in names:
         assert hasattr(G, n)
     assert G.onellm_linear_workspace_bytes() > 0
@@ -70,8 +71,8 @@ def test_layers_library_exports_its_c_surface(H):
     text = open(os.path.join(ROOT, "include", "onellm_layers.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = sorted(set(re.findall(r"\b(onellm_[a-z0-9_]+)\s*\(", text)))
-    assert names == ["onellm_decoder_create", "onellm_decoder_destroy", "onellm_decoder_forward", "onellm_layers_last_error",
-                     "onellm_layers_linear"]
+    assert names == ["onellm_decoder_create", "onellm_decoder_destroy", "onellm_decoder_forward", "onellm_layers_allow_plain_gemm",
+                     "onellm_layers_gemm_workspace_count", "onellm_layers_last_error", "onellm_layers_linear"]
     for n in names:
         assert hasattr(H, n)
 
@@ -341,3 +342,100 @@ def test_decoder_step_captured_into_a_graph_replays_identically(H, ref):
     finally:
         torch.cuda.synchronize()
         dec.close()
+
+
+# ---------------------------------------------------------------- slow or unsafe paths are loud
+
+def _harness():
+    L = ctypes.CDLL(os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so"))
+    L.h_set_launch_stream.argtypes = [ctypes.c_void_p]
+    L.h_set_launch_stream.restype = None
+    return L
+
+
+def test_new_error_codes_have_text():
+    from onellm_amd import capi
+    L = capi.lib()
+    assert b"plain kernel" in L.onellm_error_string(capi.ENOGEMMKERNEL)
+    assert b"captured" in L.onellm_error_string(capi.ECAPTURING)
+
+
+@pytest.mark.gpu
+def test_a_large_projection_without_a_library_kernel_is_an_error_not_a_slow_success(H, G, ref):
+    """With the GEMM library out of the picture (a test knob makes onellm_linear behave as if it had declined the
+    problem) a tiny product still runs - on the plain kernel, as unit-test and example sizes always did - while a
+    projection of a real model's size is refused with its own code, through the C entry point and as an exception of
+    launchLinearGemm, until the caller allows the hundred-times-slower kernel."""
+    import torch
+    from onellm_amd import capi
+    announce("linear without a library kernel")
+    rng = np.random.default_rng(1)
+    capi.tune_set("gemm_no_library", 1)
+    try:
+        for (M, K, N), big in (((3, 40, 24), False), ((16, 2048, 1024), True)):
+            x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
+            w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+            dx, dw = _dev(torch, x), _dev(torch, w)
+            y = torch.zeros((M, N), dtype=dx.dtype, device=dx.device)
+            rc = G.onellm_linear(1, dx.data_ptr(), dw.data_ptr(), y.data_ptr(), M, K, N, 0, 0, None, 0, None)
+            if not big:
+                assert rc == 0 and G.onellm_linear_last_path() == 0
+            else:
+                assert rc == capi.ENOGEMMKERNEL
+                assert H.onellm_layers_linear(1, dx.data_ptr(), dw.data_ptr(), y.data_ptr(), M, K, N, 0, 0, 0) == 1
+                assert b"plain kernel" in H.onellm_layers_last_error()
+                torch.cuda.synchronize()
+                assert not y.any()                                   # nothing ran
+                assert H.onellm_layers_allow_plain_gemm(1) == 0
+                try:
+                    assert H.onellm_layers_linear(1, dx.data_ptr(), dw.data_ptr(), y.data_ptr(), M, K, N, 0, 0, 0) == 0, H.onellm_layers_last_error()
+                    assert G.onellm_linear_last_path() == 0
+                finally:
+                    H.onellm_layers_allow_plain_gemm(0)
+            np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), ref.linear(x, w).astype(np.float64), **TOL[np.float16])
+    finally:
+        capi.tune_set("gemm_no_library", -1)
+
+
+@pytest.mark.gpu
+def test_gemm_workspace_is_per_launch_stream_and_never_created_under_capture(H):
+    """Two decoders or threads that queue on different streams of one GPU must not share the library's split-K
+    scratch: every launch stream gets its own buffer.  Creating one allocates, so the first projection on a stream
+    that is being captured is refused with a message instead of recording an allocation into the graph."""
+    import torch
+    announce("gemm workspace keying")
+    harness = _harness()
+    dev = torch.device("cuda:0")
+    x = torch.randn(4, 64, device=dev).half()
+    w = torch.randn(64, 32, device=dev).half()
+    y = torch.zeros(4, 32, dtype=torch.float16, device=dev)
+    run = lambda: H.onellm_layers_linear(1, x.data_ptr(), w.data_ptr(), y.data_ptr(), 4, 64, 32, 0, 0, 0)
+    s1, s2, s3 = torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.Stream()
+    try:
+        assert run() == 0                                            # null stream
+        torch.cuda.synchronize()
+        want = y.clone()
+        before = H.onellm_layers_gemm_workspace_count()
+        for k, s in enumerate((s1, s2, s1, s2)):
+            harness.h_set_launch_stream(s.cuda_stream)
+            y.zero_()
+            torch.cuda.synchronize()
+            assert run() == 0, H.onellm_layers_last_error()
+            torch.cuda.synchronize()
+            assert torch.equal(y, want)
+            assert H.onellm_layers_gemm_workspace_count() == before + min(k + 1, 2)
+        # a stream seen for the first time while it is being captured
+        harness.h_set_launch_stream(s3.cuda_stream)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s3):
+            x.add_(0)                                                # (something for the graph to hold)
+            rc = run()
+            msg = H.onellm_layers_last_error()
+        assert rc == 1 and b"captured" in msg, msg
+        assert H.onellm_layers_gemm_workspace_count() == before + 2
+        torch.cuda.synchronize()
+        assert run() == 0                                            # an ordinary call afterwards is fine
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)
+    finally:
+        harness.h_set_launch_stream(None)
