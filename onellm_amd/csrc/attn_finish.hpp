@@ -263,16 +263,77 @@ __device__ __forceinline__ void merge_pieces_wide(const AttnArgs& a, const Unit&
         }
 }
 
+// Fused finish, first look: how many of the unit's other pieces have arrived.  Asked a streaming iteration or two
+// before the piece ends and looked at in finish_unit, so the answer's round trip costs nothing.  Thread 0 only
+// (-1 elsewhere, and for units that are not shared or have more pieces than the register-held merge takes).
+__device__ __forceinline__ int first_look(const AttnArgs& a, const Unit& u)
+{
+    if (u.direct || !a.counters || !a.early_look || u.npieces > 8 || lane_id_per_unit() != 0) return -1;
+    return __hip_atomic_load(a.counters + u.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The merge of a unit's pieces by a piece that still holds its own state in registers: piece `mine` is taken from
+// (Ms, Ls, Os), the others are read with device-scope loads, and the arithmetic is that of merge_pieces with all
+// pieces read from memory - same batches, same order - so the unit's output does not depend on which piece merged it.
+template <typename T, int D, int GT, int NTHR, int BATCH, int E>
+__device__ __forceinline__ void merge_pieces_local(const AttnArgs& a, const Unit& u, int tid, int mine,
+                                                   const float (&Ms)[E], const float (&Ls)[E], const float (&Os)[E])
+{
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+        const int i = tid + k * NTHR;
+        const int g = i / D, d = i % D;
+        if (i >= GT * D || u.g0 + g >= a.G) continue;
+        const size_t e0 = u.p0 + (size_t)g * u.pstride;
+        float M = -INFINITY, L = 0.f, O = 0.f;
+        for (int s0 = 0; s0 < u.npieces; s0 += BATCH) {
+            float mm[BATCH], ll[BATCH], oo[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const int sp = min(s0 + j, u.npieces - 1);
+                const size_t e = e0 + (size_t)sp * u.sstride;
+                // (the loads of the own piece are issued like the others and their result dropped: no branch around a load)
+                const float pm = fetch(a.part_ml + e * 2), pl = fetch(a.part_ml + e * 2 + 1), po = fetch(a.part_o + e * D + d);
+                mm[j] = sp == mine ? Ms[k] : pm;
+                ll[j] = sp == mine ? Ls[k] : pl;
+                oo[j] = sp == mine ? Os[k] : po;
+            }
+            float bm = M;
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) bm = s0 + j < u.npieces ? fmaxf(bm, mm[j]) : bm;
+            const float keep = __builtin_amdgcn_exp2f(M - bm);
+            L *= keep;
+            O *= keep;
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const float wgt = s0 + j < u.npieces ? __builtin_amdgcn_exp2f(mm[j] - bm) : 0.f;
+                L = fmaf(ll[j], wgt, L);
+                O = fmaf(oo[j], wgt, O);
+            }
+            M = bm;
+        }
+        const int h = u.kvh * a.G + u.g0 + g;
+        static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + d] = from_f32<T>(O / L);
+    }
+}
+
 // Merge the NST softmax states the workgroup left in LDS (plus the new token's row in the last
 // split) and write either the output (single split) or this split's partial state.  The caller has
 // synchronised the workgroup on st_ml / st_acc / snew.
 template <typename T, int D, int GT, int NST, int NTHR>
 __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, float* st_ml, float* st_acc,
-                                            const float* snew, const float* sv)
+                                            const float* snew, const float* sv, int arrived_before)
 {
-    for (int i = lane_id_per_unit(); i < GT * D; i += NTHR) {
+    constexpr int E = (GT * D + NTHR - 1) / NTHR;             // elements per thread
+    const int tid = lane_id_per_unit();
+    float Ms[E], Ls[E], Os[E];
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+        const int i = tid + k * NTHR;
         const int g = i / D, d = i % D;
-        if (u.g0 + g >= a.G) continue;
+        Ms[k] = -INFINITY;
+        Ls[k] = Os[k] = 0.f;
+        if (i >= GT * D || u.g0 + g >= a.G) continue;
         float M = u.is_last ? snew[g] : -INFINITY;
         for (int r = 0; r < NST; ++r) M = fmaxf(M, st_ml[(r * GT + g) * 2]);
         float L = 0.f, O = 0.f;
@@ -286,6 +347,9 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, fl
             L += w;
             O = fmaf(sv[d], w, O);
         }
+        Ms[k] = M;
+        Ls[k] = L;
+        Os[k] = O;
         const int h = u.kvh * a.G + u.g0 + g;
         if (u.direct) {
             static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + d] = from_f32<T>(O / L);
@@ -295,13 +359,6 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, fl
             if (d == 0) {
                 a.part_ml[pi * 2] = M;
                 a.part_ml[pi * 2 + 1] = L;
-            }
-        } else {
-            const size_t pi = u.pbase + (size_t)g * u.pstride;
-            publish(a.part_o + pi * D + d, O);
-            if (d == 0) {
-                publish(a.part_ml + pi * 2, M);
-                publish(a.part_ml + pi * 2 + 1, L);
             }
         }
     }
@@ -326,10 +383,41 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, fl
     // an acquire fence in the merging piece: `a.ordered`, tuning key attn_ordered_finish) is kept and tested; its two
     // cache-maintenance instructions cost 8 % on a one-sequence step and 34 % on a 32-sequence ragged step on
     // MI355X (17.2 -> 18.5 us, 96 -> 129 us), which is why it is not the default.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();                                            // all stores done; st_ml no longer read
+    //
+    // The piece that finds all the others already there at its first look does not publish anything: it holds
+    // its own state in registers, reads the others (which were acknowledged before their adds, which came before
+    // the look) and writes the unit's output - two memory round trips fewer on the path of the piece that ends
+    // last, which with equal shares is the end of the kernel.
     int* arrived = reinterpret_cast<int*>(st_ml);                  // the merged states are no longer needed: reuse a word
-    const int tid = lane_id_per_unit();
+    __syncthreads();                                            // st_ml / st_acc no longer read by anyone
+    if (tid == 0) *arrived = arrived_before;
+    __syncthreads();
+    if (*arrived == u.npieces - 1) {
+        if (tid == 0) __hip_atomic_store(a.counters + u.counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
+        if (a.ordered) {
+            if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            __syncthreads();
+        }
+        const int mine = (int)((u.pbase - u.p0) / (size_t)u.sstride);
+        if (u.npieces <= 2) merge_pieces_local<T, D, GT, NTHR, 2, E>(a, u, tid, mine, Ms, Ls, Os);
+        else if (u.npieces <= 4) merge_pieces_local<T, D, GT, NTHR, 4, E>(a, u, tid, mine, Ms, Ls, Os);
+        else merge_pieces_local<T, D, GT, NTHR, 8, E>(a, u, tid, mine, Ms, Ls, Os);
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+        const int i = tid + k * NTHR;
+        const int g = i / D, d = i % D;
+        if (i >= GT * D || u.g0 + g >= a.G) continue;
+        const size_t pi = u.pbase + (size_t)g * u.pstride;
+        publish(a.part_o + pi * D + d, Os[k]);
+        if (d == 0) {
+            publish(a.part_ml + pi * 2, Ms[k]);
+            publish(a.part_ml + pi * 2 + 1, Ls[k]);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();                                            // all stores done
     if (tid == 0) {
         if (a.ordered) *arrived = __hip_atomic_fetch_add(a.counters + u.counter, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         else *arrived = __hip_atomic_fetch_add(a.counters + u.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -171,11 +171,14 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
         }
     };
 
+    int look = -1;                              // (fused finish: the other pieces' arrivals, asked near the end)
+    if (nfull == 0) look = first_look(a, u);
     if (r1 > r0) {
         int rbase = r0;
         if constexpr (DOUBLE_BUFFER) {
             for (int it = 0; it < nfull; it += 2) {
                 take_turns(a);
+                if (it + 2 >= nfull) look = first_look(a, u);
                 if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
                 consume(ka, va, rbase, std::false_type{});
                 if (it + 1 < nfull) {
@@ -188,6 +191,7 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
             // one register buffer: the other waves of the compute unit cover the load latency
             for (int it = 0; it < nfull; ++it) {
                 take_turns(a);
+                if (it + 1 >= nfull) look = first_look(a, u);
                 consume(ka, va, rbase, std::false_type{});
                 rbase += RPI;
                 if (it + 1 < nfull) issue(ka, va, rbase);
@@ -227,7 +231,7 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
                     st_acc[(size_t)(wave * GT + 4 * grp + r) * D + (cg * 16 + slot) * VEC + c] = o[cg * VEC + c][r];
     }
     __syncthreads();
-    finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv);
+    finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv, look);
 }
 
 template <int D, int GT, int NW, bool DOUBLE_BUFFER, bool BALANCED>
@@ -373,11 +377,14 @@ __device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeF
                     o[cg * VEC + c] = __builtin_amdgcn_mfma_f32_16x16x4f32(p[r], vv[cg * 4 + r].raw[c], o[cg * VEC + c], 0, 0, 0);
     };
 
+    int look = -1;                              // (fused finish: the other pieces' arrivals, asked near the end)
+    if (nfull == 0) look = first_look(a, u);
     if (r1 > r0) {
         int rbase = r0;
         // one register buffer: the other waves of the compute unit cover the load latency
         for (int it = 0; it < nfull; ++it) {
             take_turns(a);
+            if (it + 1 >= nfull) look = first_look(a, u);
             consume(ka, va, rbase, std::false_type{});
             rbase += RPI;
             if (it + 1 < nfull) issue(ka, va, rbase);
@@ -414,7 +421,7 @@ __device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeF
                     st_acc[(size_t)(wave * GT + 4 * grp + r) * D + (cg * 16 + slot) * VEC + c] = o[cg * VEC + c][r];
     }
     __syncthreads();
-    finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv);
+    finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv, look);
 }
 
 template <int D, int GT, int NW, bool BALANCED>

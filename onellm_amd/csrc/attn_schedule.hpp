@@ -39,6 +39,7 @@ struct AttnArgs {
     // fused finish (counters != NULL): one arrival counter per unit, zero between calls; the piece
     // that arrives last merges the unit's partial states itself and no merge kernel is launched
     int* counters;
+    int early_look;       // 1: a piece that finds all the others arrived merges the unit from its registers, unpublished
     int ordered;          // 1: the counter add is a release and the merging piece takes an acquire fence (agent scope)
 };
 

@@ -118,6 +118,8 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
         }
     };
 
+    int look = -1;                              // (fused finish: the other pieces' arrivals, asked near the end)
+    if (nfull == 0) look = first_look(a, u);
     if (r1 > r0) {
         // Full iterations are software-pipelined over two register buffers: the loads of the next
         // iteration are in flight while the current one is consumed, so a wave never sits with an
@@ -125,6 +127,7 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
         const bool none[U] = {};
         int rbase = r0;
         for (int it = 0; it < nfull; it += 2) {
+            if (it + 2 >= nfull) look = first_look(a, u);
             if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
             consume(ka, va, none, std::false_type{});
             if (it + 1 < nfull) {
@@ -161,7 +164,7 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
         }
     }
     __syncthreads();
-    finish_unit<T, D, GT, NRG, NTHR>(a, u, st_ml, st_acc, snew, sv);
+    finish_unit<T, D, GT, NRG, NTHR>(a, u, st_ml, st_acc, snew, sv, look);
 }
 
 template <typename T, int LPR, int GT, int U, int NW, bool BALANCED>

@@ -24,6 +24,7 @@ Knob g_knobs[] = {
     {"attn_gqa_valu", {-1}},     // 1: grouped-query heads on the vector ALU kernel instead of the MFMA one
     {"gemm_no_library", {-1}},   // 1: onellm_linear behaves as if the GEMM library had declined the problem (tests)
     {"attn_ordered_finish", {-1}}, // 1: release on the fused finish's counter add + acquire fence in the merging piece
+    {"attn_early_look", {-1}},   // 1 / 0: a piece that finds the unit's other pieces arrived merges it from its registers / never looks
     {"attn_turns", {-1}},        // 0: co-resident attention workgroups do not take turns at wave priority
 };
 }  // namespace

@@ -427,6 +427,8 @@ def test_fused_finish_soak_on_one_workspace(capi, dev):
                 capi.tune_set("attn_balanced_wgs", int(rng.choice([7, 100, 512, 1024])))
             if mode == 4:
                 capi.tune_set("attn_ordered_finish", 1)      # the formally ordered hand-over (release / acquire fence)
+            # the register-held merge by a piece that finds the others arrived: forced on, forced off, or the default
+            capi.tune_set("attn_early_look", [1, 0, -1][rep % 3])
             if rep % 20 == 0:
                 announce("attn fused soak, rep", rep)
             k, v = small[nb]
@@ -437,6 +439,7 @@ def test_fused_finish_soak_on_one_workspace(capi, dev):
             capi.tune_set("attn_balanced", -1)
             capi.tune_set("attn_balanced_wgs", -1)
             capi.tune_set("attn_ordered_finish", -1)
+            capi.tune_set("attn_early_look", -1)
             diff = (o_merge[:nb].float() - o_fused[:nb].float()).abs().max().item()
             assert diff <= 1e-3, "call %d (mode %d, batch %d, t %d): fused finish differs from the merge launch by %g" % (rep, mode, nb, t, diff)
         assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0, "arrival counters not back at zero"
@@ -444,6 +447,7 @@ def test_fused_finish_soak_on_one_workspace(capi, dev):
         capi.tune_set("attn_balanced", -1)
         capi.tune_set("attn_balanced_wgs", -1)
         capi.tune_set("attn_ordered_finish", -1)
+        capi.tune_set("attn_early_look", -1)
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,t", [(9, 32, 32, 600), (36, 32, 8, 600), (5, 64, 64, 1100), (20, 16, 8, 1300), (72, 32, 8, 330),
