@@ -561,6 +561,9 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     a.t_dev = t_dev; a.t_host = t_host;
     a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.G = Hq / Hkv; a.S = S;
     a.rotary_dim = rotary_dim; a.pos_offset = rope_pos_offset; a.flags = flags;
+    a.dbg_map = tune_get("dbg_map");
+    if (tune_get("dbg_lo") != -1 || tune_get("dbg_hi") != -1)
+        a.dbg = reinterpret_cast<long long*>(((unsigned long long)(unsigned)tune_get("dbg_hi") << 32) | (unsigned)tune_get("dbg_lo"));
     a.turns = tune_get("attn_turns") != 0;
     a.ordered = tune_get("attn_ordered_finish") == 1;
     a.early_look = 0;
@@ -640,10 +643,20 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
         // (what a change of unit costs a workgroup, in items: measured on the matrix-core kernel, where workgroups whose
         // equal-row shares held one / two / three units finished at 82 / 90 / 94 us of a 101 us step)
         const int user_cost = tune_get("attn_balanced_cost");
-        a.unit_cost = user_cost >= 0 ? user_cost : 3;
-        const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
         const int user_wgs = tune_get("attn_balanced_wgs");
-        long long nwg = user_wgs > 0 ? user_wgs : (uneven_grid && bal != 1 && grid_wgs < 512 ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
+        // Few long units with per-sequence lengths on the fp16 D = 128 matrix-core kernel (no more units than compute
+        // units, 4096 rows or more at the longest): one workgroup per compute unit, and a unit change charged six items.
+        // Two co-resident workgroups stream ~3 % more per unit of time, but do not finish together - measured finish
+        // times of 512 equal shares: mean 86, first 60-70, last 96 us of a 97 us step, against mean 88, last 94 with one
+        // workgroup per compute unit (config 3: 96.9 -> 94.3 us; 64 q / 8 kv heads, batch 16: 66.5 -> 64.3; lengths
+        // 7000..8192: 159 -> 155).  Many short units go the other way (96 sequences of 256..2048 rows: 79 against 86 us;
+        // D = 64, with half the bytes in flight per workgroup: 66 against 85), so they keep two per compute unit.
+        const bool few_long_units = t_dev && mfma_kernel && dtype == ONELLM_FP16 && D == 128
+                                    && (long)B * nunits <= kBalancedWorkgroups / 2 && items >= 64;
+        a.unit_cost = user_cost >= 0 ? user_cost : (few_long_units ? 6 : 3);
+        const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
+        long long nwg = user_wgs > 0 ? user_wgs
+                        : ((uneven_grid && bal != 1 && grid_wgs < 512) || few_long_units ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
         // (the matrix-core kernel for D = 256 keeps one workgroup per compute unit resident: a second 256 would only
         // queue behind the first - 16 sequences of 512..4096 rows x 4 kv heads: 65.7 -> 47.1 us)
         if (user_wgs <= 0 && mfma_kernel && dtype == ONELLM_FP16 && D == 256 && nwg > kBalancedWorkgroups / 2) nwg = kBalancedWorkgroups / 2;
