@@ -2,6 +2,7 @@
 
     python -m onellm_amd.build            # build what is out of date
     python -m onellm_amd.build --force    # rebuild everything
+    python -m onellm_amd.build --stamps   # only tests/cpp/libonellm_hip_stamps.so (attention timeline build)
 
 Outputs (next to this file): libonellm_hip.so (the C ABI of include/onellm_hip.h), libonellm_launchers.so (the
 launch* functions with oneLLM's own signatures), libonellm_gemm.so (the C ABI of include/onellm_gemm.h, over
@@ -30,6 +31,8 @@ LIB_HARNESS = os.path.join(ROOT, "tests", "cpp", "liblauncher_harness.so")
 # test-only: bare access-pattern kernels (what the memory system gives each kernel's access mix); timed by bench.py
 CEILINGS_SRC = os.path.join(ROOT, "tests", "cpp", "access_ceilings.hip")
 LIB_CEILINGS = os.path.join(ROOT, "tests", "cpp", "libaccess_ceilings.so")
+# test-only, built on request (--stamps): the kernel library with per-workgroup timeline stamps in the attention kernels
+LIB_STAMPS = os.path.join(ROOT, "tests", "cpp", "libonellm_hip_stamps.so")
 # test-only: a stand-alone C++ program that runs one decode step through the layers, like the reference's example driver
 DRIVER_SRC = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver.cpp")
 DRIVER_BIN = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver")
@@ -110,6 +113,24 @@ def kernel_resources(src):
     return out
 
 
+def build_stamps():
+    """The kernel library once more with -DONELLM_ATTN_STAMPS (tests/attn_timeline.py loads it): every attention
+    workgroup records when it started and ended and which XCD it ran on."""
+    os.makedirs(OBJ, exist_ok=True)
+    objs = []
+    for src in KERNEL_SOURCES:
+        obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".stamps.o")
+        cmd = [HIPCC, "-c", os.path.join(CSRC, src), "-o", obj, "-DONELLM_ATTN_STAMPS"] + COMMON
+        if src.endswith(".hip"):
+            cmd += DEVICE + (PRELOAD_KERNARGS if src in PRELOAD_SOURCES else [])
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for %s (stamps):\n%s" % (src, r.stderr[-4000:]))
+        objs.append(obj)
+    subprocess.run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_STAMPS] + objs, check=True)
+    return LIB_STAMPS
+
+
 def build(force=False, verbose=False):
     os.makedirs(OBJ, exist_ok=True)
     with concurrent.futures.ThreadPoolExecutor(max_workers=6) as ex:
@@ -153,5 +174,8 @@ def build(force=False, verbose=False):
 
 
 if __name__ == "__main__":
-    libs = build(force="--force" in sys.argv, verbose=True)
-    print("\n".join(libs))
+    if "--stamps" in sys.argv:
+        print(build_stamps())
+    else:
+        libs = build(force="--force" in sys.argv, verbose=True)
+        print("\n".join(libs))

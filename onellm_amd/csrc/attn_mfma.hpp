@@ -239,7 +239,9 @@ __global__ __launch_bounds__(NW * kWave)
 void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
 {
     extern __shared__ float lds[];
+    stamp_entry(a);
     for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_unit<D, GT, NW, DOUBLE_BUFFER>(a, fr, u, lds); });
+    stamp_end(a);
 }
 
 template <int D, int GT>

@@ -41,7 +41,35 @@ struct AttnArgs {
     int* counters;
     int early_look;       // 1: a piece that finds all the others arrived merges the unit from its registers, unpublished
     int ordered;          // 1: the counter add is a release and the merging piece takes an acquire fence (agent scope)
+#ifdef ONELLM_ATTN_STAMPS
+    long long* stamps;    // timeline build only: four words per workgroup (entry, end, XCC id, unused)
+#endif
 };
+
+// Timeline build (-DONELLM_ATTN_STAMPS, a separate test-side library): thread 0 of every workgroup records the
+// chip-wide 100 MHz clock at entry and after its last store was acknowledged, and the id of the XCD it runs on.
+#ifdef ONELLM_ATTN_STAMPS
+__device__ __forceinline__ void stamp_entry(const AttnArgs& a)
+{
+    if (a.stamps && threadIdx.x == 0) {
+        const long long wg = ((long long)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        a.stamps[wg * 4 + 0] = wall_clock64();
+        a.stamps[wg * 4 + 2] = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11));   // HW_REG_XCC_ID, bits 3:0
+    }
+}
+__device__ __forceinline__ void stamp_end(const AttnArgs& a)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (a.stamps && threadIdx.x == 0) {
+        const long long wg = ((long long)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        a.stamps[wg * 4 + 1] = wall_clock64();
+    }
+}
+#else
+__device__ __forceinline__ void stamp_entry(const AttnArgs&) {}
+__device__ __forceinline__ void stamp_end(const AttnArgs&) {}
+#endif
 
 // What one workgroup works on: a chunk of the history of one (sequence, kv-head) for up to GT query heads.
 struct Unit {

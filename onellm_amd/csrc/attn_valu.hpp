@@ -172,7 +172,9 @@ __global__ __launch_bounds__(NW * kWave)
 void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
 {
     extern __shared__ float lds[];
+    stamp_entry(a);
     for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { split_unit<T, LPR, LPR, GT, U, NW>(a, fr, u, lds); });
+    stamp_end(a);
 }
 
 // the same kernel for rows that do not fill their lanes (grid schedule only)

@@ -518,6 +518,12 @@ int static_scratch(hipStream_t st, void** out)
 }  // namespace
 }  // namespace onellm
 
+#ifdef ONELLM_ATTN_STAMPS
+namespace onellm { namespace { long long* g_stamp_buffer = nullptr; } }
+// timeline build only: device buffer of 4 * (workgroups of the launch) int64 words, or NULL to stop recording
+extern "C" void onellm_attn_set_stamp_buffer(void* buffer) { onellm::g_stamp_buffer = static_cast<long long*>(buffer); }
+#endif
+
 extern "C" size_t onellm_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int max_t)
 {
     (void)Hkv;
@@ -561,9 +567,9 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     a.t_dev = t_dev; a.t_host = t_host;
     a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.G = Hq / Hkv; a.S = S;
     a.rotary_dim = rotary_dim; a.pos_offset = rope_pos_offset; a.flags = flags;
-    a.dbg_map = tune_get("dbg_map");
-    if (tune_get("dbg_lo") != -1 || tune_get("dbg_hi") != -1)
-        a.dbg = reinterpret_cast<long long*>(((unsigned long long)(unsigned)tune_get("dbg_hi") << 32) | (unsigned)tune_get("dbg_lo"));
+#ifdef ONELLM_ATTN_STAMPS
+    a.stamps = g_stamp_buffer;
+#endif
     a.turns = tune_get("attn_turns") != 0;
     a.ordered = tune_get("attn_ordered_finish") == 1;
     a.early_look = 0;

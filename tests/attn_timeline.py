@@ -1,0 +1,98 @@
+"""Per-workgroup timeline of a decode-attention launch: when each workgroup ended and on which XCD it ran.
+
+    python -m onellm_amd.build --stamps          # builds tests/cpp/libonellm_hip_stamps.so (once)
+    python tests/attn_timeline.py [config2|config2_ctx512|config3|config3_full]
+
+Runs the kernel library built with -DONELLM_ATTN_STAMPS (the product sources plus two clock stamps per workgroup and
+the XCC id register) on synthetic inputs of the named BASELINE shape and prints, per XCD and per dispatch half
+(workgroups i and i + 256 land on the same compute unit), the mean / min / max end time in microseconds after the
+first workgroup's entry, over eight launches on rotating cache sets.  A measurement aid, not a test."""
+import ctypes
+import os
+import sys
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+from onellm_amd import capi  # noqa: E402
+
+SHAPES = {
+    "config2": dict(B=16, Hq=32, Hkv=32, S=4096, t=4096, ragged=False, nsets=4),
+    "config2_ctx512": dict(B=16, Hq=32, Hkv=32, S=4096, t=512, ragged=False, nsets=4),
+    "config3": dict(B=32, Hq=32, Hkv=8, S=8192, t=8192, ragged=True, nsets=3),
+    "config3_full": dict(B=32, Hq=32, Hkv=8, S=8192, t=8192, ragged=False, nsets=3),
+}
+
+
+def main():
+    name = sys.argv[1] if len(sys.argv) > 1 else "config2"
+    c = SHAPES[name]
+    lib_path = os.path.join(ROOT, "tests", "cpp", "libonellm_hip_stamps.so")
+    assert os.path.exists(lib_path), "build it first: python -m onellm_amd.build --stamps"
+    capi.LIB_PATH = lib_path
+    L = capi.lib()
+    L.onellm_attn_set_stamp_buffer.argtypes = [ctypes.c_void_p]
+    L.onellm_attn_set_stamp_buffer.restype = None
+    dev = torch.device("cuda:0")
+    D = 128
+    B, Hq, Hkv, S, t = c["B"], c["Hq"], c["Hkv"], c["S"], c["t"]
+    torch.manual_seed(2)
+    sets = [(torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half(), torch.randn(1, B, Hkv, S, D, device=dev).mul_(0.5).half())
+            for _ in range(c["nsets"])]
+    qkv = torch.randn(B, Hq + 2 * Hkv, D, device=dev).mul_(0.5).half()
+    bias = torch.randn((Hq + 2 * Hkv) * D, device=dev).mul_(0.5).half()
+    out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+    t_dev = None
+    if c["ragged"]:
+        t_dev = torch.from_numpy(np.random.default_rng(3).integers(1024, S + 1, size=B).astype(np.int32)).to(dev)
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    stamps = torch.zeros(8192 * 4, dtype=torch.int64, device=dev)
+
+    def step(i):
+        kc, vc = sets[i % len(sets)]
+        capi.decode_attn(qkv, bias, kc, vc, out, Hq, t, D, 10000.0, t_dev=t_dev, max_t=t, workspace=ws,
+                         flags=capi.ATTN_ZEROED_WORKSPACE)
+
+    for i in range(5):
+        step(i)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for i in range(50):
+        step(i)
+    ev1.record()
+    torch.cuda.synchronize()
+    print("%s: %.1f us per step (HIP events, 50 steps, stamps off)" % (name, ev0.elapsed_time(ev1) / 50 * 1e3))
+    ends, xcc = [], None
+    for rep in range(8):
+        stamps.zero_()
+        torch.cuda.synchronize()
+        L.onellm_attn_set_stamp_buffer(stamps.data_ptr())
+        step(rep)
+        torch.cuda.synchronize()
+        L.onellm_attn_set_stamp_buffer(None)
+        d = stamps.cpu().numpy().reshape(-1, 4)
+        used = d[:, 0] != 0
+        n = int(used.sum())
+        st, en = d[:n, 0], d[:n, 1]
+        xcc = d[:n, 2] & 0xF
+        ends.append((en - st.min()) / 100.0)           # 100 MHz clock
+        last_start = (st.max() - st.min()) / 100.0
+    e = np.mean(ends, axis=0)
+    n = len(e)
+    idx = np.arange(n)
+    print("workgroups %d; all started by %.1f us; end: mean %.1f, max %.1f, min %.1f us" % (n, last_start, e.mean(), e.max(), e.min()))
+    half = n // 2 if n >= 512 else n
+    for x in range(8):
+        a = e[(xcc == x) & (idx < half)]
+        line = "XCD %d: workgroups 0..%d end mean %.1f (min %.1f, max %.1f)" % (x, half - 1, a.mean(), a.min(), a.max())
+        if half < n:
+            b = e[(xcc == x) & (idx >= half)]
+            line += " | %d..%d end mean %.1f (min %.1f, max %.1f)" % (half, n - 1, b.mean(), b.min(), b.max())
+        print(line)
+
+
+if __name__ == "__main__":
+    main()
