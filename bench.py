@@ -532,8 +532,11 @@ def extras_section(capi, dev, args, with_cpu):
         from oracle import ref
         h = logits.cpu().numpy()
         cpu = time_cpu(lambda: ref.beam_topk(h, 8, 4, 4), 2.0)[0]
-    ex["beam_topk_b8_beam4_v32000_k4"] = with_graph(entry(ms, 32 * 32000 * 4, cpu),
-                                                    lambda i: capi.beam_topk(logits, 8, 4, 4, workspace=wsk))
+    e = entry(ms, 32 * 32000 * 4, cpu)
+    e["launches"] = capi.beam_topk_last_launches()          # launch by launch: both stages in one launch
+    e = with_graph(e, lambda i: capi.beam_topk(logits, 8, 4, 4, workspace=wsk))
+    e["launches_graph_replay"] = capi.beam_topk_last_launches()   # under capture: a second launch merges
+    ex["beam_topk_b8_beam4_v32000_k4"] = e
     del logits, wsk
     torch.cuda.empty_cache()
 

@@ -189,11 +189,20 @@ int onellm_kv_repeat(int dtype, const void* k_cache, const void* v_cache,
  * with K = beam = 2 the final results sit exactly where the reference's unit test reads them
  * (tests/unittests/test_beamsearch_topK.cu:33-35).
  * 1 <= K <= 8.  Slots with no candidate hold value -inf and id -1.
+ * On a stream that is not being captured both stages run in one kernel launch (the workgroup of a batch entry that
+ * stores its survivors last merges them), for up to 1024 batch entries and for the first 64 distinct workspace
+ * pointers a process passes; beyond either limit, and on a stream under capture, stage 2 is a second launch (a
+ * launch less is worth more to the host than the 1.5 us the longer kernel costs the device; a replayed graph has no
+ * host in it).  Same results either way.  Two calls that may overlap in time need two workspaces, as in the
+ * reference.
  */
 #define ONELLM_TOPK_BLOCKS_PER_ROW 8
 int onellm_beam_topk(const float* logits, int B, int beam, int V, int K,
                      float* workspace, onellm_stream_t stream);
 size_t onellm_beam_topk_workspace_bytes(int B, int beam, int K);
+/* kernel launches the last onellm_beam_topk call of this thread queued: 1 or 2 (0 before the first call or after
+ * a refused one).  No counterpart in the reference; for tests and profiles. */
+int onellm_beam_topk_last_launches(void);
 
 /* ------------------------------------------------------------------------------------------------
  * The callers either side of the decode path (built after the six entry points above).

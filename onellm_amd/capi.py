@@ -35,6 +35,7 @@ SYMBOLS = {
     "onellm_kv_repeat": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp]),
     "onellm_beam_topk": (_ci, [_vp, _ci, _ci, _ci, _ci, _vp, _vp]),
     "onellm_beam_topk_workspace_bytes": (_sz, [_ci, _ci, _ci]),
+    "onellm_beam_topk_last_launches": (_ci, []),
     "onellm_qkv_bias_rope_transpose": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci,
                                              _cf, _vp]),
     "onellm_silu_and_mul": (_ci, [_ci, _vp, _vp, _ci, _ci, _vp]),
@@ -175,6 +176,10 @@ def kv_repeat(k_cache, v_cache, k_dst, v_dst, context_len, layer=0):
 
 def beam_topk_workspace_bytes(B, beam, K):
     return lib().onellm_beam_topk_workspace_bytes(B, beam, K)
+
+
+def beam_topk_last_launches():
+    return lib().onellm_beam_topk_last_launches()
 
 
 def beam_topk(logits, B, beam, K, workspace=None):

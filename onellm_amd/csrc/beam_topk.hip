@@ -9,19 +9,58 @@
 // key 0 is the empty slot and loses against everything.  Values are read back from the logits by
 // index when results are stored, so the stored bits are the input's bits.
 //
-// Stage 1: each (row, block) pair scans the tokens it owns with a sorted K-slot list per lane in
-// registers, merges the 64 lists of a wave with lane exchanges (DPP inside 16 lanes, the crossbar
-// beyond) using a bitonic top-K merge (max of a[i] and b[K-1-i], then a bitonic sort), then the
-// waves of the workgroup through LDS.  Stage 2: one workgroup per batch entry merges the
-// beam*nblk*K survivors.  Traffic: the logits are read once (rows*V*4 bytes).
+// Stage 1: each (row, block) pair scans the tokens it owns.  A wave takes its values in batches (one
+// to sixteen per lane, all requested from memory at once) and keeps one sorted K-slot list for the whole wave in
+// registers every lane agrees on.  Of a batch it first takes a floor no member of the wave's top K can be
+// below - the lanes are cut into 2K groups, each group's largest value is found with lane exchanges, and the
+// K-th largest of those is the floor: K values at least that large exist - so one float compare per value
+// rejects all but a handful; the survivors rank themselves against each other (each one's key is read out
+// of its lane and compared in all lanes), the K best are merged into the wave's list, and that raises the
+// floor for what follows.  (Once a batch leaves survivors in more than sixteen lanes, or four in one lane -
+// ties, sorted input - the wave goes over to per-lane lists and a bitonic merge across the wave at the
+// end, which cost the same whatever the data; lists of eight always do.)  The four waves of a workgroup combine their lists through LDS with a bitonic
+// top-K merge (max of a[i] and b[K-1-i], then a bitonic sort).  Stage 2: the beam*nblk*K survivors of a
+// batch entry go through the same scan, in the stage-1 workgroup of that entry that finishes last (one
+// launch), or in a second launch with one workgroup per batch entry.  Traffic: the logits are read once
+// (rows*V*4 bytes).
+//
+// The one-launch form counts the workgroups of a batch entry that have stored their survivors in an arrival
+// counter.  The caller's workspace has no room for counters and is not zeroed, so they live in a file-scope
+// device array (zero when the module is loaded; the workgroup that merges sets its counter back to zero, so
+// every launch leaves them zero).  Launches that may overlap need counters of their own: a launch uses the
+// set that belongs to its workspace pointer (a small host-side table, filled as workspaces are first seen) -
+// two launches that share a workspace may not overlap anyway, they would overwrite each other's survivors.
+// A workspace that finds the table full, or a batch beyond the set's size, takes the two-launch form.
 #include <limits.h>
 #include <math.h>
+#include <mutex>
 #include "common.hpp"
 
 namespace onellm {
+int tune_get(const char* key);
 namespace {
 
 typedef unsigned long long Key;
+
+constexpr int kArrivalSets = 64;        // workspaces that can run the one-launch form (per process)
+constexpr int kArrivalEntries = 1024;   // batch entries per launch of the one-launch form
+__device__ unsigned g_arrivals[kArrivalSets * kArrivalEntries];
+
+thread_local int g_last_launches = 0;
+
+// the counter set of this workspace; -1: none left
+int arrival_set_of(const void* workspace)
+{
+    static std::mutex m;
+    static const void* owner[kArrivalSets];
+    static int used = 0;
+    std::lock_guard<std::mutex> lock(m);
+    for (int i = 0; i < used; ++i)
+        if (owner[i] == workspace) return i;
+    if (used == kArrivalSets) return -1;
+    owner[used] = workspace;
+    return used++;
+}
 
 __device__ __forceinline__ Key make_key(float v, int id)
 {
@@ -131,11 +170,165 @@ __device__ __forceinline__ void wave_merge(TopList<KP>& t)
     merge_xor<KP>(t, 32);
 }
 
-// workgroup of 256 lanes -> the lanes of wave 0 return the workgroup's KP best
+__device__ __forceinline__ float key_float(Key k)
+{
+    unsigned u = (unsigned)(k >> 32);
+    u ^= (u & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu;
+    return __uint_as_float(u);
+}
+
+__device__ __forceinline__ Key readlane_key(Key v, int lane)
+{
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(v & 0xFFFFFFFFu), lane);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(v >> 32), lane);
+    return ((Key)hi << 32) | lo;
+}
+
+__device__ __forceinline__ float readlane_f32(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// A value that at least KP of the wave's 64 values m reach: the lanes are cut into 2*KP groups, each group's
+// largest value is found with lane exchanges (NaN never wins against a number; a group of nothing but NaN counts
+// as -inf), and the KP-th largest of the group maxima is returned: every group counts the maxima above its own,
+// and a group that counts the most without exceeding KP-1 holds it.  The same in every lane.
+template <int KP>
+__device__ __forceinline__ float kth_group_maximum(float m)
+{
+    constexpr int NG = 2 * KP, G = 64 / NG;
+    m = fmaxf(m, dpp_f32<kDppQuadXor1>(m));
+    m = fmaxf(m, dpp_f32<kDppQuadXor2>(m));
+    if (G >= 8) m = fmaxf(m, dpp_f32<kDppRowHalfMirror>(m));
+    if (G >= 16) m = fmaxf(m, dpp_f32<kDppRowMirror>(m));
+    if (G >= 32) m = fmaxf(m, __shfl_xor(m, 16, kWave));
+    m = (m == m) ? m : -INFINITY;
+    int above = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) above += readlane_f32(m, g * G) > m ? 1 : 0;
+#pragma unroll
+    for (int i = KP - 1; i > 0; --i) {
+        const unsigned long long who = __builtin_amdgcn_ballot_w64(above == i);
+        if (who) return readlane_f32(m, __builtin_ctzll(who));
+    }
+    return readlane_f32(m, __builtin_ctzll(__builtin_amdgcn_ballot_w64(above == 0)));
+}
+
+// One wave's running top KP.  `top` holds the same values in every lane (it is only ever updated from values read
+// out of one lane, under control flow the whole wave takes); `lanes` is the per-lane list of the batch slots that
+// had too many survivors to read out one by one.
+template <int KP>
+struct WaveTop {
+    static constexpr int kRankAtMost = 16;
+    static constexpr bool kPerLaneOnly = KP > 4;   // lists of eight: ranking and merging them costs more than the per-lane road
+    TopList<KP> top, lanes;
+    float floor;
+    bool used_lanes;
+
+    __device__ __forceinline__ void clear()
+    {
+        top.clear();
+        lanes.clear();
+        floor = -INFINITY;
+        used_lanes = kPerLaneOnly;
+    }
+    // true: the wave has gone over to the per-lane lists for good; the caller inserts its values into `lanes` itself
+    __device__ __forceinline__ bool per_lane_road() const { return kPerLaneOnly || used_lanes; }
+    // before a batch: lane_max = the largest valid value this lane holds in the batch (-inf if none)
+    __device__ __forceinline__ void raise_floor(float lane_max)
+    {
+        if (kPerLaneOnly || used_lanes) return;
+        floor = fmaxf(floor, kth_group_maximum<KP>(lane_max));
+    }
+    // One candidate key per lane (0: none), in at most kRankAtMost lanes.  The lanes whose key beats the wave's K-th
+    // are the contenders: every contender counts the contenders' keys above its own (they are read out of their
+    // lanes one by one), the ones that count 0 .. KP-1 form a sorted list, and that list is merged into `top`.
+    __device__ __forceinline__ void offer(Key k)
+    {
+        const bool contends = k > top.k[KP - 1];
+        const unsigned long long m = __builtin_amdgcn_ballot_w64(contends);
+        if (m == 0) return;
+        if ((m & (m - 1)) == 0) {
+            top.insert(readlane_key(k, __builtin_ctzll(m)));
+        } else {
+            int above = 0;
+            for (unsigned long long mm = m; mm; mm &= mm - 1) above += readlane_key(k, __builtin_ctzll(mm)) > k ? 1 : 0;
+            TopList<KP> best;
+#pragma unroll
+            for (int i = 0; i < KP; ++i) {
+                const unsigned long long who = __builtin_amdgcn_ballot_w64(contends && above == i);
+                best.k[i] = who ? readlane_key(k, __builtin_ctzll(who)) : (Key)0;
+            }
+            if (top.k[0] == 0) top = best;
+            else top.merge(best);
+        }
+        if (top.k[KP - 1] != 0) floor = fmaxf(floor, key_float(top.k[KP - 1]));
+    }
+    // A batch of NV values per lane; bit j of `valid` says whether x[j] exists, and its flat index is
+    // id0 + (j / E) * id_step + j % E.  One compare per value marks what the floor does not reject (`!(x < floor)`
+    // keeps NaN, which the key order places); then each round offers every lane's next marked value, until no lane
+    // has one left - one or two rounds on ordinary data, NV on data that is all ties.
+    template <int NV, int E>
+    __device__ __forceinline__ void take(const float (&x)[NV], unsigned valid, int id0, int id_step)
+    {
+        if (kPerLaneOnly) {
+#pragma unroll
+            for (int j = 0; j < NV; ++j)
+                if ((valid >> j) & 1) lanes.insert(make_key(x[j], id0 + (j / E) * id_step + j % E));
+            return;
+        }
+        unsigned marked = valid;
+        if (!used_lanes) {
+            marked = 0;
+#pragma unroll
+            for (int j = 0; j < NV; ++j) marked |= !(x[j] < floor) ? (1u << j) : 0u;
+            marked &= valid;
+            // Ties and sorted input leave many values marked.  The rounds below cost about a hundred instructions
+            // each and a lane offers one value per round, so once a batch has a lane with four or more, or more
+            // lanes with one than can rank themselves, the wave takes the road whose cost does not depend on the
+            // data, for this batch and every later one: each value into the per-lane lists.
+            const unsigned long long holders = __builtin_amdgcn_ballot_w64(marked != 0);
+            if (holders == 0) return;
+            used_lanes = __builtin_popcountll(holders) > kRankAtMost ||
+                         __builtin_amdgcn_ballot_w64(__builtin_popcount(marked) >= 4) != 0;
+        }
+        if (used_lanes) {
+#pragma unroll
+            for (int j = 0; j < NV; ++j)
+                if ((marked >> j) & 1) lanes.insert(make_key(x[j], id0 + (j / E) * id_step + j % E));
+            return;
+        }
+        while (__builtin_amdgcn_ballot_w64(marked != 0) != 0) {
+            const int j = marked ? __builtin_ctz(marked) : 0;
+            float pick[NV];      // x[j] for a j that differs from lane to lane: halve the choice once per bit of j
+#pragma unroll
+            for (int i = 0; i < NV; ++i) pick[i] = x[i];
+#pragma unroll
+            for (int bit = 0; (NV >> bit) > 1; ++bit) {
+                const bool odd = (j >> bit) & 1;
+#pragma unroll
+                for (int i = 0; i < (NV >> (bit + 1)); ++i) pick[i] = odd ? pick[2 * i + 1] : pick[2 * i];
+            }
+            const float xv = pick[0];
+            const Key k = marked ? make_key(xv, id0 + (j / E) * id_step + j % E) : (Key)0;
+            marked &= marked - 1;
+            offer(k);
+        }
+    }
+    // after the last batch: every lane holds the wave's KP best in `top`
+    __device__ __forceinline__ void finish()
+    {
+        if (used_lanes) {
+            wave_merge<KP>(lanes);
+            top.merge(lanes);
+        }
+    }
+};
+
+// workgroup of 256 lanes, `t` the finished list of each wave -> the lanes of wave 0 return the workgroup's KP best
 template <int KP>
 __device__ __forceinline__ void block_merge(TopList<KP>& t, Key* skey)
 {
-    wave_merge<KP>(t);
     const int tid = threadIdx.x, wave = tid / kWave;
     if ((tid & (kWave - 1)) == 0) {
 #pragma unroll
@@ -156,17 +349,25 @@ __device__ __forceinline__ void block_merge(TopList<KP>& t, Key* skey)
 // ... (the reference's ownership: token tid + lane_blk*256 + m*nblk*256).  On the vector path a
 // thread reads 4 consecutive tokens of a chunk with one 16-byte load and four such loads are issued
 // before any candidate is inserted, so a block has its whole slice of the row in flight at once.
-template <int KP>
+//
+// FUSED: `set` >= 0 names the arrival counters; the workgroup that finds the other beam*nblk - 1 workgroups of its
+// batch entry arrived merges the entry's survivors and stores the final K.  Ordering: thread 0 stores the
+// workgroup's survivors, then adds to the counter with release order at device scope; the add of the last
+// arriver has acquire order and the barrier after it extends that to the workgroup, whose loads of the
+// survivors are device-scope loads (they do not take a line an earlier launch left in this compute unit's cache).
+template <int KP, bool FUSED>
 __global__ __launch_bounds__(256)
 void topk_stage1_kernel(const float* __restrict__ logits, int V, int nblk, int vec_ok, int K,
-                        float* __restrict__ vals, int* __restrict__ ids)
+                        float* __restrict__ vals, int* __restrict__ ids, int set, int beam,
+                        float* __restrict__ fvals, int* __restrict__ fids)
 {
     __shared__ Key skey[4 * KP];
+    __shared__ int s_last;
     const int row = blockIdx.x / nblk, lane_blk = blockIdx.x % nblk;
     const float* p = logits + (size_t)row * V;
     const int flat0 = row * V;
-    TopList<KP> t;
-    t.clear();
+    WaveTop<KP> w;
+    w.clear();
     if (vec_ok) {
         constexpr int PASSES = 4;
         const int nchunks = (V + 255) / 256;
@@ -177,27 +378,114 @@ void topk_stage1_kernel(const float* __restrict__ logits, int V, int nblk, int v
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) {
                 tok[q] = (c0 + nblk * 4 * q) * 256 + l4;
+                v[q] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
                 if (tok[q] < V) v[q] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + tok[q]));
             }
+            if (w.per_lane_road()) {
+#pragma unroll
+                for (int q = 0; q < PASSES; ++q) {
+                    if (tok[q] < V) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) w.lanes.insert(make_key(v[q][e], flat0 + tok[q] + e));
+                    }
+                }
+                continue;
+            }
+            float x[4 * PASSES];
+            float lane_max = -INFINITY;
+            unsigned valid = 0;
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) {
-                if (tok[q] < V) {          // V % 4 == 0 here, so tok < V means tok + 3 < V
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) t.insert(make_key(v[q][e], flat0 + tok[q] + e));
+                for (int e = 0; e < 4; ++e) x[4 * q + e] = v[q][e];
+                if (tok[q] < V) {      // V % 4 == 0 here, so tok < V means tok + 3 < V
+                    valid |= 0xFu << (4 * q);
+                    lane_max = fmaxf(fmaxf(lane_max, fmaxf(v[q][0], v[q][1])), fmaxf(v[q][2], v[q][3]));
                 }
             }
+            w.raise_floor(lane_max);
+            w.template take<4 * PASSES, 4>(x, valid, flat0 + tok[0], nblk * 4 * 256);
         }
     } else {
-        for (int tok = threadIdx.x + lane_blk * 256; tok < V; tok += nblk * 256) t.insert(make_key(p[tok], flat0 + tok));
+        constexpr int PASSES = 8;
+        for (int tok0 = threadIdx.x + lane_blk * 256; tok0 - (int)threadIdx.x < V; tok0 += nblk * 256 * PASSES) {
+            float x[PASSES];
+            unsigned valid = 0;
+#pragma unroll
+            for (int q = 0; q < PASSES; ++q) {
+                const int tok = tok0 + q * nblk * 256;
+                x[q] = -INFINITY;
+                if (tok < V) {
+                    x[q] = p[tok];
+                    valid |= 1u << q;
+                }
+            }
+            if (w.per_lane_road()) {
+#pragma unroll
+                for (int q = 0; q < PASSES; ++q)
+                    if ((valid >> q) & 1) w.lanes.insert(make_key(x[q], flat0 + tok0 + q * nblk * 256));
+                continue;
+            }
+            float lane_max = -INFINITY;
+#pragma unroll
+            for (int q = 0; q < PASSES; ++q) lane_max = fmaxf(lane_max, x[q]);
+            w.raise_floor(lane_max);
+            w.template take<PASSES, 1>(x, valid, flat0 + tok0, nblk * 256);
+        }
     }
+    w.finish();
+    TopList<KP>& t = w.top;
     block_merge<KP>(t, skey);
     if (threadIdx.x == 0) {
 #pragma unroll
         for (int i = 0; i < KP; ++i) {
             if (i < K) {
                 const int id = key_id(t.k[i]);
-                vals[(size_t)blockIdx.x * K + i] = key_value(t.k[i], id, logits);
-                ids[(size_t)blockIdx.x * K + i] = id;
+                const float v = key_value(t.k[i], id, logits);
+                if (FUSED) {
+                    __hip_atomic_store(&vals[(size_t)blockIdx.x * K + i], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(&ids[(size_t)blockIdx.x * K + i], id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else {
+                    vals[(size_t)blockIdx.x * K + i] = v;
+                    ids[(size_t)blockIdx.x * K + i] = id;
+                }
+            }
+        }
+    }
+    if (!FUSED) return;
+    const int b = row / beam, pieces = beam * nblk;
+    if (threadIdx.x == 0) {
+        unsigned* ctr = &g_arrivals[set * kArrivalEntries + b];
+        const unsigned before = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = before == (unsigned)(pieces - 1);
+        if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = last;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    const int n = pieces * K;
+    w.clear();
+    for (int i0 = 0; i0 < n; i0 += 256) {
+        const int i = i0 + threadIdx.x;
+        int id = -1;
+        float v = -INFINITY;
+        if (i < n) {
+            id = __hip_atomic_load(&ids[(size_t)b * n + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            v = __hip_atomic_load(&vals[(size_t)b * n + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        const float x[1] = {v};
+        w.raise_floor(id != -1 ? v : -INFINITY);
+        w.template take<1, 1>(x, id != -1 ? 1u : 0u, id, 0);
+    }
+    w.finish();
+    block_merge<KP>(t, skey);
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            if (i < K) {
+                const int id = key_id(t.k[i]);
+                fvals[(size_t)b * K + i] = key_value(t.k[i], id, logits);
+                fids[(size_t)b * K + i] = id;
             }
         }
     }
@@ -211,12 +499,18 @@ void topk_stage2_kernel(const float* __restrict__ logits, const float* __restric
 {
     __shared__ Key skey[4 * KP];
     const int b = blockIdx.x;
-    TopList<KP> t;
-    t.clear();
-    for (int i = threadIdx.x; i < n; i += 256) {
-        const int id = ids[(size_t)b * n + i];
-        if (id != -1) t.insert(make_key(vals[(size_t)b * n + i], id));
+    WaveTop<KP> w;
+    w.clear();
+    for (int i0 = 0; i0 < n; i0 += 256) {
+        const int i = i0 + threadIdx.x;
+        const int id = i < n ? ids[(size_t)b * n + i] : -1;
+        const float v = i < n ? vals[(size_t)b * n + i] : -INFINITY;
+        const float x[1] = {v};
+        w.raise_floor(id != -1 ? v : -INFINITY);
+        w.template take<1, 1>(x, id != -1 ? 1u : 0u, id, 0);
     }
+    w.finish();
+    TopList<KP>& t = w.top;
     block_merge<KP>(t, skey);
     if (threadIdx.x == 0) {
 #pragma unroll
@@ -239,10 +533,32 @@ int launch_topk(const float* logits, int B, int beam, int V, int K, int nblk, fl
     float* fvals = reinterpret_cast<float*>(ids + n1);
     int* fids = reinterpret_cast<int*>(fvals + (size_t)B * K);
     const int vec_ok = (V % 4 == 0) && aligned16(logits);
-    hipLaunchKernelGGL((topk_stage1_kernel<KP>), dim3(B * beam * nblk), dim3(256), 0, st, logits, V, nblk, vec_ok, K, vals, ids);
+    // One launch costs the host a launch less and the device about 1.5 us more (the store - count - load chain
+    // of the last workgroup is longer than a second launch's start-up): it is the form of a stream that runs
+    // launch by launch, where the host is the limit; a stream under capture, whose launches will be replayed
+    // without the host, gets the two-launch form.
+    int two = tune_get("topk_two_launches");
+    if (two < 0) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cs) != hipSuccess) {
+            (void)hipGetLastError();
+            cs = hipStreamCaptureStatusNone;
+        }
+        two = cs != hipStreamCaptureStatusNone;
+    }
+    const int set = (B <= kArrivalEntries && !two) ? arrival_set_of(ws) : -1;
+    if (set >= 0) {
+        hipLaunchKernelGGL((topk_stage1_kernel<KP, true>), dim3(B * beam * nblk), dim3(256), 0, st, logits, V, nblk, vec_ok, K,
+                           vals, ids, set, beam, fvals, fids);
+        g_last_launches = 1;
+        return launch_status();
+    }
+    hipLaunchKernelGGL((topk_stage1_kernel<KP, false>), dim3(B * beam * nblk), dim3(256), 0, st, logits, V, nblk, vec_ok, K,
+                       vals, ids, -1, beam, fvals, fids);
     int rc = launch_status();
     if (rc) return rc;
     hipLaunchKernelGGL((topk_stage2_kernel<KP>), dim3(B), dim3(256), 0, st, logits, vals, ids, beam * nblk * K, K, fvals, fids);
+    g_last_launches = 2;
     return launch_status();
 }
 
@@ -260,6 +576,7 @@ extern "C" int onellm_beam_topk(const float* logits, int B, int beam, int V, int
                                 onellm_stream_t stream)
 {
     using namespace onellm;
+    g_last_launches = 0;
     if (!logits || !workspace || B <= 0 || beam <= 0 || V <= 0) return ONELLM_EINVAL;
     if (K < 1 || K > 8) return ONELLM_EUNSUPPORTED;
     if ((long)B * beam * V > (long)INT_MAX - 1) return ONELLM_EUNSUPPORTED;   // ids are int32 flat indices
@@ -270,3 +587,5 @@ extern "C" int onellm_beam_topk(const float* logits, int B, int beam, int V, int
     if (K <= 4) return launch_topk<4>(logits, B, beam, V, K, nblk, workspace, st);
     return launch_topk<8>(logits, B, beam, V, K, nblk, workspace, st);
 }
+
+extern "C" int onellm_beam_topk_last_launches(void) { return onellm::g_last_launches; }

@@ -25,6 +25,7 @@ Knob g_knobs[] = {
     {"gemm_no_library", {-1}},   // 1: onellm_linear behaves as if the GEMM library had declined the problem (tests)
     {"attn_ordered_finish", {-1}}, // 1: release on the fused finish's counter add + acquire fence in the merging piece
     {"attn_early_look", {-1}},   // 1 / 0: a piece that finds the unit's other pieces arrived merges it from its registers / never looks
+    {"topk_two_launches", {-1}}, // beam top-K: 1 = always a second launch for the merge of the survivors, 0 = one launch wherever it can be (also under capture)
     {"attn_turns", {-1}},        // 0: co-resident attention workgroups do not take turns at wave priority
 };
 }  // namespace

@@ -19,7 +19,7 @@ def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ["onellm_decode_attn", "onellm_decode_attn_workspace_bytes", "onellm_rmsnorm",
                  "onellm_fused_add_bias_residual_rmsnorm", "onellm_kv_append", "onellm_kv_repeat",
-                 "onellm_beam_topk", "onellm_beam_topk_workspace_bytes", "onellm_error_string", "onellm_hip_version",
+                 "onellm_beam_topk", "onellm_beam_topk_workspace_bytes", "onellm_beam_topk_last_launches", "onellm_error_string", "onellm_hip_version",
                  "onellm_qkv_bias_rope_transpose", "onellm_silu_and_mul", "onellm_topk_sample",
                  "onellm_decode_attn_static"]:
         assert must in names

@@ -1,4 +1,6 @@
 """GPU parity of KV concat, KV repeat and beam top-K against the CPU oracle (bit-exact), through the C ABI."""
+import zlib
+
 import numpy as np
 import pytest
 import torch
@@ -99,13 +101,21 @@ def test_repeat_matches_oracle(capi, ref, dev, dtype, Hq, Hkv, D):
 
 # ---------------------------------------------------------------- beam top-K
 
+@pytest.fixture(params=["one_launch", "two_launches"])
+def topk_form(request, capi):
+    """Both forms of the second stage: merged by the last stage-1 workgroup of a batch entry, or by a second launch."""
+    capi.tune_set("topk_two_launches", 1 if request.param == "two_launches" else 0)
+    yield request.param
+    capi.tune_set("topk_two_launches", -1)
+
+
 def _lexsort_topk(flat_vals, flat_ids, K):
     order = np.lexsort((flat_ids, -flat_vals.astype(np.float64)))[:K]
     return flat_vals[order], flat_ids[order]
 
 
-def test_topk_reference_unit_vector(capi, dev):
-    announce("topk unit vector")
+def test_topk_reference_unit_vector(capi, dev, topk_form):
+    announce("topk unit vector", topk_form)
     logits = torch.arange(60000, dtype=torch.float32, device=dev).view(2, 30000)
     ws, _, _, fv, fi = capi.beam_topk(logits, 1, 2, 2)
     np.testing.assert_array_equal(fi.cpu().numpy(), [[59999, 59998]])
@@ -115,8 +125,8 @@ def test_topk_reference_unit_vector(capi, dev):
     assert w[2 * 1 * 2 * 8 * 2] == 59999.0 and w.view(np.int32)[2 * 1 * 2 * 8 * 2 + 1 * 2] == 59999
 
 
-def test_topk_config5_planted_ties(capi, ref, dev):
-    announce("topk cfg5")
+def test_topk_config5_planted_ties(capi, ref, dev, topk_form):
+    announce("topk cfg5", topk_form)
     rng = np.random.default_rng(5)
     B, beam, V, K = 8, 4, 32000, 4
     logits = (rng.standard_normal((B * beam, V)) * 2.0).astype(np.float32)
@@ -139,8 +149,8 @@ def test_topk_config5_planted_ties(capi, ref, dev):
 
 @pytest.mark.parametrize("B,beam,V,K", [(1, 1, 1, 1), (2, 3, 100, 8), (3, 2, 257, 5), (1, 4, 2049, 3), (5, 1, 50000, 2),
                                         (2, 2, 128256, 4), (1, 1, 3, 8)])
-def test_topk_shapes_with_heavy_ties(capi, ref, dev, B, beam, V, K):
-    announce("topk", B, beam, V, K)
+def test_topk_shapes_with_heavy_ties(capi, ref, dev, B, beam, V, K, topk_form):
+    announce("topk", B, beam, V, K, topk_form)
     rng = np.random.default_rng(V + K)
     # few distinct values => many ties, the order of equal values is what is being checked
     logits = rng.integers(-3, 4, size=(B * beam, V)).astype(np.float32)
@@ -151,8 +161,72 @@ def test_topk_shapes_with_heavy_ties(capi, ref, dev, B, beam, V, K):
     np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), wfv.view(np.uint32))
 
 
-def test_topk_negative_infinity_and_run_to_run(capi, ref, dev):
-    announce("topk -inf")
+def _pattern(name, rows, V, rng):
+    if name == "normal":
+        return rng.standard_normal((rows, V)).astype(np.float32)
+    if name == "ascending":        # every later token beats all earlier ones: nothing can be rejected early
+        return (np.arange(rows * V, dtype=np.float32).reshape(rows, V) * 0.25)
+    if name == "descending":
+        return -(np.arange(rows * V, dtype=np.float32).reshape(rows, V) * 0.25)
+    if name == "all_equal":
+        return np.full((rows, V), 1.5, np.float32)
+    if name == "masked_ranges":    # whole stretches of the vocabulary at -inf, as a banned-token mask leaves them
+        a = rng.standard_normal((rows, V)).astype(np.float32)
+        for r in range(rows):
+            lo = int(rng.integers(0, V))
+            a[r, lo:lo + V // 3] = -np.inf
+            a[r, ::7] = -np.inf
+        return a
+    if name == "few_finite":       # fewer finite values than K in some rows
+        a = np.full((rows, V), -np.inf, np.float32)
+        for r in range(rows):
+            idx = rng.integers(0, V, size=r % 4)
+            a[r, idx] = rng.standard_normal(len(idx)).astype(np.float32)
+        return a
+    if name == "sawtooth":         # rising runs of 64 tokens: many lanes of a wave hold a contender at once
+        return ((np.arange(rows * V) % 64).astype(np.float32) + rng.integers(0, 3, size=rows * V).astype(np.float32)).reshape(rows, V)
+    raise ValueError(name)
+
+
+@pytest.mark.parametrize("pattern", ["normal", "ascending", "descending", "all_equal", "masked_ranges", "few_finite", "sawtooth"])
+@pytest.mark.parametrize("B,beam,V,K", [(2, 2, 32000, 4), (1, 3, 32000, 8), (2, 1, 50257, 2), (1, 2, 128256, 1), (1, 2, 151937, 5)])
+def test_topk_data_patterns(capi, ref, dev, topk_form, pattern, B, beam, V, K):
+    """What the scan does depends on the data (how many values pass the floor, how many lanes hold a contender at
+    once, how many rounds a batch takes); the result must not.  Vocabulary sizes with and without the 16-byte
+    path, one to four batches per wave."""
+    announce("topk pattern", pattern, B, beam, V, K, topk_form)
+    rng = np.random.default_rng(zlib.crc32(("%s %d %d" % (pattern, V, K)).encode()))
+    logits = _pattern(pattern, B * beam, V, rng)
+    _, v1, i1, fv, fi = capi.beam_topk(torch.from_numpy(logits).to(dev), B, beam, K)
+    w1v, w1i, wfv, wfi = ref.beam_topk(logits, B, beam, K)
+    np.testing.assert_array_equal(i1.cpu().numpy(), w1i)
+    np.testing.assert_array_equal(v1.cpu().numpy().view(np.uint32), w1v.view(np.uint32))
+    np.testing.assert_array_equal(fi.cpu().numpy(), wfi)
+    np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), wfv.view(np.uint32))
+
+
+def test_topk_nan_inputs_finish_and_keep_the_finite_order(capi, dev, topk_form):
+    """NaN has no place in the reference's order (its comparisons are all false for NaN); here a NaN with the sign
+    bit clear sorts above +inf and one with it set below -inf.  Checked: the call finishes, the ids are valid, and a
+    row's finite values keep their order below the positive NaNs."""
+    announce("topk NaN", topk_form)
+    B, beam, V, K = 1, 2, 4096, 4
+    rng = np.random.default_rng(3)
+    logits = rng.standard_normal((B * beam, V)).astype(np.float32)
+    logits[0, [10, 2000]] = np.float32(np.nan)
+    logits[1, 77] = -np.float32(np.nan)
+    logits.view(np.uint32)[1, 77] |= 0x80000000
+    _, _, _, fv, fi = capi.beam_topk(torch.from_numpy(logits).to(dev), B, beam, K)
+    ids = fi.cpu().numpy()[0]
+    assert list(ids[:2]) == [10, 2000] and np.isnan(fv.cpu().numpy()[0, :2]).all()
+    finite = logits.reshape(-1).copy()
+    finite[[10, 2000, V + 77]] = -np.inf
+    order = np.lexsort((np.arange(finite.size), -finite.astype(np.float64)))[:2]
+    np.testing.assert_array_equal(ids[2:], order)
+
+
+def test_topk_negative_infinity_and_run_to_run(capi, ref, dev, topk_form):
+    announce("topk -inf", topk_form)
     logits = np.full((2, 1000), -np.inf, np.float32)
     logits[0, 500] = 1.0
     d = torch.from_numpy(logits).to(dev)
@@ -165,10 +239,10 @@ def test_topk_negative_infinity_and_run_to_run(capi, ref, dev):
     assert torch.equal(a, fi2)
 
 
-def test_topk_zeros_of_both_signs_and_extreme_values(capi, ref, dev):
+def test_topk_zeros_of_both_signs_and_extreme_values(capi, ref, dev, topk_form):
     """-0.0 and +0.0 tie (the lower index wins) and every stored value carries the bits of the input it came from:
     zeros keep their sign, denormals, the largest finite value and infinities come back unchanged."""
-    announce("topk signed zeros and extreme values")
+    announce("topk signed zeros and extreme values", topk_form)
     B, beam, V, K = 2, 2, 600, 4
     logits = -np.abs(np.random.default_rng(17).standard_normal((B * beam, V)).astype(np.float32)) - 1.0
     logits[0, [5, 300, 599]] = [-0.0, 0.0, -0.0]                 # three zeros on top: indices 5, 300, 599 in this order
@@ -185,3 +259,76 @@ def test_topk_zeros_of_both_signs_and_extreme_values(capi, ref, dev):
     np.testing.assert_array_equal(got_i[0], [5, 300, 599, V + 7])
     flat = logits.reshape(-1)
     np.testing.assert_array_equal(got_v.view(np.uint32), flat[got_i].view(np.uint32))   # the input's own bits
+
+
+def test_topk_one_launch_repeats_on_one_workspace_and_falls_back_past_its_limits(capi, ref, dev):
+    """The one-launch form leaves its arrival counters as it found them: 150 calls on one workspace, shapes and K
+    changing from call to call, all equal to the oracle.  A process that passes more distinct workspaces than there are
+    counter sets gets the two-launch form for the surplus ones, with the same results."""
+    announce("topk one launch: repeats, changing shapes, more workspaces than counter sets")
+    rng = np.random.default_rng(99)
+    shapes = [(8, 4, 32000, 4), (3, 2, 257, 5), (1, 4, 2049, 3), (5, 1, 5000, 2), (2, 3, 100, 8), (16, 2, 1024, 1)]
+    cases = []
+    for B, beam, V, K in shapes:
+        logits = rng.integers(-50, 51, size=(B * beam, V)).astype(np.float32)
+        cases.append((B, beam, K, torch.from_numpy(logits).to(dev), ref.beam_topk(logits, B, beam, K)))
+    big = torch.empty(max(capi.beam_topk_workspace_bytes(B, beam, K) for B, beam, _, K in shapes) // 4, dtype=torch.float32, device=dev)
+    launches = set()
+    for it in range(150):
+        B, beam, K, d, want = cases[it % len(cases)]
+        _, v1, i1, fv, fi = capi.beam_topk(d, B, beam, K, workspace=big)
+        launches.add(capi.beam_topk_last_launches())
+        np.testing.assert_array_equal(i1.cpu().numpy(), want[1], err_msg="call %d" % it)
+        np.testing.assert_array_equal(fi.cpu().numpy(), want[3], err_msg="call %d" % it)
+        np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), want[2].view(np.uint32), err_msg="call %d" % it)
+    assert launches == {1}, launches
+    B, beam, K, d, want = cases[0]
+    held = [torch.empty(capi.beam_topk_workspace_bytes(B, beam, K) // 4, dtype=torch.float32, device=dev) for _ in range(80)]
+    seen = []
+    for w in held:
+        _, _, _, fv, fi = capi.beam_topk(d, B, beam, K, workspace=w)
+        seen.append(capi.beam_topk_last_launches())
+        np.testing.assert_array_equal(fi.cpu().numpy(), want[3])
+        np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), want[2].view(np.uint32))
+    assert seen[-1] == 2 and set(seen) == {1, 2}, seen
+    # a workspace the table knows keeps its one-launch form
+    capi.beam_topk(d, B, beam, K, workspace=big)
+    assert capi.beam_topk_last_launches() == 1
+
+
+@pytest.mark.parametrize("forced_one_launch", [False, True])
+def test_topk_graph_replays(capi, ref, dev, forced_one_launch):
+    """Captured once, replayed five times with eager calls on the same workspace (and so the same arrival counters) in
+    between: every replay equals the oracle.  A capturing stream gets the two-launch form unless told otherwise."""
+    announce("topk under graph replay, one launch forced:", forced_one_launch)
+    rng = np.random.default_rng(7)
+    B, beam, V, K = 8, 4, 32000, 4
+    logits = rng.integers(-1000, 1001, size=(B * beam, V)).astype(np.float32)
+    want = ref.beam_topk(logits, B, beam, K)
+    d = torch.from_numpy(logits).to(dev)
+    ws = torch.empty(capi.beam_topk_workspace_bytes(B, beam, K) // 4, dtype=torch.float32, device=dev)
+    capi.beam_topk(d, B, beam, K, workspace=ws)
+    assert capi.beam_topk_last_launches() == 1
+    torch.cuda.synchronize()
+    capi.tune_set("topk_two_launches", 0 if forced_one_launch else -1)
+    try:
+        side = torch.cuda.Stream()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                capi.beam_topk(d, B, beam, K, workspace=ws)
+            assert capi.beam_topk_last_launches() == (1 if forced_one_launch else 2)
+    finally:
+        capi.tune_set("topk_two_launches", -1)
+    torch.cuda.synchronize()
+    n1 = B * beam * 8 * K
+    for rep in range(5):
+        ws.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        fv = ws[2 * n1:2 * n1 + B * K].view(B, K).cpu().numpy()
+        fi = ws[2 * n1 + B * K:2 * n1 + 2 * B * K].view(torch.int32).view(B, K).cpu().numpy()
+        np.testing.assert_array_equal(fi, want[3], err_msg="replay %d" % rep)
+        np.testing.assert_array_equal(fv.view(np.uint32), want[2].view(np.uint32), err_msg="replay %d" % rep)
+        _, _, _, _, fi2 = capi.beam_topk(d, B, beam, K, workspace=ws)      # eager, same counters
+        np.testing.assert_array_equal(fi2.cpu().numpy(), want[3])

@@ -61,8 +61,11 @@ def test_streaming_kernels_keep_full_occupancy(resources):
     # norm rows of up to 16 KiB (the measured shapes): 512 threads per row, four workgroups per CU = eight waves per SIMD
     for name, r in _matching(resources["norms.hip"], r"norm_row_kernelI(f|6__half)Li[12]ELi512E").items():
         assert r["occupancy"] == 8 and r["vgprs"] <= 64, (name, r)
-    for src in ("kv_cache.hip", "activation.hip", "beam_topk.hip", "sampling.hip"):
+    for src in ("kv_cache.hip", "activation.hip", "sampling.hip"):
         for name, r in resources[src].items():
             assert r["occupancy"] == 8, (src, name, r)
+    # beam top-K: one 4-wave workgroup per CU is all a launch brings; the wave-wide list lives in scalar registers
+    for name, r in resources["beam_topk.hip"].items():
+        assert r["occupancy"] >= 4 and r["vgprs"] <= 64, (name, r)
     for name, r in _matching(resources["prefill_rope.hip"], r"rows_kernel").items():
         assert r["occupancy"] >= 4, (name, r)
