@@ -76,8 +76,23 @@ def time_steps(fn, steps, warmup):
 def time_steps_median(fn, steps, warmup, blocks=3):
     """Median of `blocks` consecutive time_steps() measurements (each `steps` launches): one disturbed block - another
     process's burst, a clock change - does not decide the figure."""
+    settle(fn)
     times = sorted(time_steps(fn, steps, warmup if k == 0 else 2) for k in range(blocks))
     return times[len(times) // 2]
+
+
+def settle(fn, seconds=0.02):
+    """Keep the GPU busy with the step for ~20 ms before an extras line is timed.  Coming out of an idle phase the
+    clocks take 10-15 ms to settle (the same kernel measured 159 us for its first ten launches, 171-187 for the next
+    sixty, 158.6 from then on); the headline value is not treated this way - it follows --warmup / --steps."""
+    import time
+    import torch
+    t0, i = time.perf_counter(), 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
 
 
 def time_steps_graph(fn, per_graph=20, replays=10):

@@ -42,12 +42,13 @@ struct AttnArgs {
     int early_look;       // 1: a piece that finds all the others arrived merges the unit from its registers, unpublished
     int ordered;          // 1: the counter add is a release and the merging piece takes an acquire fence (agent scope)
 #ifdef ONELLM_ATTN_STAMPS
-    long long* stamps;    // timeline build only: four words per workgroup (entry, end, XCC id, unused)
+    long long* stamps;    // timeline build only: four words per workgroup (entry, end, XCC id, HW_ID)
 #endif
 };
 
 // Timeline build (-DONELLM_ATTN_STAMPS, a separate test-side library): thread 0 of every workgroup records the
-// chip-wide 100 MHz clock at entry and after its last store was acknowledged, and the id of the XCD it runs on.
+// chip-wide 100 MHz clock at entry and after its last store was acknowledged, the id of the XCD and of the compute
+// unit (shader engine, array, unit) it runs on.
 #ifdef ONELLM_ATTN_STAMPS
 __device__ __forceinline__ void stamp_entry(const AttnArgs& a)
 {
@@ -55,6 +56,7 @@ __device__ __forceinline__ void stamp_entry(const AttnArgs& a)
         const long long wg = ((long long)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
         a.stamps[wg * 4 + 0] = wall_clock64();
         a.stamps[wg * 4 + 2] = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11));   // HW_REG_XCC_ID, bits 3:0
+        a.stamps[wg * 4 + 3] = __builtin_amdgcn_s_getreg(4 | (0 << 6) | ((32 - 1) << 11));   // HW_REG_HW_ID: cu 11:8, sh 12, se 15:13
     }
 }
 __device__ __forceinline__ void stamp_end(const AttnArgs& a)

@@ -1,7 +1,7 @@
 """Per-workgroup timeline of a decode-attention launch: when each workgroup ended and on which XCD it ran.
 
     python -m onellm_amd.build --stamps          # builds tests/cpp/libonellm_hip_stamps.so (once)
-    python tests/attn_timeline.py [config2|config2_ctx512|config3|config3_full]
+    python tests/attn_timeline.py [config2|config2_ctx512|config2_ctx16|config3|config3_full] [knob=value ...]
 
 Runs the kernel library built with -DONELLM_ATTN_STAMPS (the product sources plus two clock stamps per workgroup and
 the XCC id register) on synthetic inputs of the named BASELINE shape and prints, per XCD and per dispatch half
@@ -21,6 +21,7 @@ from onellm_amd import capi  # noqa: E402
 SHAPES = {
     "config2": dict(B=16, Hq=32, Hkv=32, S=4096, t=4096, ragged=False, nsets=4),
     "config2_ctx512": dict(B=16, Hq=32, Hkv=32, S=4096, t=512, ragged=False, nsets=4),
+    "config2_ctx16": dict(B=16, Hq=32, Hkv=32, S=4096, t=16, ragged=False, nsets=4),       # launch and drain only
     "config3": dict(B=32, Hq=32, Hkv=8, S=8192, t=8192, ragged=True, nsets=3),
     "config3_full": dict(B=32, Hq=32, Hkv=8, S=8192, t=8192, ragged=False, nsets=3),
 }
@@ -35,6 +36,10 @@ def main():
     L = capi.lib()
     L.onellm_attn_set_stamp_buffer.argtypes = [ctypes.c_void_p]
     L.onellm_attn_set_stamp_buffer.restype = None
+    for kv in sys.argv[2:]:                      # internal tuning knobs, e.g. attn_balanced_wgs=512
+        key, value = kv.split("=")
+        capi.tune_set(key, int(value))
+        print("knob", key, "=", value)
     dev = torch.device("cuda:0")
     D = 128
     B, Hq, Hkv, S, t = c["B"], c["Hq"], c["Hkv"], c["S"], c["t"]
@@ -65,24 +70,29 @@ def main():
     ev1.record()
     torch.cuda.synchronize()
     print("%s: %.1f us per step (HIP events, 50 steps, stamps off)" % (name, ev0.elapsed_time(ev1) / 50 * 1e3))
-    ends, xcc = [], None
+    ends, xcc, cu, alone = [], None, None, []
     for rep in range(8):
         stamps.zero_()
         torch.cuda.synchronize()
         L.onellm_attn_set_stamp_buffer(stamps.data_ptr())
+        ev0.record()
         step(rep)
+        ev1.record()
         torch.cuda.synchronize()
+        alone.append(ev0.elapsed_time(ev1) * 1e3)
         L.onellm_attn_set_stamp_buffer(None)
         d = stamps.cpu().numpy().reshape(-1, 4)
         used = d[:, 0] != 0
         n = int(used.sum())
         st, en = d[:n, 0], d[:n, 1]
         xcc = d[:n, 2] & 0xF
+        cu = ((d[:n, 3] >> 8) & 0xFF) | (xcc << 8)      # (XCD, shader engine, array, unit)
         ends.append((en - st.min()) / 100.0)           # 100 MHz clock
         last_start = (st.max() - st.min()) / 100.0
     e = np.mean(ends, axis=0)
     n = len(e)
     idx = np.arange(n)
+    print("one launch at a time, between two events: %.1f us (median of %d)" % (float(np.median(alone)), len(alone)))
     print("workgroups %d; all started by %.1f us; end: mean %.1f, max %.1f, min %.1f us" % (n, last_start, e.mean(), e.max(), e.min()))
     half = n // 2 if n >= 512 else n
     for x in range(8):
@@ -92,6 +102,20 @@ def main():
             b = e[(xcc == x) & (idx >= half)]
             line += " | %d..%d end mean %.1f (min %.1f, max %.1f)" % (half, n - 1, b.mean(), b.min(), b.max())
         print(line)
+    by_compute_unit(ends[-1], cu)
+
+
+
+def by_compute_unit(e, cu):
+    """How the workgroups of the last launch were spread over the compute units, and when those of a unit with one, two,
+    three ... of them ended."""
+    units, counts = np.unique(cu, return_counts=True)
+    print("compute units used: %d; workgroups per unit: %s" % (len(units), dict(zip(*np.unique(counts, return_counts=True)))))
+    per_unit = dict(zip(units, counts))
+    share = np.array([per_unit[c] for c in cu])
+    for k in sorted(set(share)):
+        a = e[share == k]
+        print("  units with %d workgroup(s): %d workgroups end mean %.1f (min %.1f, max %.1f)" % (k, a.size, a.mean(), a.min(), a.max()))
 
 
 if __name__ == "__main__":
