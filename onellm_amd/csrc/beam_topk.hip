@@ -215,8 +215,8 @@ __device__ __forceinline__ float kth_group_maximum(float m)
 }
 
 // One wave's running top KP.  `top` holds the same values in every lane (it is only ever updated from values read
-// out of one lane, under control flow the whole wave takes); `lanes` is the per-lane list of the batch slots that
-// had too many survivors to read out one by one.
+// out of one lane, under control flow the whole wave takes); `lanes` is the per-lane list the wave goes over to, for
+// good, once a batch leaves too many survivors to rank (lists of eight use nothing else).
 template <int KP>
 struct WaveTop {
     static constexpr int kRankAtMost = 16;
