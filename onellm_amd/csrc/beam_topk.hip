@@ -271,10 +271,32 @@ struct WaveTop {
     template <int NV, int E>
     __device__ __forceinline__ void take(const float (&x)[NV], unsigned valid, int id0, int id_step)
     {
+        take_with<NV>(x, valid, [&](int j) { return id0 + (j / E) * id_step + j % E; });
+    }
+    // the same with the flat indices in an array (the survivors of an earlier stage carry theirs)
+    template <int NV>
+    __device__ __forceinline__ void take(const float (&x)[NV], unsigned valid, const int (&id)[NV])
+    {
+        take_with<NV>(x, valid, [&](int j) {
+            int pick[NV];
+#pragma unroll
+            for (int i = 0; i < NV; ++i) pick[i] = id[i];
+#pragma unroll
+            for (int bit = 0; (NV >> bit) > 1; ++bit) {
+                const bool odd = (j >> bit) & 1;
+#pragma unroll
+                for (int i = 0; i < (NV >> (bit + 1)); ++i) pick[i] = odd ? pick[2 * i + 1] : pick[2 * i];
+            }
+            return pick[0];
+        });
+    }
+    template <int NV, class IdOf>
+    __device__ __forceinline__ void take_with(const float (&x)[NV], unsigned valid, IdOf id_of)
+    {
         if (kPerLaneOnly) {
 #pragma unroll
             for (int j = 0; j < NV; ++j)
-                if ((valid >> j) & 1) lanes.insert(make_key(x[j], id0 + (j / E) * id_step + j % E));
+                if ((valid >> j) & 1) lanes.insert(make_key(x[j], id_of(j)));
             return;
         }
         unsigned marked = valid;
@@ -295,7 +317,7 @@ struct WaveTop {
         if (used_lanes) {
 #pragma unroll
             for (int j = 0; j < NV; ++j)
-                if ((marked >> j) & 1) lanes.insert(make_key(x[j], id0 + (j / E) * id_step + j % E));
+                if ((marked >> j) & 1) lanes.insert(make_key(x[j], id_of(j)));
             return;
         }
         while (__builtin_amdgcn_ballot_w64(marked != 0) != 0) {
@@ -310,7 +332,7 @@ struct WaveTop {
                 for (int i = 0; i < (NV >> (bit + 1)); ++i) pick[i] = odd ? pick[2 * i + 1] : pick[2 * i];
             }
             const float xv = pick[0];
-            const Key k = marked ? make_key(xv, id0 + (j / E) * id_step + j % E) : (Key)0;
+            const Key k = marked ? make_key(xv, id_of(j)) : (Key)0;
             marked &= marked - 1;
             offer(k);
         }
@@ -341,6 +363,57 @@ __device__ __forceinline__ void block_merge(TopList<KP>& t, Key* skey)
 #pragma unroll
             for (int i = 0; i < KP; ++i) o.k[i] = skey[w * KP + i];
             t.merge(o);
+        }
+    }
+}
+
+// One wave merges the n survivors (value, flat index; index -1 = empty slot) of a batch entry, four per lane and
+// batch, and its lane 0 stores the K best.  DEVICE_SCOPE: the survivors were stored by other workgroups of this
+// launch, so they are read with device-scope loads.
+template <int KP, bool DEVICE_SCOPE>
+__device__ __forceinline__ void merge_survivors(const float* __restrict__ logits, const float* vals, const int* ids, int n, int K,
+                                                float* __restrict__ fvals, int* __restrict__ fids)
+{
+    constexpr int NV = 4;
+    const int lane = threadIdx.x & (kWave - 1);
+    WaveTop<KP> w;
+    w.clear();
+    for (int base = 0; base < n; base += NV * kWave) {
+        float x[NV];
+        int id[NV];
+        unsigned valid = 0;
+        float lane_max = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int i = base + j * kWave + lane;
+            x[j] = -INFINITY;
+            id[j] = -1;
+            if (i < n) {
+                if (DEVICE_SCOPE) {
+                    id[j] = __hip_atomic_load(&ids[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    x[j] = __hip_atomic_load(&vals[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else {
+                    id[j] = ids[i];
+                    x[j] = vals[i];
+                }
+            }
+            if (id[j] != -1) {
+                valid |= 1u << j;
+                lane_max = fmaxf(lane_max, x[j]);
+            }
+        }
+        w.raise_floor(lane_max);
+        w.template take<NV>(x, valid, id);
+    }
+    w.finish();
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            if (i < K) {
+                const int id = key_id(w.top.k[i]);
+                fvals[i] = key_value(w.top.k[i], id, logits);
+                fids[i] = id;
+            }
         }
     }
 }
@@ -463,65 +536,19 @@ void topk_stage1_kernel(const float* __restrict__ logits, int V, int nblk, int v
     }
     __syncthreads();
     if (!s_last) return;
+    if (threadIdx.x >= kWave) return;
     const int n = pieces * K;
-    w.clear();
-    for (int i0 = 0; i0 < n; i0 += 256) {
-        const int i = i0 + threadIdx.x;
-        int id = -1;
-        float v = -INFINITY;
-        if (i < n) {
-            id = __hip_atomic_load(&ids[(size_t)b * n + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            v = __hip_atomic_load(&vals[(size_t)b * n + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        const float x[1] = {v};
-        w.raise_floor(id != -1 ? v : -INFINITY);
-        w.template take<1, 1>(x, id != -1 ? 1u : 0u, id, 0);
-    }
-    w.finish();
-    block_merge<KP>(t, skey);
-    if (threadIdx.x == 0) {
-#pragma unroll
-        for (int i = 0; i < KP; ++i) {
-            if (i < K) {
-                const int id = key_id(t.k[i]);
-                fvals[(size_t)b * K + i] = key_value(t.k[i], id, logits);
-                fids[(size_t)b * K + i] = id;
-            }
-        }
-    }
+    merge_survivors<KP, true>(logits, vals + (size_t)b * n, ids + (size_t)b * n, n, K, fvals + (size_t)b * K, fids + (size_t)b * K);
 }
 
-// grid = B; merges the n = beam*nblk*K stage-1 survivors of one batch entry
+// grid = B, one wave each; merges the n = beam*nblk*K stage-1 survivors of one batch entry
 template <int KP>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(kWave)
 void topk_stage2_kernel(const float* __restrict__ logits, const float* __restrict__ vals, const int* __restrict__ ids,
                         int n, int K, float* __restrict__ fvals, int* __restrict__ fids)
 {
-    __shared__ Key skey[4 * KP];
     const int b = blockIdx.x;
-    WaveTop<KP> w;
-    w.clear();
-    for (int i0 = 0; i0 < n; i0 += 256) {
-        const int i = i0 + threadIdx.x;
-        const int id = i < n ? ids[(size_t)b * n + i] : -1;
-        const float v = i < n ? vals[(size_t)b * n + i] : -INFINITY;
-        const float x[1] = {v};
-        w.raise_floor(id != -1 ? v : -INFINITY);
-        w.template take<1, 1>(x, id != -1 ? 1u : 0u, id, 0);
-    }
-    w.finish();
-    TopList<KP>& t = w.top;
-    block_merge<KP>(t, skey);
-    if (threadIdx.x == 0) {
-#pragma unroll
-        for (int i = 0; i < KP; ++i) {
-            if (i < K) {
-                const int id = key_id(t.k[i]);
-                fvals[(size_t)b * K + i] = key_value(t.k[i], id, logits);
-                fids[(size_t)b * K + i] = id;
-            }
-        }
-    }
+    merge_survivors<KP, false>(logits, vals + (size_t)b * n, ids + (size_t)b * n, n, K, fvals + (size_t)b * K, fids + (size_t)b * K);
 }
 
 template <int KP>
@@ -557,7 +584,7 @@ int launch_topk(const float* logits, int B, int beam, int V, int K, int nblk, fl
                        vals, ids, -1, beam, fvals, fids);
     int rc = launch_status();
     if (rc) return rc;
-    hipLaunchKernelGGL((topk_stage2_kernel<KP>), dim3(B), dim3(256), 0, st, logits, vals, ids, beam * nblk * K, K, fvals, fids);
+    hipLaunchKernelGGL((topk_stage2_kernel<KP>), dim3(B), dim3(kWave), 0, st, logits, vals, ids, beam * nblk * K, K, fvals, fids);
     g_last_launches = 2;
     return launch_status();
 }
