@@ -148,7 +148,9 @@ def test_topk_config5_planted_ties(capi, ref, dev, topk_form):
 
 
 @pytest.mark.parametrize("B,beam,V,K", [(1, 1, 1, 1), (2, 3, 100, 8), (3, 2, 257, 5), (1, 4, 2049, 3), (5, 1, 50000, 2),
-                                        (2, 2, 128256, 4), (1, 1, 3, 8)])
+                                        (2, 2, 128256, 4), (1, 1, 3, 8),
+                                        # more survivors per batch entry than one pass of the merging wave holds (256)
+                                        (2, 8, 1000, 8), (1, 16, 3000, 4), (1, 40, 500, 2)])
 def test_topk_shapes_with_heavy_ties(capi, ref, dev, B, beam, V, K, topk_form):
     announce("topk", B, beam, V, K, topk_form)
     rng = np.random.default_rng(V + K)
