@@ -176,52 +176,67 @@ __device__ __forceinline__ void merge_pieces(const AttnArgs& a, const Unit& u, i
     }
 }
 
-// The same for a unit with many pieces (a long sequence of a small batch is cut into up to 64): the (m, l)
-// pairs of all pieces go through LDS first - one round trip - where each head's maximum, its pieces' weights
-// and its sum are worked out once, a head per wave at a time; then only the partial sums are read, about 32
-// loads in flight per thread over all of its elements, instead of one element and sixteen pieces at a time
-// (eight round trips become two at 64 pieces and two elements per thread: the first batch of sums is
-// requested together with the pairs).  The order of every sum is
-// fixed, so the result does not depend on which piece arrived last.  `lds` holds (2 * npieces + 1) * GT floats.
-template <typename T, int D, int GT, int NTHR, int INFLIGHT>
-__device__ __forceinline__ void merge_pieces_wide(const AttnArgs& a, const Unit& u, int tid, float* lds)
+// The same for a unit with many pieces (a long sequence of a small batch is cut into up to 64).  Read one float at a
+// time, 32 pieces x 2 KiB take a workgroup 4.5-5 us however the loads are batched: 384 load instructions of 256
+// bytes from one compute unit, two thirds of them for (m, l) pairs every thread of a head reads again.  Here the
+// pairs go through LDS first - one round trip, one 8-byte load per (piece, head) - where each head's maximum, its
+// pieces' weights and its sum are worked out once, a head per wave at a time; and the partial sums are read 16
+// bytes at a time by the threads that own four consecutive output elements (the first batch is requested together
+// with the pairs).  The order of every sum is fixed, so the result does not depend on which piece arrived last.
+// `lds` holds (2 * npieces + 1) * GT floats.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t device_scope_window(const void* base)
 {
-    constexpr int E = (GT * D + NTHR - 1) / NTHR;             // elements per thread
-    constexpr int BATCH = INFLIGHT / E < 4 ? 4 : (INFLIGHT / E > 32 ? 32 : INFLIGHT / E);   // (more would cost the single-head kernel registers)
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7FFFFFFF, 0x00020000);
+}
+constexpr int kDeviceScopeLoad = 16;          // sc1
+__device__ __forceinline__ f32x4 fetch16(__amdgpu_buffer_rsrc_t w, unsigned byte_offset)
+{
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(w, byte_offset, 0, kDeviceScopeLoad));
+}
+
+template <typename T, int D, int GT, int NTHR>
+__device__ __forceinline__ void merge_pieces_vec(const AttnArgs& a, const Unit& u, int tid, float* lds)
+{
+    static_assert(D % 4 == 0, "four consecutive elements of a head per thread");
+    constexpr int NQ = GT * D / 4;                            // groups of four output elements
+    constexpr int E = (NQ + NTHR - 1) / NTHR;                 // groups per thread
+    constexpr int BATCH = E >= 4 ? 4 : (E == 2 ? 8 : 16);     // pieces in flight: 16 loads of 16 bytes per thread
     constexpr int NWAVE = NTHR / kWave;
     const int P = u.npieces;
     float* lw = lds;                                          // [P][GT]: m, then the weight 2^(m - max)
     float* ll = lds + P * GT;                                 // [P][GT]: l
     float* lL = ll + P * GT;                                  // [GT]: the head's sum
+    const __amdgpu_buffer_rsrc_t wo = device_scope_window(a.part_o + u.p0 * D);
+    const __amdgpu_buffer_rsrc_t wml = device_scope_window(a.part_ml + u.p0 * 2);
     bool valid[E];
     int hg[E];
-    const float* po[E];
-    float O[E];
+    unsigned off[E];                                          // byte offset of the group in piece 0's entry
+    f32x4 O[E];
 #pragma unroll
     for (int k = 0; k < E; ++k) {
-        const int i = tid + k * NTHR;
-        hg[k] = i / D;
-        valid[k] = i < GT * D && u.g0 + hg[k] < a.G;
-        if (!valid[k]) hg[k] = 0;                             // (a thread without an element reads the tile's first head and stores nothing:
-        po[k] = a.part_o + (u.p0 + (size_t)hg[k] * u.pstride) * D + i % D;   //  the loads below stay free of branches)
-        O[k] = 0.f;
+        const int q = tid + k * NTHR;
+        hg[k] = (4 * q) / D;
+        valid[k] = q < NQ && u.g0 + hg[k] < a.G;
+        if (!valid[k]) hg[k] = 0;                             // (reads the tile's first head and stores nothing: no branches around the loads)
+        off[k] = (unsigned)(((size_t)hg[k] * u.pstride * D + (valid[k] ? (4 * q) % D : 0)) * sizeof(float));
+        O[k] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    float oo[E][BATCH];
+    const unsigned piece_step = (unsigned)((size_t)u.sstride * D * sizeof(float));
+    f32x4 oo[E][BATCH];
     auto request = [&](int s0) {
 #pragma unroll
         for (int k = 0; k < E; ++k)
 #pragma unroll
-            for (int j = 0; j < BATCH; ++j)
-                oo[k][j] = fetch(po[k] + (size_t)min(s0 + j, P - 1) * u.sstride * D);
+            for (int j = 0; j < BATCH; ++j) oo[k][j] = fetch16(wo, off[k] + (unsigned)min(s0 + j, P - 1) * piece_step);
     };
-    // the first batch of partial sums travels together with the (m, l) pairs
     request(0);
     for (int p = tid; p < P * GT; p += NTHR) {
         const int sp = p / GT, g = p % GT;
         if (u.g0 + g < a.G) {
-            const size_t e = u.p0 + (size_t)g * u.pstride + (size_t)sp * u.sstride;
-            lw[p] = fetch(a.part_ml + e * 2);
-            ll[p] = fetch(a.part_ml + e * 2 + 1);
+            const unsigned e = (unsigned)(((size_t)g * u.pstride + (size_t)sp * u.sstride) * 2 * sizeof(float));
+            const auto ml = __builtin_amdgcn_raw_buffer_load_b64(wml, e, 0, kDeviceScopeLoad);
+            lw[p] = __uint_as_float(ml[0]);
+            ll[p] = __uint_as_float(ml[1]);
         }
     }
     __syncthreads();
@@ -232,7 +247,7 @@ __device__ __forceinline__ void merge_pieces_wide(const AttnArgs& a, const Unit&
             float M = -INFINITY;
             for (int sp = lane; sp < P; sp += kWave) M = fmaxf(M, lw[sp * GT + g]);
 #pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, kWave));
+            for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, kWave));
             float L = 0.f;
             for (int sp = lane; sp < P; sp += kWave) {
                 const float wgt = __builtin_amdgcn_exp2f(lw[sp * GT + g] - M);   // every piece has a finite maximum
@@ -250,16 +265,20 @@ __device__ __forceinline__ void merge_pieces_wide(const AttnArgs& a, const Unit&
         for (int k = 0; k < E; ++k)
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
-                const float wgt = lw[min(s0 + j, P - 1) * GT + hg[k]];
-                O[k] = fmaf(oo[k][j], s0 + j < P ? wgt : 0.f, O[k]);
+                const float wgt = s0 + j < P ? lw[min(s0 + j, P - 1) * GT + hg[k]] : 0.f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) O[k][c] = fmaf(oo[k][j][c], wgt, O[k][c]);
             }
     }
 #pragma unroll
     for (int k = 0; k < E; ++k)
         if (valid[k]) {
-            const int i = tid + k * NTHR;
+            const int q = tid + k * NTHR;
             const int h = u.kvh * a.G + u.g0 + hg[k];
-            static_cast<T*>(a.out)[((size_t)u.b * a.Hq + h) * D + i % D] = from_f32<T>(O[k] / lL[hg[k]]);
+            const float L = lL[hg[k]];
+            T* out = static_cast<T*>(a.out) + ((size_t)u.b * a.Hq + h) * D + (4 * q) % D;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) out[c] = from_f32<T>(O[k][c] / L);
         }
 }
 
@@ -434,11 +453,8 @@ __device__ __forceinline__ void finish_unit(const AttnArgs& a, const Unit& u, fl
     if (u.npieces <= 2) merge_pieces<T, D, GT, NTHR, 2>(a, u, tid);
     else if (u.npieces <= 4) merge_pieces<T, D, GT, NTHR, 4>(a, u, tid);
     else if (u.npieces <= 8) merge_pieces<T, D, GT, NTHR, 8>(a, u, tid);
-    // (where a thread has 128 partial sums or more to read - measured: 32 q / 8 kv heads, batch 1, 8192 rows, 64 pieces x 2
-    // elements 16.9 -> 16.5 us; 64 q heads, 32768 rows, 32 x 4: 35.4 -> 32.3; batch 2, 32 x 2: 20.0 -> 21.1, hence
-    // not there.  st_acc: NST * GT * D floats, free by now)
-    else if (u.npieces * ((GT * D + NTHR - 1) / NTHR) >= 128 && 2 * u.npieces + 1 <= NST * D)
-        merge_pieces_wide<T, D, GT, NTHR, 32>(a, u, tid, st_acc);
+    // (more than eight: 16-byte loads and the pairs through LDS - st_acc: NST * GT * D floats, free by now)
+    else if (2 * u.npieces + 1 <= NST * D) merge_pieces_vec<T, D, GT, NTHR>(a, u, tid, st_acc);
     else merge_pieces<T, D, GT, NTHR, 16>(a, u, tid);
 }
 
