@@ -26,8 +26,8 @@ HBM_PEAK_GBPS = 8000.0   # MI355X, published
 # each scaled by the same counter's reading for a 1 GiB device copy: x1.99994 and x1.0000), keyed by context, and
 # the digest of the attention sources the counted kernel was built from: when the sources change the figure is
 # withheld (traffic: null) until the counter runs are repeated and both are updated together.
-MEASURED_TRAFFIC_BYTES = {4096: 1074420933}
-MEASURED_TRAFFIC_SOURCES = "7b41be1ff66290dd"
+MEASURED_TRAFFIC_BYTES = {4096: 1074438341}
+MEASURED_TRAFFIC_SOURCES = "449cb23c0c63426a"
 ATTENTION_SOURCES = ["decode_attn.hip", "attn_schedule.hpp", "attn_finish.hpp", "attn_valu.hpp", "attn_mfma.hpp", "common.hpp", "rope.hpp"]
 
 
