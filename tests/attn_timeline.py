@@ -116,6 +116,11 @@ def by_compute_unit(e, cu):
     for k in sorted(set(share)):
         a = e[share == k]
         print("  units with %d workgroup(s): %d workgroups end mean %.1f (min %.1f, max %.1f)" % (k, a.size, a.mean(), a.min(), a.max()))
+    # when a compute unit is done with all it was given: the step ends with the last of them
+    last = np.array([e[cu == c].max() for c in units])
+    first = np.array([e[cu == c].min() for c in units])
+    print("  a compute unit's last workgroup ends: mean %.1f, min %.1f, max %.1f, 10th / 90th percentile %.1f / %.1f; its first: mean %.1f"
+          % (last.mean(), last.min(), last.max(), np.percentile(last, 10), np.percentile(last, 90), first.mean()))
 
 
 if __name__ == "__main__":
