@@ -392,10 +392,12 @@ def ceilings_section(dev, steps, warmup):
     best("fill_512MiB", 512 * MiB, lambda pol: (lambda i: ac.fill(big[i % 3], 1.0, pol)))
     half = [b[:256 * MiB] for b in big] + [b[256 * MiB:] for b in big]
     best("copy_256MiB", 2 * 256 * MiB, lambda pol: (lambda i: ac.copy(half[(i + 3) % 6], half[i % 6], pol)))
-    # one read fanned out to four stores: 64 MiB in, 4 x 64 MiB out, as the KV repeat with four query heads per kv head
-    fan_src = [b[:64 * MiB] for b in big]
-    fan_dst = [b[128 * MiB:384 * MiB].view(4, 64 * MiB) for b in big]
-    best("one_read_four_stores_64MiB", 5 * 64 * MiB, lambda pol: (lambda i: ac.fanout(fan_dst[i % 3], fan_src[i % 3], 4, pol)))
+    # one read fanned out to four stores, as the KV repeat with four query heads per kv head lays them out: the source a
+    # row of 2 MiB chunks (one kv head's 8192 x 128 fp16 rows), the four copies of a chunk side by side
+    fan_src = [b[:100 * MiB] for b in big]
+    fan_dst = [b[100 * MiB:500 * MiB] for b in big]
+    best("one_read_four_stores_2MiB_chunks", 5 * 100 * MiB,
+         lambda pol: (lambda i: ac.fanout(fan_dst[i % 3], fan_src[i % 3], 4, pol, chunk=2 * MiB)))
     # rows read, reduced and written back in place (+ a row-sized vector every workgroup reads): the norm kernels' mix
     for row_bytes in (8192, 16384):
         per = 8192 * row_bytes
@@ -423,7 +425,7 @@ CEILING_OF = {
     "decode_attn_gqa_fused_b16_q64_kv8_len8192": "read_stream_512MiB",
     "decode_attn_gqa_fused_fp32_b8_q64_kv8_len8192": "read_stream_512MiB",
     "decode_attn_fp32_b8_h32_ctx4096": "read_stream_512MiB",
-    "kv_repeat_b32_q32_kv8_len1024-8192": "one_read_four_stores_64MiB",
+    "kv_repeat_b32_q32_kv8_len1024-8192": "one_read_four_stores_2MiB_chunks",
     "rmsnorm_8192x4096": "rows_in_place_8192x8192B", "fused_norm_8192x4096": "row_pairs_in_place_8192x8192B",
     "rmsnorm_8192x8192": "rows_in_place_8192x16384B", "fused_norm_8192x8192": "row_pairs_in_place_8192x16384B",
     "prefill_qkv_bias_rope_4x2048_tokens_32x128": "copy_256MiB", "swiglu_8192x11008": "copy_256MiB",

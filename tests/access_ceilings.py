@@ -14,7 +14,7 @@ SYMBOLS = {
     "ceiling_fill": (_ci, [_vp, _sz, _cf, _ci, _vp]),
     "ceiling_copy": (_ci, [_vp, _vp, _sz, _ci, _vp]),
     "ceiling_rows": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
-    "ceiling_fanout": (_ci, [_vp, _vp, _sz, _ci, _sz, _ci, _vp]),
+    "ceiling_fanout": (_ci, [_vp, _vp, _sz, _ci, _sz, _sz, _ci, _vp]),
 }
 _lib = None
 
@@ -68,8 +68,9 @@ def rows(a, b, shared, policy):
                            shared.data_ptr() if shared is not None else None, n, row_bytes, policy, _stream()), "ceiling_rows")
 
 
-def fanout(dst, src, G, policy):
-    """dst [G, ...src.shape] <- src repeated G times."""
+def fanout(dst, src, G, policy, chunk=0):
+    """dst [G, ...src.shape] <- src repeated G times; with chunk (bytes) the source is a row of chunks and dst holds the
+    G copies of each chunk side by side ([chunks, G, chunk])."""
     nbytes = src.numel() * src.element_size()
     assert dst.numel() * dst.element_size() == G * nbytes
-    _ok(lib().ceiling_fanout(dst.data_ptr(), src.data_ptr(), nbytes, G, nbytes, policy, _stream()), "ceiling_fanout")
+    _ok(lib().ceiling_fanout(dst.data_ptr(), src.data_ptr(), nbytes, G, nbytes, chunk, policy, _stream()), "ceiling_fanout")

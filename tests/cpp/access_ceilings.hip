@@ -112,13 +112,20 @@ __global__ __launch_bounds__(512) void rows_kernel(char* __restrict__ a, char* _
     }
 }
 
+// chunk == 0: copy g of the whole source starts at dst + g * dst_stride.  chunk > 0: the source is a row of chunks and
+// the G copies of a chunk follow each other (chunk c, copy g at (c * G + g) * chunk) - how the KV repeat lays out the
+// query heads of one kv head.
 template <int LA, int SA>
-__global__ __launch_bounds__(256) void fanout_kernel(char* __restrict__ dst, const char* __restrict__ src, int G, size_t dst_stride)
+__global__ __launch_bounds__(256) void fanout_kernel(char* __restrict__ dst, const char* __restrict__ src, int G, size_t dst_stride,
+                                                     size_t chunk)
 {
-    const __amdgpu_buffer_rsrc_t ds = descriptor(src + (size_t)blockIdx.x * 4096, 4096);
+    const size_t off = (size_t)blockIdx.x * 4096;
+    const __amdgpu_buffer_rsrc_t ds = descriptor(src + off, 4096);
     const f32x4 v = load16<LA>(ds, threadIdx.x * 16);
+    const size_t base = chunk ? (off / chunk) * chunk * G + off % chunk : off;
+    const size_t step = chunk ? chunk : dst_stride;
     for (int g = 0; g < G; ++g) {
-        const __amdgpu_buffer_rsrc_t dd = descriptor(dst + (size_t)g * dst_stride + (size_t)blockIdx.x * 4096, 4096);
+        const __amdgpu_buffer_rsrc_t dd = descriptor(dst + (size_t)g * step + base, 4096);
         store16<SA>(dd, threadIdx.x * 16, v);
     }
 }
@@ -215,14 +222,16 @@ int ceiling_rows(void* a, void* b, const void* shared, int rows, int row_bytes, 
     return status();
 }
 
-// src_bytes of src copied to G destinations dst, dst + dst_stride, ...
-int ceiling_fanout(void* dst, const void* src, size_t src_bytes, int G, size_t dst_stride, int policy, void* stream)
+// src_bytes of src copied to G destinations dst, dst + dst_stride, ... (chunk == 0), or chunk by chunk with the G
+// copies of a chunk side by side (chunk > 0, a multiple of 4 KiB that divides src_bytes; dst_stride is not used)
+int ceiling_fanout(void* dst, const void* src, size_t src_bytes, int G, size_t dst_stride, size_t chunk, int policy, void* stream)
 {
-    if (!dst || !src || src_bytes == 0 || src_bytes % 4096 || G < 1 || dst_stride < src_bytes) return -1;
+    if (!dst || !src || src_bytes == 0 || src_bytes % 4096 || G < 1) return -1;
+    if (chunk ? (chunk % 4096 || src_bytes % chunk) : dst_stride < src_bytes) return -1;
     const dim3 grid((unsigned)(src_bytes / 4096));
     hipStream_t st = (hipStream_t)stream;
     switch (policy) {
-#define X(i, la, sa) case i: hipLaunchKernelGGL((fanout_kernel<la, sa>), grid, dim3(256), 0, st, (char*)dst, (const char*)src, G, dst_stride); break;
+#define X(i, la, sa) case i: hipLaunchKernelGGL((fanout_kernel<la, sa>), grid, dim3(256), 0, st, (char*)dst, (const char*)src, G, dst_stride, chunk); break;
         CEILING_POLICIES(X)
 #undef X
         default: return -1;

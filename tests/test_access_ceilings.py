@@ -26,6 +26,9 @@ def test_each_pattern_moves_its_bytes(dev, policy):
     fan = torch.zeros(4, src.numel(), device=dev)
     ac.fanout(fan, src, 4, policy)
     assert all(torch.equal(fan[i], src) for i in range(4))
+    chunks = torch.zeros(16, 4, src.numel() // 16, device=dev)          # 16 chunks of 256 KiB, four copies side by side
+    ac.fanout(chunks, src, 4, policy, chunk=src.numel() * 4 // 16)
+    assert all(torch.equal(chunks[:, i].reshape(-1), src) for i in range(4))
     for row_elems in (2048, 4096, 8192):                                # 8, 16, 32 KiB rows of fp32
         a = torch.randn(64, row_elems, device=dev, generator=g)
         b = torch.randn(64, row_elems, device=dev, generator=g)
