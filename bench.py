@@ -398,6 +398,10 @@ def ceilings_section(dev, steps, warmup):
     fan_dst = [b[100 * MiB:500 * MiB] for b in big]
     best("one_read_four_stores_2MiB_chunks", 5 * 100 * MiB,
          lambda pol: (lambda i: ac.fanout(fan_dst[i % 3], fan_src[i % 3], 4, pol, chunk=2 * MiB)))
+    # the prefill QKV kernel's transposing copy: 8192 tokens x 96 heads x 256-byte rows, token-major to head-major
+    tm = [b[:8192 * 96 * 256].view(8192, 96, 256) for b in big]
+    hm = [b[256 * MiB:256 * MiB + 8192 * 96 * 256].view(4, 96, 2048, 256) for b in big]
+    best("regroup_8192_tokens_x_96_rows_of_256B", 2 * 8192 * 96 * 256, lambda pol: (lambda i: ac.regroup(hm[i % 3], tm[i % 3], 2048, pol)))
     # rows read, reduced and written back in place (+ a row-sized vector every workgroup reads): the norm kernels' mix
     for row_bytes in (8192, 16384):
         per = 8192 * row_bytes
@@ -411,7 +415,7 @@ def ceilings_section(dev, steps, warmup):
              lambda pol: (lambda i: ac.rows(views[i % n], None, shared, pol)))
         best("row_pairs_in_place_8192x%dB" % row_bytes, 4 * per + 2 * row_bytes,
              lambda pol: (lambda i: ac.rows(views[(2 * i) % n], views[(2 * i + 1) % n], shared, pol)))
-    del big, half, fan_src, fan_dst, views
+    del big, half, fan_src, fan_dst, views, tm, hm
     torch.cuda.empty_cache()
     return out
 
@@ -428,7 +432,7 @@ CEILING_OF = {
     "kv_repeat_b32_q32_kv8_len1024-8192": "one_read_four_stores_2MiB_chunks",
     "rmsnorm_8192x4096": "rows_in_place_8192x8192B", "fused_norm_8192x4096": "row_pairs_in_place_8192x8192B",
     "rmsnorm_8192x8192": "rows_in_place_8192x16384B", "fused_norm_8192x8192": "row_pairs_in_place_8192x16384B",
-    "prefill_qkv_bias_rope_4x2048_tokens_32x128": "copy_256MiB", "swiglu_8192x11008": "copy_256MiB",
+    "prefill_qkv_bias_rope_4x2048_tokens_32x128": "regroup_8192_tokens_x_96_rows_of_256B", "swiglu_8192x11008": "copy_256MiB",
 }
 
 

@@ -1,5 +1,5 @@
 """ctypes binding of tests/cpp/libaccess_ceilings.so: bare access-pattern kernels (pure read, fill, copy, in-place
-row read-reduce-write, one-read-G-stores) whose measured rate is the ceiling of the product kernel with the same
+row read-reduce-write, one-read-G-stores, token-major to head-major regrouping) whose measured rate is the ceiling of the product kernel with the same
 access mix on the GPU at hand.  Test-side only: bench.py times them beside the product kernels, a GPU test checks
 that each moves the bytes it claims to."""
 import ctypes
@@ -15,6 +15,7 @@ SYMBOLS = {
     "ceiling_copy": (_ci, [_vp, _vp, _sz, _ci, _vp]),
     "ceiling_rows": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "ceiling_fanout": (_ci, [_vp, _vp, _sz, _ci, _sz, _sz, _ci, _vp]),
+    "ceiling_regroup": (_ci, [_vp, _vp, _ci, _ci, _ci, _ci, _vp]),
 }
 _lib = None
 
@@ -74,3 +75,10 @@ def fanout(dst, src, G, policy, chunk=0):
     nbytes = src.numel() * src.element_size()
     assert dst.numel() * dst.element_size() == G * nbytes
     _ok(lib().ceiling_fanout(dst.data_ptr(), src.data_ptr(), nbytes, G, nbytes, chunk, policy, _stream()), "ceiling_fanout")
+
+
+def regroup(dst, src, seq_tokens, policy):
+    """src [tokens, heads, 256 bytes] -> dst [tokens // seq_tokens, heads, seq_tokens, 256 bytes]."""
+    tokens, heads = src.shape[0], src.shape[1]
+    assert src[0, 0].numel() * src.element_size() == 256 and dst.numel() == src.numel()
+    _ok(lib().ceiling_regroup(dst.data_ptr(), src.data_ptr(), tokens, heads, seq_tokens, policy, _stream()), "ceiling_regroup")

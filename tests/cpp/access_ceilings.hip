@@ -14,6 +14,9 @@
 //             the shape of RMSNorm (1 buffer) and of the fused add-residual norm (2 buffers); optionally every
 //             workgroup also reads a row-sized vector shared by all rows (gamma)
 //   fanout  : one stream in, G streams out (the KV repeat)
+//   regroup : rows of 256 bytes stored token-major [tokens][heads] copied to head-major [sequences][heads][tokens of
+//             the sequence] - the transposing copy of the prefill QKV kernel, eight tokens per workgroup, a head's
+//             eight rows leaving as one 2 KiB store
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
@@ -130,6 +133,29 @@ __global__ __launch_bounds__(256) void fanout_kernel(char* __restrict__ dst, con
     }
 }
 
+// 256 threads: 16-byte piece tid % 16 of the row, token (tid / 16) % 8 of the workgroup's eight, heads tid / 128 + 2 k;
+// eight heads in flight per thread, as in the product kernel
+template <int LA, int SA>
+__global__ __launch_bounds__(256) void regroup_kernel(char* __restrict__ dst, const char* __restrict__ src, unsigned bytes,
+                                                      int heads, int seq_tokens)
+{
+    const __amdgpu_buffer_rsrc_t ds = descriptor(src, bytes), dd = descriptor(dst, bytes);
+    const unsigned piece = threadIdx.x & 15, tl = (threadIdx.x >> 4) & 7, h0 = threadIdx.x >> 7;
+    const unsigned tok = blockIdx.x * 8 + tl;
+    const unsigned b = tok / seq_tokens, sq = tok % seq_tokens;
+    const unsigned in = tok * heads * 256u + piece * 16u;
+    const unsigned out = (b * heads * seq_tokens + sq) * 256u + piece * 16u, head_step = (unsigned)seq_tokens * 256u;
+    for (unsigned hb = h0; hb < (unsigned)heads; hb += 16) {
+        f32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (hb + 2 * u < (unsigned)heads) v[u] = load16<LA>(ds, in + (hb + 2 * u) * 256u);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (hb + 2 * u < (unsigned)heads) store16<SA>(dd, out + (hb + 2 * u) * head_step, v[u]);
+    }
+}
+
 inline int status() { return (int)hipGetLastError(); }
 
 // policy pairs the library is built for: index -> (load aux, store aux)
@@ -232,6 +258,24 @@ int ceiling_fanout(void* dst, const void* src, size_t src_bytes, int G, size_t d
     hipStream_t st = (hipStream_t)stream;
     switch (policy) {
 #define X(i, la, sa) case i: hipLaunchKernelGGL((fanout_kernel<la, sa>), grid, dim3(256), 0, st, (char*)dst, (const char*)src, G, dst_stride, chunk); break;
+        CEILING_POLICIES(X)
+#undef X
+        default: return -1;
+    }
+    return status();
+}
+
+// tokens * heads rows of 256 bytes, token-major in src, head-major per sequence of seq_tokens tokens in dst
+// (tokens a multiple of 8 and of seq_tokens; the whole buffer below 4 GiB)
+int ceiling_regroup(void* dst, const void* src, int tokens, int heads, int seq_tokens, int policy, void* stream)
+{
+    if (!dst || !src || tokens <= 0 || heads <= 0 || seq_tokens <= 0 || tokens % 8 || tokens % seq_tokens) return -1;
+    const size_t bytes = (size_t)tokens * heads * 256;
+    if (bytes >= (1ull << 32)) return -1;
+    const dim3 grid((unsigned)(tokens / 8));
+    hipStream_t st = (hipStream_t)stream;
+    switch (policy) {
+#define X(i, la, sa) case i: hipLaunchKernelGGL((regroup_kernel<la, sa>), grid, dim3(256), 0, st, (char*)dst, (const char*)src, (unsigned)bytes, heads, seq_tokens); break;
         CEILING_POLICIES(X)
 #undef X
         default: return -1;

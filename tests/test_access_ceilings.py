@@ -29,6 +29,10 @@ def test_each_pattern_moves_its_bytes(dev, policy):
     chunks = torch.zeros(16, 4, src.numel() // 16, device=dev)          # 16 chunks of 256 KiB, four copies side by side
     ac.fanout(chunks, src, 4, policy, chunk=src.numel() * 4 // 16)
     assert all(torch.equal(chunks[:, i].reshape(-1), src) for i in range(4))
+    tm = torch.randn(64, 6, 64, device=dev, generator=g)                # 64 tokens x 6 heads x 256 bytes, sequences of 16
+    hm = torch.zeros(4, 6, 16, 64, device=dev)
+    ac.regroup(hm, tm, 16, policy)
+    assert torch.equal(hm, tm.view(4, 16, 6, 64).permute(0, 2, 1, 3).contiguous())
     for row_elems in (2048, 4096, 8192):                                # 8, 16, 32 KiB rows of fp32
         a = torch.randn(64, row_elems, device=dev, generator=g)
         b = torch.randn(64, row_elems, device=dev, generator=g)
