@@ -3,9 +3,12 @@
  * Replaces launchLinearGemm (src/kernels/qkv_linear.cu:8-66, declared src/kernels/qkv_linear.h:9-14) and the
  * cublasWrapper::Gemm call under it (src/kernels/cublas_wrapper.cc:33-85).  The multiplication itself is a library
  * GEMM (hipBLASLt, fp32 accumulation); this entry point adds what the reference re-creates on every call: a handle
- * per device and a cached plan per (dtype, M, K, N, layout).  Small shapes the library has no kernel for (unit-test
- * and example-driver sizes, up to 2^24 multiply-adds) run a plain kernel in this library; a larger one returns
- * ONELLM_ENOGEMMKERNEL unless the caller has allowed the plain kernel, which is about a hundred times slower.
+ * per device and a cached plan per (dtype, M, K, N, layout).  For the few rows of a decode step (fp16, W as [K, N],
+ * M <= 32, K a multiple of 64, N of 8) the library also holds a kernel of its own that streams the weights once
+ * through the matrix cores; onellm_linear_tune times it beside the library's algorithms and onellm_linear runs
+ * whichever won.  Small shapes the library has no kernel for (unit-test and example-driver sizes, up to 2^24
+ * multiply-adds) run a plain kernel in this library; a larger one returns ONELLM_ENOGEMMKERNEL unless the caller has
+ * allowed the plain kernel, which is about a hundred times slower.
  *
  * Kept out of libonellm_hip.so so that the decode-path kernels do not pull in the BLAS library.
  */
@@ -29,18 +32,21 @@ extern "C" {
 int onellm_linear(int dtype, const void* x, const void* w, void* y, int M, int K, int N, int ldy, int w_is_nk,
                   void* workspace, size_t workspace_bytes, onellm_stream_t stream);
 
-/* Optional, once per shape (for example when a model is loaded): times the library's candidate algorithms for this
- * problem on stand-in operands it allocates and frees itself, and makes onellm_linear use the fastest one for this
- * (dtype, M, K, N, ldy, w_is_nk, workspace or not) from then on instead of the library's first suggestion.
- * Synchronises the stream.  best_us / first_us (either may be NULL) receive the time of the chosen algorithm and of
- * the library's first suggestion.  ONELLM_EUNSUPPORTED if the library has no algorithm for the problem. */
+/* Optional, once per shape (for example when a model is loaded): times the library's candidate algorithms and, where
+ * it applies, the configurations of this library's few-row kernel for this problem on stand-in operands it allocates
+ * and frees itself, and makes onellm_linear use the fastest for this (dtype, M, K, N, ldy, w_is_nk, workspace or not)
+ * from then on instead of the library's first suggestion.  The timing runs rotate over enough copies of W (640 MB, at
+ * most 16) that every run meets its matrix cold, as a projection inside a model does.  Synchronises the stream.
+ * best_us / first_us (either may be NULL) receive the time of the chosen algorithm and of the library's first
+ * suggestion.  ONELLM_EUNSUPPORTED if nothing takes the problem. */
 int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
                        onellm_stream_t stream, float* best_us, float* first_us);
 
 /* workspace size onellm_linear can make use of (a constant; any smaller size is valid too) */
 size_t onellm_linear_workspace_bytes(void);
 
-/* 1 if the last onellm_linear call on this thread ran the library GEMM, 0 if it ran the plain fallback kernel */
+/* what the last onellm_linear call on this thread ran: 1 the library GEMM, 2 this library's few-row kernel, 0 the
+ * plain fallback kernel */
 int onellm_linear_last_path(void);
 
 /* allow != 0: problems of any size may run the plain kernel when the library declines them (process-wide; off by

@@ -40,7 +40,7 @@ DRIVER_BIN = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver")
 KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip", "sampling.hip",
                   "tuning.cpp"]
 LAUNCHER_SOURCES = ["launchers.cpp"]
-GEMM_SOURCES = ["linear.hip"]
+GEMM_SOURCES = ["linear.hip", "skinny_gemm.hip"]
 LAYER_SOURCES = ["layers.cpp", "layers_capi.cpp"]
 
 # packed fp32 VALU forms are switched off on purpose (code generation only; scalar fp32 code is

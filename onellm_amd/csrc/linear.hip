@@ -1,5 +1,7 @@
 // y = x . W for the projections around the decode path: hipBLASLt with a per-device handle and cached
-// plans, plus a plain kernel for shapes the library declines.
+// plans, this library's own kernel for a decode step's few rows where timing finds it faster (skinny_gemm.hip),
+// plus a plain kernel for shapes the library declines.
+#include <algorithm>
 #include <atomic>
 #include <map>
 #include <mutex>
@@ -8,6 +10,7 @@
 #include <hip/hip_fp16.h>
 #include <hipblaslt/hipblaslt.h>
 #include "onellm_gemm.h"
+#include "skinny_gemm.hpp"
 
 namespace onellm {
 int tune_get(const char* key);     // libonellm_hip.so's tuning table
@@ -48,7 +51,8 @@ void linear_plain_kernel(const T* __restrict__ x, const T* __restrict__ w, T* __
 }
 
 struct Plan {
-    bool usable = false;
+    bool usable = false;                     // the library's objects below are there
+    SkinnyConfig skinny;                     // set by the tuning run when this library's few-row kernel won
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
     hipblasLtMatmulHeuristicResult_t heur{};
@@ -178,7 +182,11 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
     constexpr int kWant = 32;
     hipblasLtMatmulHeuristicResult_t cand[kWant];
     const int n = candidates(handle, p, workspace_bytes, cand, kWant);
-    if (n == 0) {
+    constexpr int kWantOwn = 64;
+    SkinnyConfig own[kWantOwn];
+    const int n_own = (tune_get("gemm_skinny") != 0 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk))
+                          ? skinny_candidates(M, K, N, workspace_bytes, own, kWantOwn) : 0;
+    if (n == 0 && n_own == 0) {
         destroy_plan(p);
         return ONELLM_EUNSUPPORTED;
     }
@@ -192,36 +200,52 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
 
     // stand-in operands of the right size (values do not matter for the timing; 0x3c3c.. is ~1.06 in fp16 and a
     // small normal number in fp32)
+    // The weights of a model are far larger than the chip's caches, so a projection always meets its matrix cold.  A
+    // timing loop over one matrix would not: it stays in the 256 MB memory-side cache and every candidate looks up to
+    // twice as fast as it will be (a 7B down projection, 90 MB: 29 us warm, 50 us cold with the same algorithm).  The
+    // runs therefore rotate over enough copies of W to exceed that cache.
     const size_t esz = dtype == ONELLM_FP16 ? 2 : 4;
-    void *x = nullptr, *w = nullptr, *y = nullptr;
+    const size_t w_bytes = (size_t)K * N * esz;
+    constexpr size_t kColdBytes = 640u << 20;
+    constexpr int kMaxCopies = 16;
+    const int copies = (int)std::min<size_t>(kMaxCopies, std::max<size_t>(2, (kColdBytes + w_bytes - 1) / w_bytes));
+    void *x = nullptr, *y = nullptr, *w[kMaxCopies] = {};
     hipEvent_t t0 = nullptr, t1 = nullptr;
     int rc = 0;
     auto cleanup = [&] {
         if (x) (void)hipFree(x);
-        if (w) (void)hipFree(w);
+        for (void* c : w)
+            if (c) (void)hipFree(c);
         if (y) (void)hipFree(y);
         if (t0) (void)hipEventDestroy(t0);
         if (t1) (void)hipEventDestroy(t1);
     };
-    if ((e = hipMalloc(&x, (size_t)M * K * esz)) != hipSuccess || (e = hipMalloc(&w, (size_t)K * N * esz)) != hipSuccess ||
-        (e = hipMalloc(&y, (size_t)M * ldy * esz)) != hipSuccess || (e = hipEventCreate(&t0)) != hipSuccess ||
+    e = hipMalloc(&x, (size_t)M * K * esz);
+    for (int c = 0; c < copies && e == hipSuccess; ++c) e = hipMalloc(&w[c], w_bytes);
+    if (e != hipSuccess || (e = hipMalloc(&y, (size_t)M * ldy * esz)) != hipSuccess || (e = hipEventCreate(&t0)) != hipSuccess ||
         (e = hipEventCreate(&t1)) != hipSuccess) {
         cleanup();
         destroy_plan(p);
         return (int)e;
     }
     (void)hipMemsetAsync(x, 0x3c, (size_t)M * K * esz, st);
-    (void)hipMemsetAsync(w, 0x3c, (size_t)K * N * esz, st);
+    for (int c = 0; c < copies; ++c) (void)hipMemsetAsync(w[c], 0x3c, w_bytes, st);
     const float alpha = 1.f, beta = 0.f;
-    int best = -1;
-    float best_ms = 0.f, first_ms = 0.f;
-    constexpr int kWarm = 2, kRuns = 8;
-    for (int i = 0; i < n; ++i) {
+    int best = -1, best_own = -1;
+    float best_ms = 0.f, first_ms = 0.f, best_own_ms = 0.f;
+    constexpr int kWarm = 2;
+    const int runs = std::max(8, copies);
+    // candidate i of the library (i < n) or of this library's kernel (i >= n), timed over `runs` launches
+    for (int i = 0; i < n + n_own; ++i) {
         bool ok = true;
-        for (int r = 0; r < kWarm + kRuns && ok; ++r) {
+        for (int r = 0; r < kWarm + runs && ok; ++r) {
             if (r == kWarm) (void)hipEventRecord(t0, st);
-            ok = hipblasLtMatmul(handle, p.desc, &alpha, w, p.la, x, p.lb, &beta, y, p.lc, y, p.lc, &cand[i].algo, workspace,
-                                 workspace_bytes, st) == HIPBLAS_STATUS_SUCCESS;
+            const void* wc = w[r % copies];
+            if (i < n)
+                ok = hipblasLtMatmul(handle, p.desc, &alpha, wc, p.la, x, p.lb, &beta, y, p.lc, y, p.lc, &cand[i].algo, workspace,
+                                     workspace_bytes, st) == HIPBLAS_STATUS_SUCCESS;
+            else
+                ok = skinny_launch(own[i - n], x, wc, y, M, K, N, ldy, workspace, workspace_bytes, st) == 0;
         }
         (void)hipEventRecord(t1, st);
         if ((e = hipEventSynchronize(t1)) != hipSuccess) {
@@ -231,19 +255,30 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
         if (!ok) continue;
         float ms = 0.f;
         (void)hipEventElapsedTime(&ms, t0, t1);
-        ms /= kRuns;
+        ms /= runs;
         if (i == 0) first_ms = ms;
-        if (best < 0 || ms < best_ms) {
-            best = i;
-            best_ms = ms;
+        if (i < n) {
+            if (best < 0 || ms < best_ms) {
+                best = i;
+                best_ms = ms;
+            }
+        } else if (best_own < 0 || ms < best_own_ms) {
+            best_own = i - n;
+            best_own_ms = ms;
         }
     }
     cleanup();
-    if (rc != 0 || best < 0) {
+    if (rc != 0 || (best < 0 && best_own < 0)) {
         destroy_plan(p);
         return rc != 0 ? rc : ONELLM_EUNSUPPORTED;
     }
-    p.heur = cand[best];
+    if (best >= 0) p.heur = cand[best];
+    else destroy_plan(p);                    // (the library has nothing for this problem: the plan is this library's kernel alone)
+    // this library's kernel is taken when it is clearly ahead (3 %: two near-equal timings should not flip a plan)
+    if (best_own >= 0 && (best < 0 || best_own_ms < 0.97f * best_ms)) {
+        p.skinny = own[best_own];
+        best_ms = best_own_ms;
+    }
     {
         // (a plan in the table is only ever used under this lock or as a copy taken under it by a call that was
         // queued before this one returns: the stream was synchronised above, so the old objects are idle)
@@ -299,6 +334,26 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
         }
     }
     if (tune_get("gemm_no_library") == 1) plan.usable = false;
+    // this library's few-row kernel: where the tuning run chose it (tuning key gemm_skinny = 0: never; 1: wherever it
+    // takes the problem, with a default configuration if none was timed)
+    {
+        const int want = tune_get("gemm_skinny");
+        SkinnyConfig c = plan.skinny;
+        if (want == 0) c = SkinnyConfig{};
+        else if (want == 1 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk)) {
+            const int pick = tune_get("gemm_skinny_config");             // 100 * variant + slices along K (tests)
+            if (pick >= 0) c = SkinnyConfig{pick / 100, pick % 100};
+            else if (c.variant < 0) c = skinny_default(M, K, N, workspace_bytes);
+        }
+        if (c.variant >= 0) {
+            const int rc = skinny_launch(c, x, w, y, M, K, N, ldy, workspace, workspace_bytes, st);
+            if (rc == 0) {
+                t_last_path = 2;
+                return 0;
+            }
+            if (rc != ONELLM_EUNSUPPORTED) return rc;        // (declined as given - alignment, workspace: on to the library)
+        }
+    }
     if (plan.usable) {
         const float alpha = 1.f, beta = 0.f;
         const hipblasStatus_t s = hipblasLtMatmul(handle, plan.desc, &alpha, w, plan.la, x, plan.lb, &beta, y, plan.lc, y,

@@ -1,0 +1,35 @@
+// y[M, N] = x[M, K] . W[K, N] for a handful of rows (a decode step's batch): fp16 operands, fp32 accumulation on the
+// matrix cores, the weights streamed once.  Host interface; the kernel is in skinny_gemm.hip.
+// (internal to libonellm_gemm.so: onellm_linear and onellm_linear_tune are its callers)
+#pragma once
+#include <stddef.h>
+#include <hip/hip_runtime.h>
+
+namespace onellm {
+
+constexpr int kSkinnyMaxRows = 32;          // M above this goes to the library
+
+// how one problem is run: which instantiation of the kernel, and in how many slices along K
+struct SkinnyConfig {
+    int variant = -1;                       // -1: not this kernel
+    int splits = 0;
+};
+
+// Whether the kernel takes the problem at all (shape and layout only; pointers are checked at launch).
+bool skinny_shape_ok(int dtype, int M, int K, int N, int ldy, int w_is_nk);
+
+// Configurations worth timing for a problem, `max` at most; with_workspace_bytes bounds the slices along K (a sliced
+// run keeps its partial sums in the caller's workspace).  Returns how many were written.
+int skinny_candidates(int M, int K, int N, size_t with_workspace_bytes, SkinnyConfig* out, int max);
+
+// A reasonable configuration without timing anything (what a forced run uses); variant -1 if there is none.
+SkinnyConfig skinny_default(int M, int K, int N, size_t with_workspace_bytes);
+
+// Queues the multiplication.  0, ONELLM_EUNSUPPORTED (this kernel does not take the problem as given: alignment,
+// workspace too small, no counter set left for a sliced run - the caller goes on to the library) or a hipError_t.
+// A sliced run (splits > 1) uses `workspace` for partial sums; calls that share a workspace must not overlap, which
+// is the library's rule for the same buffer as well.
+int skinny_launch(SkinnyConfig c, const void* x, const void* w, void* y, int M, int K, int N, int ldy, void* workspace,
+                  size_t workspace_bytes, hipStream_t stream);
+
+}  // namespace onellm

@@ -22,6 +22,8 @@ Knob g_knobs[] = {
     {"attn_fused_finish", {-1}}, // 0: keep the separate merge launch even when the workspace is declared zeroed
     {"prefill_generic", {-1}},   // 1: the index-walking prefill kernel also where the row-walking one applies
     {"attn_gqa_valu", {-1}},     // 1: grouped-query heads on the vector ALU kernel instead of the MFMA one
+    {"gemm_skinny", {-1}},       // onellm_linear's own few-row kernel: 0 = never (not timed either), 1 = wherever it takes the problem; default: where the tuning run chose it
+    {"gemm_skinny_config", {-1}}, // with gemm_skinny = 1: 100 * kernel variant + slices along K, instead of the timed or default choice (tests)
     {"gemm_no_library", {-1}},   // 1: onellm_linear behaves as if the GEMM library had declined the problem (tests)
     {"attn_ordered_finish", {-1}}, // 1: release on the fused finish's counter add + acquire fence in the merging piece
     {"attn_early_look", {-1}},   // 1 / 0: a piece that finds the unit's other pieces arrived merges it from its registers / never looks

@@ -124,7 +124,8 @@ def test_linear_matches_the_oracle(H, G, ref, dtype, M, K, N):
     assert H.onellm_layers_linear(code, dx.data_ptr(), dw.data_ptr(), y.data_ptr(), M, K, N, 0, 0, 0) == 0, H.onellm_layers_last_error()
     np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[dtype])
     if K >= 4096:
-        assert G.onellm_linear_last_path() == 1, "the projection shapes of a 7B layer must run the library GEMM"
+        # (the library GEMM, or this library's few-row kernel where the timing run of the layer shim chose it)
+        assert G.onellm_linear_last_path() in (1, 2), "the projection shapes of a 7B layer must not run the plain kernel"
     # W given as [N, K]
     dwt = _dev(torch, w.T)
     y2 = torch.zeros_like(y)
@@ -138,6 +139,109 @@ def test_linear_matches_the_oracle(H, G, ref, dtype, M, K, N):
     got = pair.cpu().numpy().astype(np.float64)
     np.testing.assert_allclose(got[:, 0], want.astype(np.float64), **TOL[dtype])
     np.testing.assert_allclose(got[:, 1], ref.linear(x, w2).astype(np.float64), **TOL[dtype])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,ldy", [(1, 64, 8, 0), (3, 128, 72, 0), (16, 4096, 4096, 0), (16, 11008, 4096, 0), (7, 4096, 12288, 0),
+                                       (16, 4096, 11008, 22016), (32, 4096, 4096, 0), (17, 256, 136, 140), (16, 1024, 200, 0)])
+def test_few_row_kernel_matches_the_oracle_in_every_configuration(G, ref, M, K, N, ldy):
+    """onellm_linear's own kernel for a decode step's rows, forced (tuning key gemm_skinny = 1) through every kernel
+    variant and every number of slices along K that takes the problem: fp16 parity with the oracle, untouched
+    padding columns, the same bits on a second call (the sliced runs reuse one workspace and its arrival counters)."""
+    import torch
+    from onellm_amd import capi
+    announce("few-row linear", M, K, N, ldy)
+    rng = np.random.default_rng(M * 131 + N)
+    x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    want = ref.linear(x, w).astype(np.float64)
+    dx, dw = _dev(torch, x), _dev(torch, w)
+    ld = ldy or N
+    ws = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dx.device)
+    ran = []
+    capi.tune_set("gemm_skinny", 1)
+    try:
+        for variant in range(8):
+            for splits in (1, 2, 3, 4, 6, 8, 16):
+                capi.tune_set("gemm_skinny_config", 100 * variant + splits)
+                outs = []
+                for rep in range(2):
+                    y = torch.full((M, ld), float("nan"), dtype=torch.float16, device=dx.device)
+                    capi.linear(dx, dw, y, ldy=ld, workspace=ws)
+                    torch.cuda.synchronize()
+                    outs.append(y.cpu().numpy())
+                if G.onellm_linear_last_path() != 2:
+                    continue                               # (this configuration does not take the problem: the library ran)
+                ran.append((variant, splits))
+                got = outs[0]
+                np.testing.assert_allclose(got[:, :N].astype(np.float64), want, err_msg=str((variant, splits)), **TOL[np.float16])
+                assert np.isnan(got[:, N:]).all(), (variant, splits)
+                assert np.array_equal(outs[0][:, :N], outs[1][:, :N]), (variant, splits)
+    finally:
+        capi.tune_set("gemm_skinny", -1)
+        capi.tune_set("gemm_skinny_config", -1)
+    assert len(ran) >= 3, ran
+    assert any(s > 1 for _, s in ran) or K < 128, ran
+
+
+@pytest.mark.gpu
+def test_few_row_kernel_declines_what_it_is_not_built_for(G, ref):
+    """Forced or not, a problem outside the kernel's rules (fp32, W as [N, K], too many rows, K not in whole
+    64-row blocks, N or the row stride not in whole pieces, a misaligned operand) runs the library as before."""
+    import torch
+    from onellm_amd import capi
+    capi.tune_set("gemm_skinny", 1)
+    try:
+        for dtype, M, K, N, nk, shift in [(np.float32, 4, 128, 64, False, 0), (np.float16, 4, 128, 64, True, 0), (np.float16, 33, 128, 64, False, 0),
+                                          (np.float16, 4, 96, 64, False, 0), (np.float16, 4, 128, 68, False, 0), (np.float16, 4, 128, 64, False, 1)]:
+            announce("few-row linear declines", dtype.__name__, M, K, N, nk, shift)
+            rng = np.random.default_rng(K + N)
+            x = (rng.standard_normal((M, K)) * 0.5).astype(dtype)
+            w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(dtype)
+            dx = _dev(torch, x)
+            wbuf = torch.zeros(K * N + 8, dtype=dx.dtype, device=dx.device)
+            dw = wbuf[shift:shift + K * N].view(N, K) if nk else wbuf[shift:shift + K * N].view(K, N)
+            dw.copy_(_dev(torch, w.T if nk else w))
+            y = torch.zeros((M, N), dtype=dx.dtype, device=dx.device)
+            rc = G.onellm_linear(1 if dtype == np.float16 else 0, dx.data_ptr(), dw.data_ptr(), y.data_ptr(), M, K, N, 0, int(nk), None, 0, None)
+            torch.cuda.synchronize()
+            assert rc == 0 and G.onellm_linear_last_path() != 2
+            np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), ref.linear(x, w).astype(np.float64), **TOL[dtype])
+    finally:
+        capi.tune_set("gemm_skinny", -1)
+
+
+@pytest.mark.gpu
+def test_tuning_run_times_the_few_row_kernel_and_keeps_results_right(G, ref):
+    """onellm_linear_tune on a decode-step projection (cold weights: it rotates over copies of W) leaves a plan -
+    the library's algorithm or this library's kernel, whichever was faster - that still matches the oracle; with
+    gemm_skinny = 0 the plan is the library's."""
+    import torch
+    from onellm_amd import capi
+    M, K, N = 16, 2048, 4096
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    want = ref.linear(x, w).astype(np.float64)
+    dx, dw = _dev(torch, x), _dev(torch, w)
+    ws = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dx.device)
+    announce("linear tune", M, K, N)
+    best, first = capi.linear_tune(capi.FP16, M, K, N, workspace=ws)
+    assert 0 < best <= first * 1.5
+    y = torch.zeros((M, N), dtype=torch.float16, device=dx.device)
+    capi.linear(dx, dw, y, workspace=ws)
+    torch.cuda.synchronize()
+    assert G.onellm_linear_last_path() in (1, 2)
+    np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), want, **TOL[np.float16])
+    capi.tune_set("gemm_skinny", 0)
+    try:
+        y.zero_()
+        capi.linear(dx, dw, y, workspace=ws)
+        torch.cuda.synchronize()
+        assert G.onellm_linear_last_path() == 1
+        np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), want, **TOL[np.float16])
+    finally:
+        capi.tune_set("gemm_skinny", -1)
 
 
 def _random_layers(rng, dtype, Hq, Hkv, D, I, L, bias=True):
@@ -372,7 +476,8 @@ def test_a_large_projection_without_a_library_kernel_is_an_error_not_a_slow_succ
     rng = np.random.default_rng(1)
     capi.tune_set("gemm_no_library", 1)
     try:
-        for (M, K, N), big in (((3, 40, 24), False), ((16, 2048, 1024), True)):
+        # (40 rows: more than this library's own few-row kernel takes, which would otherwise step in for the library)
+        for (M, K, N), big in (((3, 40, 24), False), ((40, 2048, 1024), True)):
             x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
             w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
             dx, dw = _dev(torch, x), _dev(torch, w)
