@@ -246,19 +246,22 @@ def cpu_norm(N, H, fused, budget_s):
 def decoder_layer_section(capi, dev, args):
     """One whole decoder layer of the Llama-2-7B shape at batch 16, ctx 4096, as LlamaSelfDecoder sequences it:
     RMSNorm -> qkv projection -> fused masked attention -> output projection -> fused add-bias-residual-RMSNorm ->
-    gate / up projections -> SwiGLU -> down projection -> fused add-bias-residual-RMSNorm.  The projections are library
-    GEMMs (hipBLASLt through onellm_linear); everything else is this repository's kernels."""
+    gate / up projections -> SwiGLU -> down projection -> fused add-bias-residual-RMSNorm.  The projections go through
+    onellm_linear (hipBLASLt or this repository's few-row kernel, whichever its tuning run found faster); everything
+    else is this repository's kernels.  Steps rotate over three sets of weights and of caches (1.2 GB and 3.2 GB), so
+    that every step meets its weights cold, as a layer inside a 32-layer model does."""
     import torch
     B, H, D, S, I, t = 16, 32, 128, 4096, 11008, 4096
     hid = H * D
     g = torch.Generator(device=dev).manual_seed(7)
     rnd = lambda *shape, scale=1.0: (torch.randn(*shape, device=dev, generator=g) * scale).half()
-    wqkv, wo = rnd(hid, 3 * hid, scale=hid ** -0.5), rnd(hid, hid, scale=hid ** -0.5)
-    wg, wu, wd = rnd(hid, I, scale=hid ** -0.5), rnd(hid, I, scale=hid ** -0.5), rnd(I, hid, scale=I ** -0.5)
+    NSETS = 3
+    wsets = [dict(wqkv=rnd(hid, 3 * hid, scale=hid ** -0.5), wo=rnd(hid, hid, scale=hid ** -0.5), wgate=rnd(hid, I, scale=hid ** -0.5),
+                  wup=rnd(hid, I, scale=hid ** -0.5), wdown=rnd(I, hid, scale=I ** -0.5)) for _ in range(NSETS)]
     bqkv, bo, bd = rnd(3 * hid, scale=0.1), rnd(hid, scale=0.1), rnd(hid, scale=0.1)
     g1, g2, g3 = (torch.rand(hid, device=dev, generator=g) + 0.5).half(), (torch.rand(hid, device=dev, generator=g) + 0.5).half(), \
         (torch.rand(hid, device=dev, generator=g) + 0.5).half()
-    sets = [(rnd(1, B, H, S, D, scale=0.5), rnd(1, B, H, S, D, scale=0.5)) for _ in range(3)]
+    sets = [(rnd(1, B, H, S, D, scale=0.5), rnd(1, B, H, S, D, scale=0.5)) for _ in range(NSETS)]
     x0 = rnd(B, hid)
     x, y = x0.clone(), torch.empty_like(x0)
     qkv, att = torch.empty(B, 3 * H, D, dtype=torch.float16, device=dev), torch.empty(B, hid, dtype=torch.float16, device=dev)
@@ -274,27 +277,27 @@ def decoder_layer_section(capi, dev, args):
         capi.rmsnorm(y, g1, 1e-5)
 
     def proj_qkv(i):
-        capi.linear(y, wqkv, qkv.view(B, 3 * hid), workspace=ws_gemm)
+        capi.linear(y, wsets[i % NSETS]["wqkv"], qkv.view(B, 3 * hid), workspace=ws_gemm)
 
     def attention(i):
         kc, vc = sets[i % len(sets)]
         capi.decode_attn(qkv, bqkv, kc, vc, att, H, t, D, 10000.0, rope_pos_offset=-1, workspace=ws_attn)
 
     def proj_out(i):
-        capi.linear(att, wo, y, workspace=ws_gemm)
+        capi.linear(att, wsets[i % NSETS]["wo"], y, workspace=ws_gemm)
 
     def norm_mid(i):
         capi.fused_add_bias_residual_rmsnorm(x, y, bo, g2, 1e-5)
 
     def proj_gate_up(i):
-        capi.linear(y, wg, pair, ldy=2 * I, workspace=ws_gemm)
-        capi.linear(y, wu, pair.view(-1)[I:], ldy=2 * I, workspace=ws_gemm)
+        capi.linear(y, wsets[i % NSETS]["wgate"], pair, ldy=2 * I, workspace=ws_gemm)
+        capi.linear(y, wsets[i % NSETS]["wup"], pair.view(-1)[I:], ldy=2 * I, workspace=ws_gemm)
 
     def swiglu(i):
         capi.silu_and_mul(pair, act)
 
     def proj_down(i):
-        capi.linear(act, wd, y, workspace=ws_gemm)
+        capi.linear(act, wsets[i % NSETS]["wdown"], y, workspace=ws_gemm)
 
     def norm_out(i):
         capi.fused_add_bias_residual_rmsnorm(x, y, bd, g3, 1e-5)
@@ -312,33 +315,35 @@ def decoder_layer_section(capi, dev, args):
     steps = max(args.steps // 3, 10)
     # the whole layer as the C++ LlamaSelfDecoder queues it (one call per step; its output-projection and down-projection
     # biases are applied by the fused norms, as above)
-    dec = capi.SelfDecoder(capi.FP16, B, H, H, D, I, S, D, 10000.0, 1e-5,
-                           [dict(attn_norm=g1, ffn_norm=g2, wqkv=wqkv, bqkv=bqkv, wo=wo, bo=bo, wdown=wd, bdown=bd, wgate=wg, wup=wu)],
-                           g3)
+    def decoder(k, **kw):
+        return capi.SelfDecoder(capi.FP16, B, H, H, D, I, S, D, 10000.0, 1e-5,
+                                [dict(attn_norm=g1, ffn_norm=g2, bqkv=bqkv, bo=bo, bdown=bd, **wsets[k])], g3, **kw)
+
+    decs = [decoder(k) for k in range(NSETS)]
 
     def layer_cpp(i):
         if i % 8 == 0:
             x.copy_(x0)
-        kc, vc = sets[i % len(sets)]
-        dec.forward(t, x, y, kc, vc)
+        kc, vc = sets[i % NSETS]
+        decs[i % NSETS].forward(t, x, y, kc, vc)
 
     ms = time_steps(layer_cpp, steps, max(args.warmup // 3, 3))
-    dec.close()
+    for d in decs:
+        d.close()
 
     # the same step captured once into a HIP graph on a side stream and replayed (one graph per cache set)
     side = torch.cuda.Stream()
-    dec_g = capi.SelfDecoder(capi.FP16, B, H, H, D, I, S, D, 10000.0, 1e-5,
-                             [dict(attn_norm=g1, ffn_norm=g2, wqkv=wqkv, bqkv=bqkv, wo=wo, bo=bo, wdown=wd, bdown=bd, wgate=wg, wup=wu)],
-                             g3, stream=side.cuda_stream)
+    decs_g = [decoder(k, stream=side.cuda_stream) for k in range(NSETS)]
     torch.cuda.synchronize()
     graphs = []
     with torch.cuda.stream(side):
-        dec_g.forward(t, x, y, sets[0][0], sets[0][1])          # ordinary step first: buffers and GEMM plans
+        for d in decs_g:
+            d.forward(t, x, y, sets[0][0], sets[0][1])          # ordinary step first: buffers and GEMM plans
     torch.cuda.synchronize()
-    for kc, vc in sets:
+    for d, (kc, vc) in zip(decs_g, sets):
         gr = torch.cuda.CUDAGraph()
         with torch.cuda.graph(gr, stream=side):
-            dec_g.forward(t, x, y, kc, vc)
+            d.forward(t, x, y, kc, vc)
         graphs.append(gr)
 
     def layer_graph(i):
@@ -349,17 +354,22 @@ def decoder_layer_section(capi, dev, args):
     ms_graph = time_steps(layer_graph, steps, 3)
     torch.cuda.synchronize()
     del graphs
-    dec_g.close()
+    for d in decs_g:
+        d.close()
     ms_py = time_steps(layer, steps, 3)
-    weight_bytes = 2 * (wqkv.numel() + wo.numel() + wg.numel() + wu.numel() + wd.numel())
+    weight_bytes = 2 * sum(w.numel() for w in wsets[0].values())
     nb = weight_bytes + attn_bytes(B, H, H, D, [t] * B, 2)
     e = entry(ms, nb)
-    e["parts_us"] = {name: round(time_steps(fn, steps, 3) * 1e3, 2) for name, fn in parts}
+    e["parts_us"], e["gemm_path"] = {}, {}
+    path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel"}
+    for name, fn in parts:
+        e["parts_us"][name] = round(time_steps(fn, steps, 3) * 1e3, 2)
+        if name.endswith("_proj"):
+            e["gemm_path"][name] = path_names.get(capi.gemm_lib().onellm_linear_last_path(), "?")
     e["us_same_sequence_from_python"] = round(ms_py * 1e3, 2)
     e["us_graph_replay"] = round(ms_graph * 1e3, 2)
-    e["gemm_path"] = "hipBLASLt" if capi.gemm_lib().onellm_linear_last_path() == 1 else "plain kernel"
-    e["note"] = ("bytes = the five weight matrices (%d) + the attention step's algorithmic bytes; parts are timed "
-                 "one at a time, so their sum includes a launch gap per part" % weight_bytes)
+    e["note"] = ("bytes = the five weight matrices (%d) + the attention step's algorithmic bytes; steps rotate over %d sets of "
+                 "weights and caches; parts are timed one at a time, so their sum includes a launch gap per part" % (weight_bytes, NSETS))
     return {"decoder_layer_llama7b_b16_ctx4096": e}
 
 
