@@ -269,8 +269,9 @@ def decoder_layer_section(capi, dev, args):
     ws_attn = torch.empty(capi.decode_attn_workspace_bytes(B, H, H, D, t), dtype=torch.uint8, device=dev)
     ws_gemm = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dev)
 
-    for (K_, N_, ld_) in ((hid, 3 * hid, 0), (hid, hid, 0), (hid, I, 2 * I), (I, hid, 0)):
+    for (K_, N_, ld_) in ((hid, 3 * hid, 0), (hid, hid, 0), (I, hid, 0)):
         capi.linear_tune(capi.FP16, B, K_, N_, ldy=ld_, workspace=ws_gemm)
+    capi.linear_pair_tune(capi.FP16, B, hid, I, ldy=2 * I, workspace=ws_gemm)
 
     def norm_in(i):
         y.copy_(x)
@@ -290,8 +291,7 @@ def decoder_layer_section(capi, dev, args):
         capi.fused_add_bias_residual_rmsnorm(x, y, bo, g2, 1e-5)
 
     def proj_gate_up(i):
-        capi.linear(y, wsets[i % NSETS]["wgate"], pair, ldy=2 * I, workspace=ws_gemm)
-        capi.linear(y, wsets[i % NSETS]["wup"], pair.view(-1)[I:], ldy=2 * I, workspace=ws_gemm)
+        capi.linear_pair(y, wsets[i % NSETS]["wgate"], wsets[i % NSETS]["wup"], pair, pair.view(-1)[I:], ldy=2 * I, workspace=ws_gemm)
 
     def swiglu(i):
         capi.silu_and_mul(pair, act)
@@ -361,7 +361,7 @@ def decoder_layer_section(capi, dev, args):
     nb = weight_bytes + attn_bytes(B, H, H, D, [t] * B, 2)
     e = entry(ms, nb)
     e["parts_us"], e["gemm_path"] = {}, {}
-    path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel"}
+    path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel", 3: "own few-row kernel, both in one launch"}
     for name, fn in parts:
         e["parts_us"][name] = round(time_steps(fn, steps, 3) * 1e3, 2)
         if name.endswith("_proj"):

@@ -48,6 +48,12 @@ class cublasWrapper;   // carried for signature compatibility only; may be null,
 void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool trans_a = false, bool trans_b = false,
                       bool shared_out_buf = false);
 
+// Both projections of a feed-forward block that share their input (the reference calls launchLinearGemm twice,
+// src/layers/ffn/ffn.cpp:61-62): output {2, M, N} holds first's result in its first half and second's in the other,
+// rows interleaved as [M, 2, N], exactly as the two calls leave it; where the few-row kernel of the projection
+// library takes the problem both go out in one launch.  The weights are {K, N} matrices of one shape.
+void launchLinearGemmPair(Tensor* input, BaseWeight& first, BaseWeight& second, Tensor* output);
+
 // launchLinearGemm times the GEMM library's candidate algorithms the first time it sees a shape and keeps the fastest;
 // that first call synchronises the null stream.  Switch it off to keep every call asynchronous (for example before
 // capturing a step into a graph; shapes tuned earlier stay tuned).

@@ -42,11 +42,25 @@ int onellm_linear(int dtype, const void* x, const void* w, void* y, int M, int K
 int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
                        onellm_stream_t stream, float* best_us, float* first_us);
 
+/* Two projections that share their input and shape - the gate and up projections of a feed-forward block
+ * (src/layers/ffn/ffn.cpp:61-62 calls launchLinearGemm twice): y_first = x . w_first, y_second = x . w_second, both
+ * with row stride ldy.  The result is that of two onellm_linear calls; where this library's few-row kernel takes the
+ * problem and onellm_linear_pair_tune found it faster, both go out in one launch. */
+int onellm_linear_pair(int dtype, const void* x, const void* w_first, const void* w_second, void* y_first, void* y_second,
+                       int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
+                       onellm_stream_t stream);
+
+/* Optional, once per shape: onellm_linear_tune for the single projection, then the one-launch forms of the pair
+ * against two tuned calls, on stand-in operands as above.  best_us / two_calls_us (either may be NULL) receive the time
+ * of what onellm_linear_pair will run from then on and of the two-call sequence. */
+int onellm_linear_pair_tune(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
+                            onellm_stream_t stream, float* best_us, float* two_calls_us);
+
 /* workspace size onellm_linear can make use of (a constant; any smaller size is valid too) */
 size_t onellm_linear_workspace_bytes(void);
 
-/* what the last onellm_linear call on this thread ran: 1 the library GEMM, 2 this library's few-row kernel, 0 the
- * plain fallback kernel */
+/* what the last onellm_linear / onellm_linear_pair call on this thread ran: 1 the library GEMM, 2 this library's
+ * few-row kernel, 3 that kernel for both projections of a pair in one launch, 0 the plain fallback kernel */
 int onellm_linear_last_path(void);
 
 /* allow != 0: problems of any size may run the plain kernel when the library declines them (process-wide; off by

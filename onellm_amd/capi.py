@@ -233,6 +233,8 @@ GEMM_SYMBOLS = {
     "onellm_linear_tune": (_ci, [_ci, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp, ctypes.POINTER(_cf), ctypes.POINTER(_cf)]),
     "onellm_linear_workspace_bytes": (_sz, []),
     "onellm_linear_last_path": (_ci, []),
+    "onellm_linear_pair": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
+    "onellm_linear_pair_tune": (_ci, [_ci, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp, ctypes.POINTER(_cf), ctypes.POINTER(_cf)]),
     "onellm_linear_allow_plain": (_ci, [_ci]),
 }
 _gemm = None
@@ -266,6 +268,30 @@ def linear_tune(dtype_code, M, K, N, ldy=0, w_is_nk=False, workspace=None):
                                        ctypes.byref(first))
     _check(rc, "onellm_linear_tune")
     return best.value, first.value
+
+
+def linear_pair_tune(dtype_code, M, K, N, ldy=0, w_is_nk=False, workspace=None):
+    """Tune the single projection, then time the one-launch forms of a pair against two calls; returns
+    (best_us, two_calls_us)."""
+    best, two = _cf(0.0), _cf(0.0)
+    rc = gemm_lib().onellm_linear_pair_tune(dtype_code, M, K, N, int(ldy), int(bool(w_is_nk)), _ptr(workspace),
+                                            workspace.numel() if workspace is not None else 0, _stream(), ctypes.byref(best),
+                                            ctypes.byref(two))
+    _check(rc, "onellm_linear_pair_tune")
+    return best.value, two.value
+
+
+def linear_pair(x, w_first, w_second, y_first, y_second, w_is_nk=False, ldy=0, workspace=None):
+    """y_first = x . w_first and y_second = x . w_second (same shapes, row stride ldy): the gate / up pair."""
+    M, K = x.shape
+    N = w_first.shape[0] if w_is_nk else w_first.shape[1]
+    assert w_first.shape == w_second.shape and (w_first.shape[1] if w_is_nk else w_first.shape[0]) == K
+    assert x.dtype == w_first.dtype == w_second.dtype == y_first.dtype == y_second.dtype
+    assert x.is_cuda and x.is_contiguous() and w_first.is_contiguous() and w_second.is_contiguous()
+    rc = gemm_lib().onellm_linear_pair(_dt(x), x.data_ptr(), w_first.data_ptr(), w_second.data_ptr(), y_first.data_ptr(),
+                                       y_second.data_ptr(), M, K, N, int(ldy), int(bool(w_is_nk)), _ptr(workspace),
+                                       workspace.numel() if workspace is not None else 0, _stream())
+    _check(rc, "onellm_linear_pair")
 
 
 def linear(x, w, y, w_is_nk=False, ldy=0, workspace=None):

@@ -99,6 +99,20 @@ void tune_once(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* ws, s
     (void)onellm_linear_tune(dtype, M, K, N, ldy, w_is_nk, ws, ws_bytes, onellmGetLaunchStream(), nullptr, nullptr);   // best effort
 }
 
+// the same for the one-launch forms of a pair of projections (the key's last element tells the two tables apart)
+void tune_pair_once(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* ws, size_t ws_bytes)
+{
+    {
+        std::lock_guard<std::mutex> g(g_tuned_mu);
+        const auto key = std::make_tuple(dtype, M, K, N, ldy, w_is_nk + 2);
+        if (!g_autotune || g_tuned.count(key)) return;
+        if (stream_is_capturing(onellmGetLaunchStream())) return;
+        g_tuned.insert(key);
+        g_tuned.insert(std::make_tuple(dtype, M, K, N, ldy, w_is_nk));    // (the pair's tuning run covers the single projection)
+    }
+    (void)onellm_linear_pair_tune(dtype, M, K, N, ldy, w_is_nk, ws, ws_bytes, onellmGetLaunchStream(), nullptr, nullptr);   // best effort
+}
+
 Tensor* new_buffer(BaseAllocator* a, DataType t, std::vector<int> shape)
 {
     size_t n = elt_bytes(t);
@@ -159,6 +173,29 @@ void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool tr
     const int rc = onellm_linear(dtype_code, input->data, weight.data, y, M, K, N, ldy, trans_b ? 1 : 0, ws.ptr, ws.bytes,
                                  onellmGetLaunchStream());
     if (rc != 0) throw std::runtime_error(std::string("[TM][ERROR] launchLinearGemm: ") + onellm_error_string(rc) + " \n");
+}
+
+// the two launchLinearGemm calls of src/layers/ffn/ffn.cpp:61-62 (gate, then up with shared_out_buf) as one
+void launchLinearGemmPair(Tensor* input, BaseWeight& first, BaseWeight& second, Tensor* output)
+{
+    require(input && output && input->data && output->data && first.data && second.data, "launchLinearGemmPair: null tensor or weight");
+    require(input->dtype == output->dtype, "launchLinearGemmPair: input and output element types differ");
+    require(first.shape.size() == 2 && second.shape == first.shape, "launchLinearGemmPair: the weights must be two matrices of one shape");
+    const size_t e = elt_bytes(input->dtype);
+    const WeightType want = input->dtype == FP32 ? WeightType::FP32_W : WeightType::FP16_W;
+    require(first.type == want && second.type == want, "launchLinearGemmPair: weight element type does not match the activations");
+    const int M = rows_of(input), K = cols_of(input), N = first.shape[1];
+    require(first.shape[0] == K, "launchLinearGemmPair: inner sizes differ (" + std::to_string(K) + " vs " + std::to_string(first.shape[0]) + ")");
+    require(output->shape.size() == 3 && output->shape[0] == 2 && output->shape[1] == M && output->shape[2] == N,
+            "launchLinearGemmPair: the output must be the {2, M, N} pair buffer");
+    const int ldy = 2 * N;
+    char* y = static_cast<char*>(output->data);
+    const GemmWorkspace::Buffer ws = g_gemm_ws.get(onellmGetLaunchStream());
+    const int dtype_code = input->dtype == FP32 ? ONELLM_FP32 : ONELLM_FP16;
+    tune_pair_once(dtype_code, M, K, N, ldy, 0, ws.ptr, ws.bytes);
+    const int rc = onellm_linear_pair(dtype_code, input->data, first.data, second.data, y, y + (size_t)N * e, M, K, N, ldy, 0, ws.ptr,
+                                      ws.bytes, onellmGetLaunchStream());
+    if (rc != 0) throw std::runtime_error(std::string("[TM][ERROR] launchLinearGemmPair: ") + onellm_error_string(rc) + " \n");
 }
 
 // ------------------------------------------------------------------------------------------- attention layer
@@ -268,8 +305,7 @@ void LLaMAFFNLayer::forward(TensorMap& inputs, TensorMap& outputs, LLaMAFFNWeigh
     if (ffn_input.dtype == FP16) allocForForward<half>(rows);
     else allocForForward<float>(rows);
 
-    launchLinearGemm(&ffn_input, weights.gate, SwiGLU_input);
-    launchLinearGemm(&ffn_input, weights.up, SwiGLU_input, false, false, true);
+    launchLinearGemmPair(&ffn_input, weights.gate, weights.up, SwiGLU_input);
     if (ffn_input.dtype == FP16)
         launchAct(static_cast<const half*>(SwiGLU_input->data), static_cast<half*>(down_proj_input->data), rows, inter_size);
     else

@@ -155,6 +155,84 @@ hipblasLtHandle_t device_handle(DeviceState& ds)
 }  // namespace
 }  // namespace onellm
 
+namespace onellm {
+namespace {
+
+// Stand-in operands for a timing run (values do not matter; 0x3c3c.. is ~1.06 in fp16 and a small normal number in
+// fp32), two events, and the loop that times one candidate.
+//
+// The weights of a model are far larger than the chip's caches, so a projection always meets its matrix cold.  A
+// timing loop over one matrix would not: it stays in the 256 MB memory-side cache and every candidate looks up to
+// twice as fast as it will be (a 7B down projection, 90 MB: 29 us warm, 50 us cold with the same algorithm).  The
+// runs therefore rotate over enough copies of W to exceed that cache.
+struct TimingRig {
+    static constexpr int kMaxCopies = 16;
+    static constexpr size_t kColdBytes = 640u << 20;
+    void *x = nullptr, *y = nullptr, *w[kMaxCopies] = {};
+    int copies = 0;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+
+    hipError_t make(size_t x_bytes, size_t y_bytes, size_t w_bytes, hipStream_t st)
+    {
+        copies = (int)std::min<size_t>(kMaxCopies, std::max<size_t>(2, (kColdBytes + w_bytes - 1) / w_bytes));
+        copies &= ~1;                                            // (pairs of matrices for the two-problem launch)
+        hipError_t e = hipMalloc(&x, x_bytes);
+        for (int c = 0; c < copies && e == hipSuccess; ++c) e = hipMalloc(&w[c], w_bytes);
+        if (e == hipSuccess) e = hipMalloc(&y, y_bytes);
+        if (e == hipSuccess) e = hipEventCreate(&t0);
+        if (e == hipSuccess) e = hipEventCreate(&t1);
+        if (e != hipSuccess) return e;
+        (void)hipMemsetAsync(x, 0x3c, x_bytes, st);
+        for (int c = 0; c < copies; ++c) (void)hipMemsetAsync(w[c], 0x3c, w_bytes, st);
+        return hipSuccess;
+    }
+    ~TimingRig()
+    {
+        if (x) (void)hipFree(x);
+        for (void* c : w)
+            if (c) (void)hipFree(c);
+        if (y) (void)hipFree(y);
+        if (t0) (void)hipEventDestroy(t0);
+        if (t1) (void)hipEventDestroy(t1);
+    }
+    // milliseconds per call of run(r) (true: queued), over `runs` calls after two that do not count; negative when a
+    // call was refused; rc receives a hipError_t if the stream failed
+    template <typename F>
+    float time(F&& run, int runs, hipStream_t st, int& rc)
+    {
+        constexpr int kWarm = 2;
+        bool ok = true;
+        for (int r = 0; r < kWarm + runs && ok; ++r) {
+            if (r == kWarm) (void)hipEventRecord(t0, st);
+            ok = run(r);
+        }
+        (void)hipEventRecord(t1, st);
+        const hipError_t e = hipEventSynchronize(t1);
+        if (e != hipSuccess) {
+            rc = (int)e;
+            return -1.f;
+        }
+        if (!ok) return -1.f;
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, t0, t1);
+        return ms / runs;
+    }
+};
+
+// what runs the two projections of a feed-forward block that share their input: key (M, K, N, ldy, workspace or not);
+// variant -1: two ordinary calls
+std::map<std::tuple<int, int, int, int, int, int>, SkinnyConfig> g_pair_plans;      // (first element: device)
+
+bool stream_capturing(hipStream_t st)
+{
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) (void)hipGetLastError();
+    return capturing != hipStreamCaptureStatusNone;
+}
+
+}  // namespace
+}  // namespace onellm
+
 extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
                                   onellm_stream_t stream, float* best_us, float* first_us)
 {
@@ -185,89 +263,50 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
     constexpr int kWantOwn = 64;
     SkinnyConfig own[kWantOwn];
     const int n_own = (tune_get("gemm_skinny") != 0 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk))
-                          ? skinny_candidates(M, K, N, workspace_bytes, own, kWantOwn) : 0;
+                          ? skinny_candidates(M, K, N, workspace_bytes, 1, own, kWantOwn) : 0;
     if (n == 0 && n_own == 0) {
         destroy_plan(p);
         return ONELLM_EUNSUPPORTED;
     }
     // the timing runs allocate, synchronise and launch: none of that may happen on a stream that is being captured
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) (void)hipGetLastError();
-    if (capturing != hipStreamCaptureStatusNone) {
+    if (stream_capturing(st)) {
         destroy_plan(p);
         return ONELLM_ECAPTURING;
     }
-
-    // stand-in operands of the right size (values do not matter for the timing; 0x3c3c.. is ~1.06 in fp16 and a
-    // small normal number in fp32)
-    // The weights of a model are far larger than the chip's caches, so a projection always meets its matrix cold.  A
-    // timing loop over one matrix would not: it stays in the 256 MB memory-side cache and every candidate looks up to
-    // twice as fast as it will be (a 7B down projection, 90 MB: 29 us warm, 50 us cold with the same algorithm).  The
-    // runs therefore rotate over enough copies of W to exceed that cache.
     const size_t esz = dtype == ONELLM_FP16 ? 2 : 4;
-    const size_t w_bytes = (size_t)K * N * esz;
-    constexpr size_t kColdBytes = 640u << 20;
-    constexpr int kMaxCopies = 16;
-    const int copies = (int)std::min<size_t>(kMaxCopies, std::max<size_t>(2, (kColdBytes + w_bytes - 1) / w_bytes));
-    void *x = nullptr, *y = nullptr, *w[kMaxCopies] = {};
-    hipEvent_t t0 = nullptr, t1 = nullptr;
     int rc = 0;
-    auto cleanup = [&] {
-        if (x) (void)hipFree(x);
-        for (void* c : w)
-            if (c) (void)hipFree(c);
-        if (y) (void)hipFree(y);
-        if (t0) (void)hipEventDestroy(t0);
-        if (t1) (void)hipEventDestroy(t1);
-    };
-    e = hipMalloc(&x, (size_t)M * K * esz);
-    for (int c = 0; c < copies && e == hipSuccess; ++c) e = hipMalloc(&w[c], w_bytes);
-    if (e != hipSuccess || (e = hipMalloc(&y, (size_t)M * ldy * esz)) != hipSuccess || (e = hipEventCreate(&t0)) != hipSuccess ||
-        (e = hipEventCreate(&t1)) != hipSuccess) {
-        cleanup();
-        destroy_plan(p);
-        return (int)e;
-    }
-    (void)hipMemsetAsync(x, 0x3c, (size_t)M * K * esz, st);
-    for (int c = 0; c < copies; ++c) (void)hipMemsetAsync(w[c], 0x3c, w_bytes, st);
-    const float alpha = 1.f, beta = 0.f;
     int best = -1, best_own = -1;
     float best_ms = 0.f, first_ms = 0.f, best_own_ms = 0.f;
-    constexpr int kWarm = 2;
-    const int runs = std::max(8, copies);
-    // candidate i of the library (i < n) or of this library's kernel (i >= n), timed over `runs` launches
-    for (int i = 0; i < n + n_own; ++i) {
-        bool ok = true;
-        for (int r = 0; r < kWarm + runs && ok; ++r) {
-            if (r == kWarm) (void)hipEventRecord(t0, st);
-            const void* wc = w[r % copies];
-            if (i < n)
-                ok = hipblasLtMatmul(handle, p.desc, &alpha, wc, p.la, x, p.lb, &beta, y, p.lc, y, p.lc, &cand[i].algo, workspace,
-                                     workspace_bytes, st) == HIPBLAS_STATUS_SUCCESS;
-            else
-                ok = skinny_launch(own[i - n], x, wc, y, M, K, N, ldy, workspace, workspace_bytes, st) == 0;
+    {
+        TimingRig rig;
+        if ((e = rig.make((size_t)M * K * esz, (size_t)M * ldy * esz, (size_t)K * N * esz, st)) != hipSuccess) {
+            destroy_plan(p);
+            return (int)e;
         }
-        (void)hipEventRecord(t1, st);
-        if ((e = hipEventSynchronize(t1)) != hipSuccess) {
-            rc = (int)e;
-            break;
-        }
-        if (!ok) continue;
-        float ms = 0.f;
-        (void)hipEventElapsedTime(&ms, t0, t1);
-        ms /= runs;
-        if (i == 0) first_ms = ms;
-        if (i < n) {
-            if (best < 0 || ms < best_ms) {
-                best = i;
-                best_ms = ms;
+        const float alpha = 1.f, beta = 0.f;
+        const int runs = std::max(8, rig.copies);
+        // candidate i of the library (i < n) or of this library's kernel (i >= n)
+        for (int i = 0; i < n + n_own && rc == 0; ++i) {
+            const float ms = rig.time([&](int r) {
+                const void* wc = rig.w[r % rig.copies];
+                if (i < n)
+                    return hipblasLtMatmul(handle, p.desc, &alpha, wc, p.la, rig.x, p.lb, &beta, rig.y, p.lc, rig.y, p.lc, &cand[i].algo,
+                                           workspace, workspace_bytes, st) == HIPBLAS_STATUS_SUCCESS;
+                return skinny_launch(own[i - n], rig.x, wc, rig.y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st) == 0;
+            }, runs, st, rc);
+            if (ms < 0.f) continue;
+            if (i == 0) first_ms = ms;
+            if (i < n) {
+                if (best < 0 || ms < best_ms) {
+                    best = i;
+                    best_ms = ms;
+                }
+            } else if (best_own < 0 || ms < best_own_ms) {
+                best_own = i - n;
+                best_own_ms = ms;
             }
-        } else if (best_own < 0 || ms < best_own_ms) {
-            best_own = i - n;
-            best_own_ms = ms;
         }
     }
-    cleanup();
     if (rc != 0 || (best < 0 && best_own < 0)) {
         destroy_plan(p);
         return rc != 0 ? rc : ONELLM_EUNSUPPORTED;
@@ -289,6 +328,62 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
     }
     if (best_us) *best_us = best_ms * 1e3f;
     if (first_us) *first_us = first_ms * 1e3f;
+    return 0;
+}
+
+extern "C" int onellm_linear_pair_tune(int dtype, int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
+                                       onellm_stream_t stream, float* best_us, float* two_calls_us)
+{
+    using namespace onellm;
+    // the single projection first: the two-call sequence below is what the pair has to beat
+    int rc = onellm_linear_tune(dtype, M, K, N, ldy, w_is_nk, workspace, workspace_bytes, stream, nullptr, nullptr);
+    if (rc != 0) return rc;
+    if (ldy == 0) ldy = N;
+    if (!workspace) workspace_bytes = 0;
+    if (workspace_bytes > kWorkspaceBytes) workspace_bytes = kWorkspaceBytes;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    constexpr int kWantOwn = 64;
+    SkinnyConfig own[kWantOwn];
+    const int n_own = (tune_get("gemm_skinny") != 0 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk))
+                          ? skinny_candidates(M, K, N, workspace_bytes, 2, own, kWantOwn) : 0;
+    const size_t esz = dtype == ONELLM_FP16 ? 2 : 4;
+    float two_ms = -1.f, best_ms = -1.f;
+    SkinnyConfig chosen;
+    {
+        TimingRig rig;
+        // (two outputs of M rows each, one after the other)
+        if ((e = rig.make((size_t)M * K * esz, 2 * (size_t)M * ldy * esz, (size_t)K * N * esz, st)) != hipSuccess) return (int)e;
+        void* y_second = static_cast<char*>(rig.y) + (size_t)M * ldy * esz;
+        const int runs = std::max(8, rig.copies);
+        two_ms = rig.time([&](int r) {
+            const void *w0 = rig.w[(2 * r) % rig.copies], *w1 = rig.w[(2 * r + 1) % rig.copies];
+            return onellm_linear(dtype, rig.x, w0, rig.y, M, K, N, ldy, w_is_nk, workspace, workspace_bytes, stream) == 0 &&
+                   onellm_linear(dtype, rig.x, w1, y_second, M, K, N, ldy, w_is_nk, workspace, workspace_bytes, stream) == 0;
+        }, runs, st, rc);
+        if (rc != 0) return rc;
+        if (two_ms < 0.f) return ONELLM_EUNSUPPORTED;
+        best_ms = two_ms;
+        for (int i = 0; i < n_own && rc == 0; ++i) {
+            const float ms = rig.time([&](int r) {
+                const void *w0 = rig.w[(2 * r) % rig.copies], *w1 = rig.w[(2 * r + 1) % rig.copies];
+                return skinny_launch(own[i], rig.x, w0, rig.y, w1, y_second, M, K, N, ldy, workspace, workspace_bytes, st) == 0;
+            }, runs, st, rc);
+            if (ms >= 0.f && ms < 0.97f * two_ms && ms < best_ms) {
+                best_ms = ms;
+                chosen = own[i];
+            }
+        }
+        if (rc != 0) return rc;
+    }
+    {
+        std::lock_guard<std::mutex> g(g_mu);
+        g_pair_plans[std::make_tuple(dev, M, K, N, ldy, workspace_bytes ? 1 : 0)] = chosen;
+    }
+    if (best_us) *best_us = best_ms * 1e3f;
+    if (two_calls_us) *two_calls_us = two_ms * 1e3f;
     return 0;
 }
 
@@ -343,10 +438,10 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
         else if (want == 1 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk)) {
             const int pick = tune_get("gemm_skinny_config");             // 100 * variant + slices along K (tests)
             if (pick >= 0) c = SkinnyConfig{pick / 100, pick % 100};
-            else if (c.variant < 0) c = skinny_default(M, K, N, workspace_bytes);
+            else if (c.variant < 0) c = skinny_default(M, K, N, workspace_bytes, 1);
         }
         if (c.variant >= 0) {
-            const int rc = skinny_launch(c, x, w, y, M, K, N, ldy, workspace, workspace_bytes, st);
+            const int rc = skinny_launch(c, x, w, y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st);
             if (rc == 0) {
                 t_last_path = 2;
                 return 0;
@@ -370,4 +465,48 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
     t_last_path = 0;
     return dtype == ONELLM_FP16 ? run_plain<__half>(x, w, y, M, K, N, ldy, w_is_nk, st)
                                 : run_plain<float>(x, w, y, M, K, N, ldy, w_is_nk, st);
+}
+
+extern "C" int onellm_linear_pair(int dtype, const void* x, const void* w_first, const void* w_second, void* y_first, void* y_second,
+                                  int M, int K, int N, int ldy, int w_is_nk, void* workspace, size_t workspace_bytes,
+                                  onellm_stream_t stream)
+{
+    using namespace onellm;
+    if (dtype != ONELLM_FP32 && dtype != ONELLM_FP16) return ONELLM_EINVAL;
+    if (M < 0 || K <= 0 || N <= 0) return ONELLM_EINVAL;
+    if (ldy == 0) ldy = N;
+    if (ldy < N) return ONELLM_EINVAL;
+    if (M == 0) return 0;
+    if (!x || !w_first || !w_second || !y_first || !y_second) return ONELLM_EINVAL;
+    if (!workspace) workspace_bytes = 0;
+    if (workspace_bytes > kWorkspaceBytes) workspace_bytes = kWorkspaceBytes;
+    const int want = tune_get("gemm_skinny");
+    if (want != 0 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk)) {
+        SkinnyConfig c;
+        int dev = 0;
+        const hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return (int)e;
+        {
+            std::lock_guard<std::mutex> g(g_mu);
+            auto it = g_pair_plans.find(std::make_tuple(dev, M, K, N, ldy, workspace_bytes ? 1 : 0));
+            if (it != g_pair_plans.end()) c = it->second;
+        }
+        if (want == 1) {
+            const int pick = tune_get("gemm_skinny_config");
+            if (pick >= 0) c = SkinnyConfig{pick / 100, pick % 100};
+            else if (c.variant < 0) c = skinny_default(M, K, N, workspace_bytes, 2);
+        }
+        if (c.variant >= 0) {
+            const int rc = skinny_launch(c, x, w_first, y_first, w_second, y_second, M, K, N, ldy, workspace, workspace_bytes,
+                                         static_cast<hipStream_t>(stream));
+            if (rc == 0) {
+                t_last_path = 3;
+                return 0;
+            }
+            if (rc != ONELLM_EUNSUPPORTED) return rc;
+        }
+    }
+    const int rc = onellm_linear(dtype, x, w_first, y_first, M, K, N, ldy, w_is_nk, workspace, workspace_bytes, stream);
+    if (rc != 0) return rc;
+    return onellm_linear(dtype, x, w_second, y_second, M, K, N, ldy, w_is_nk, workspace, workspace_bytes, stream);
 }

@@ -45,6 +45,8 @@ struct SkinnyArgs {
     const void* x;
     const void* w;
     void* y;
+    const void* w_second;                    // a launch of two problems that share x and shape (grid.z = 2): the other W and y
+    void* y_second;
     float* partial;                          // [panels][splits][rows][NT]
     unsigned* counters;                      // [panels]
     int M, K, N, ldy, splits;
@@ -78,13 +80,15 @@ void skinny_gemm_kernel(const SkinnyArgs a)
     constexpr int ROWS = MT * 16;
     constexpr int NTHR = NW * kWave;
     const int panel = blockIdx.x, split = blockIdx.y;
+    const bool second = blockIdx.z != 0;
+    const int slot = second ? gridDim.x + panel : panel;         // where this panel's partial sums and counter are
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int nl = lane & 15, kg = lane >> 4;
     const int n0 = panel * NT;
     const int nsb = a.K / kSuperBlock;
     const int sb0 = (int)((long long)nsb * split / a.splits), sb1 = (int)((long long)nsb * (split + 1) / a.splits);
-    const __amdgpu_buffer_rsrc_t rw = window(a.w, (unsigned)((size_t)a.K * a.N * 2));
+    const __amdgpu_buffer_rsrc_t rw = window(second ? a.w_second : a.w, (unsigned)((size_t)a.K * a.N * 2));
     const __amdgpu_buffer_rsrc_t rx = window(a.x, (unsigned)((size_t)a.M * a.K * 2));
     // byte offsets of this lane inside super-block 0; a column past N reads the next row's start (or nothing, in the
     // last row) and its sums are dropped at the end, a row of x past M reads past the buffer, i.e. zeros
@@ -180,7 +184,7 @@ void skinny_gemm_kernel(const SkinnyArgs a)
         __shared__ int s_last;
         const __amdgpu_buffer_rsrc_t rp = window(a.partial, 0x7FFFFFFFu);
         const unsigned panel_bytes = (unsigned)(ROWS * NT * 4);
-        const unsigned mine = ((unsigned)panel * a.splits + split) * panel_bytes;
+        const unsigned mine = ((unsigned)slot * a.splits + split) * panel_bytes;
 #pragma unroll
         for (int p = 0; p < PER; ++p) {
             const int piece = p * NTHR + tid;
@@ -190,14 +194,14 @@ void skinny_gemm_kernel(const SkinnyArgs a)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0) {
-            const unsigned before = __hip_atomic_fetch_add(&a.counters[panel], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned before = __hip_atomic_fetch_add(&a.counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const int last = before == (unsigned)(a.splits - 1);
-            if (last) __hip_atomic_store(&a.counters[panel], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
+            if (last) __hip_atomic_store(&a.counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
             s_last = last;
         }
         __syncthreads();
         if (!s_last) return;
-        const unsigned all = (unsigned)panel * a.splits * panel_bytes;
+        const unsigned all = (unsigned)slot * a.splits * panel_bytes;
 #pragma unroll
         for (int p = 0; p < PER; ++p) {
             const int piece = p * NTHR + tid;
@@ -224,7 +228,7 @@ void skinny_gemm_kernel(const SkinnyArgs a)
         const int m = piece / (NT / 4), n = n0 + 4 * (piece % (NT / 4));
         if (piece < PIECES && m < a.M && n < a.N) {
             const f16x4 o = {(_Float16)sum[p][0], (_Float16)sum[p][1], (_Float16)sum[p][2], (_Float16)sum[p][3]};
-            *reinterpret_cast<f16x4*>(reinterpret_cast<_Float16*>(a.y) + (size_t)m * a.ldy + n) = o;
+            *reinterpret_cast<f16x4*>(reinterpret_cast<_Float16*>(second ? a.y_second : a.y) + (size_t)m * a.ldy + n) = o;
         }
     }
 }
@@ -251,16 +255,16 @@ const Variant g_variants[] = {
 constexpr int kVariants = (int)(sizeof(g_variants) / sizeof(g_variants[0]));
 
 int panels_of(const Variant& v, int N) { return (N + v.nt - 1) / v.nt; }
-size_t partial_bytes(const Variant& v, int splits, int N)
+size_t partial_bytes(const Variant& v, int splits, int N, int problems)
 {
-    return splits > 1 ? (size_t)panels_of(v, N) * splits * v.mt * 16 * v.nt * sizeof(float) : 0;
+    return splits > 1 ? (size_t)problems * panels_of(v, N) * splits * v.mt * 16 * v.nt * sizeof(float) : 0;
 }
-bool config_fits(const Variant& v, int splits, int M, int K, int N, size_t ws_bytes)
+bool config_fits(const Variant& v, int splits, int M, int K, int N, size_t ws_bytes, int problems)
 {
     if (M > v.mt * 16 || (v.mt == 2 && M <= 16)) return false;
     if (splits < 1 || splits > K / kSuperBlock) return false;
-    if (panels_of(v, N) > kCounterPanels) return false;
-    const size_t need = partial_bytes(v, splits, N);
+    if (problems * panels_of(v, N) > kCounterPanels) return false;
+    const size_t need = partial_bytes(v, splits, N, problems);
     return need <= ws_bytes && need < (1u << 30);
 }
 
@@ -316,30 +320,30 @@ bool skinny_shape_ok(int dtype, int M, int K, int N, int ldy, int w_is_nk)
     return true;
 }
 
-int skinny_candidates(int M, int K, int N, size_t ws_bytes, SkinnyConfig* out, int max)
+int skinny_candidates(int M, int K, int N, size_t ws_bytes, int problems, SkinnyConfig* out, int max)
 {
     static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16};
     int n = 0;
     for (int v = 0; v < kVariants; ++v)
         for (int s : kSplits) {
-            if (!config_fits(g_variants[v], s, M, K, N, ws_bytes)) continue;
-            const long long panels = panels_of(g_variants[v], N);
+            if (!config_fits(g_variants[v], s, M, K, N, ws_bytes, problems)) continue;
+            const long long panels = (long long)problems * panels_of(g_variants[v], N);
             if (s > 1 && (panels * s > 2048 || panels >= 1024)) continue;   // slicing is for problems that do not fill the chip
             if (n < max) out[n++] = SkinnyConfig{v, s};
         }
     return n;
 }
 
-SkinnyConfig skinny_default(int M, int K, int N, size_t ws_bytes)
+SkinnyConfig skinny_default(int M, int K, int N, size_t ws_bytes, int problems)
 {
     SkinnyConfig best;
     long long best_gap = 0;
     SkinnyConfig cand[64];
-    const int n = skinny_candidates(M, K, N, ws_bytes, cand, 64);
+    const int n = skinny_candidates(M, K, N, ws_bytes, problems, cand, 64);
     for (int i = 0; i < n; ++i) {
         const Variant& v = g_variants[cand[i].variant];
         if (v.nt != 64 || (cand[i].variant != 0 && cand[i].variant != 4)) continue;       // the 64-column, two-stage form
-        long long gap = (long long)panels_of(v, N) * cand[i].splits - 256;
+        long long gap = (long long)problems * panels_of(v, N) * cand[i].splits - 256;
         if (gap < 0) gap = -gap;
         if (best.variant < 0 || gap < best_gap) {
             best = cand[i];
@@ -350,17 +354,20 @@ SkinnyConfig skinny_default(int M, int K, int N, size_t ws_bytes)
     return best;
 }
 
-int skinny_launch(SkinnyConfig c, const void* x, const void* w, void* y, int M, int K, int N, int ldy, void* workspace,
-                  size_t workspace_bytes, hipStream_t stream)
+int skinny_launch(SkinnyConfig c, const void* x, const void* w, void* y, const void* w_second, void* y_second, int M, int K, int N,
+                  int ldy, void* workspace, size_t workspace_bytes, hipStream_t stream)
 {
     if (ldy == 0) ldy = N;
     if (c.variant < 0 || c.variant >= kVariants || !skinny_shape_ok(ONELLM_FP16, M, K, N, ldy, 0)) return ONELLM_EUNSUPPORTED;
     const Variant& v = g_variants[c.variant];
+    const int problems = w_second ? 2 : 1;
     if (!workspace) workspace_bytes = 0;
-    if (!config_fits(v, c.splits, M, K, N, workspace_bytes)) return ONELLM_EUNSUPPORTED;
+    if (!config_fits(v, c.splits, M, K, N, workspace_bytes, problems)) return ONELLM_EUNSUPPORTED;
     if (!aligned(x, 16) || !aligned(w, 16) || !aligned(y, 8)) return ONELLM_EUNSUPPORTED;
+    if (w_second && (!y_second || !aligned(w_second, 16) || !aligned(y_second, 8))) return ONELLM_EUNSUPPORTED;
     SkinnyArgs a{};
     a.x = x; a.w = w; a.y = y;
+    a.w_second = w_second; a.y_second = y_second;
     a.M = M; a.K = K; a.N = N; a.ldy = ldy; a.splits = c.splits;
     if (c.splits > 1) {
         if (!aligned(workspace, 16)) return ONELLM_EUNSUPPORTED;
@@ -372,7 +379,7 @@ int skinny_launch(SkinnyConfig c, const void* x, const void* w, void* y, int M, 
         a.partial = static_cast<float*>(workspace);
         a.counters = counters + (size_t)set * kCounterPanels;
     }
-    v.launch(a, dim3(panels_of(v, N), c.splits), stream);
+    v.launch(a, dim3(panels_of(v, N), c.splits, problems), stream);
     return (int)hipGetLastError();
 }
 

@@ -51,8 +51,8 @@ def test_gemm_library_exports_what_its_header_declares(G):
     text = open(os.path.join(ROOT, "include", "onellm_gemm.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = sorted(set(re.findall(r"\b(onellm_[a-z0-9_]+)\s*\(", text)))
-    assert names == ["onellm_linear", "onellm_linear_allow_plain", "onellm_linear_last_path", "onellm_linear_tune",
-                     "onellm_linear_workspace_bytes"]
+    assert names == ["onellm_linear", "onellm_linear_allow_plain", "onellm_linear_last_path", "onellm_linear_pair",
+                     "onellm_linear_pair_tune", "onellm_linear_tune", "onellm_linear_workspace_bytes"]
     for n in names:
         assert hasattr(G, n)
     assert G.onellm_linear_workspace_bytes() > 0
@@ -182,6 +182,58 @@ def test_few_row_kernel_matches_the_oracle_in_every_configuration(G, ref, M, K, 
         capi.tune_set("gemm_skinny_config", -1)
     assert len(ran) >= 3, ran
     assert any(s > 1 for _, s in ran) or K < 128, ran
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N", [(16, 4096, 11008), (5, 256, 72), (20, 512, 200)])
+def test_pair_of_projections_in_one_launch_matches_two_calls_and_the_oracle(G, ref, M, K, N):
+    """onellm_linear_pair (the gate / up projections into the [M, 2, N] buffer the SwiGLU kernel reads): forced through
+    the one-launch configurations, both halves match the oracle and are bit-identical to two onellm_linear calls
+    with the same configuration; after a tuning run the chosen form still matches."""
+    import torch
+    from onellm_amd import capi
+    announce("linear pair", M, K, N)
+    rng = np.random.default_rng(N + M)
+    x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
+    w0 = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    w1 = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    want0, want1 = ref.linear(x, w0).astype(np.float64), ref.linear(x, w1).astype(np.float64)
+    dx, d0, d1 = _dev(torch, x), _dev(torch, w0), _dev(torch, w1)
+    ws = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dx.device)
+
+    def run_pair():
+        pair = torch.full((M, 2, N), float("nan"), dtype=torch.float16, device=dx.device)
+        capi.linear_pair(dx, d0, d1, pair, pair.view(-1)[N:], ldy=2 * N, workspace=ws)
+        torch.cuda.synchronize()
+        return pair.cpu().numpy()
+
+    ran = 0
+    capi.tune_set("gemm_skinny", 1)
+    try:
+        for variant in range(7):
+            for splits in (1, 2, 4, 8):
+                capi.tune_set("gemm_skinny_config", 100 * variant + splits)
+                got = run_pair()
+                if G.onellm_linear_last_path() != 3:
+                    continue
+                ran += 1
+                np.testing.assert_allclose(got[:, 0].astype(np.float64), want0, err_msg=str((variant, splits)), **TOL[np.float16])
+                np.testing.assert_allclose(got[:, 1].astype(np.float64), want1, err_msg=str((variant, splits)), **TOL[np.float16])
+                two = torch.full((M, 2, N), float("nan"), dtype=torch.float16, device=dx.device)
+                capi.linear(dx, d0, two, ldy=2 * N, workspace=ws)
+                capi.linear(dx, d1, two.view(-1)[N:], ldy=2 * N, workspace=ws)
+                torch.cuda.synchronize()
+                assert G.onellm_linear_last_path() == 2
+                assert np.array_equal(got, two.cpu().numpy()), (variant, splits)
+    finally:
+        capi.tune_set("gemm_skinny", -1)
+        capi.tune_set("gemm_skinny_config", -1)
+    assert ran >= 3
+    best, two_calls = capi.linear_pair_tune(capi.FP16, M, K, N, ldy=2 * N, workspace=ws)
+    assert 0 < best <= two_calls
+    got = run_pair()
+    np.testing.assert_allclose(got[:, 0].astype(np.float64), want0, **TOL[np.float16])
+    np.testing.assert_allclose(got[:, 1].astype(np.float64), want1, **TOL[np.float16])
 
 
 @pytest.mark.gpu
