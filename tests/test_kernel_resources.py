@@ -12,7 +12,8 @@ import pytest
 
 from onellm_amd import build
 
-SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip", "sampling.hip"]
+SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip", "sampling.hip",
+           "skinny_gemm.hip"]
 
 
 @pytest.fixture(scope="module")
@@ -69,3 +70,13 @@ def test_streaming_kernels_keep_full_occupancy(resources):
         assert r["occupancy"] >= 4 and r["vgprs"] <= 64, (name, r)
     for name, r in _matching(resources["prefill_rope.hip"], r"rows_kernel").items():
         assert r["occupancy"] >= 4, (name, r)
+
+
+def test_few_row_gemm_keeps_two_workgroups_per_compute_unit(resources):
+    # the projection kernel's variants up to 16 rows: one stage of 128 columns or two of 64 leave room for two 4-wave
+    # workgroups per CU (the cut runs launch 256-768 of them); the two-stage 128-column form is the one-per-CU variant
+    res = resources["skinny_gemm.hip"]
+    for name, r in _matching(res, r"skinny_gemm_kernelILi1ELi(1ELi4ELi8|2ELi4ELi4|1ELi4ELi4)E").items():
+        assert r["occupancy"] >= 2, (name, r)
+    for name, r in res.items():
+        assert r["vgprs"] + r["agprs"] <= 512 and r["scratch"] == 0, (name, r)
