@@ -143,7 +143,8 @@ def test_linear_matches_the_oracle(H, G, ref, dtype, M, K, N):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,K,N,ldy", [(1, 64, 8, 0), (3, 128, 72, 0), (16, 4096, 4096, 0), (16, 11008, 4096, 0), (7, 4096, 12288, 0),
-                                       (16, 4096, 11008, 22016), (32, 4096, 4096, 0), (17, 256, 136, 140), (16, 1024, 200, 0)])
+                                       (16, 4096, 11008, 22016), (32, 4096, 4096, 0), (17, 256, 136, 140), (16, 1024, 200, 0),
+                                       (4, 4096, 32000, 0)])
 def test_few_row_kernel_matches_the_oracle_in_every_configuration(G, ref, M, K, N, ldy):
     """onellm_linear's own kernel for a decode step's rows, forced (tuning key gemm_skinny = 1) through every kernel
     variant and every number of slices along K that takes the problem: fp16 parity with the oracle, untouched
