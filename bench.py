@@ -373,6 +373,47 @@ def decoder_layer_section(capi, dev, args):
     return {"decoder_layer_llama7b_b16_ctx4096": e}
 
 
+def projections_section(capi, dev, steps):
+    """The four projections of a Llama-2-7B layer at batch 16 through onellm_linear / onellm_linear_pair, each over
+    enough different weight matrices that every launch meets its matrix cold: the tuned plan as it is (hipBLASLt or the
+    repository's few-row kernel, whichever the tuning run found faster) and, beside it, hipBLASLt's best algorithm
+    alone (tuning key gemm_skinny = 0).  Algorithmic bytes = the weights."""
+    import torch
+    M, hid, I = 16, 4096, 11008
+    ws = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dev)
+    path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel", 3: "own few-row kernel, both in one launch"}
+    out = {}
+    for name, K, N, pair in (("qkv", hid, 3 * hid, False), ("out", hid, hid, False), ("gate_up_pair", hid, I, True), ("down", I, hid, False)):
+        w_bytes = 2 * K * N * (2 if pair else 1)
+        n = max(2, min(16, -(-(640 << 20) // (2 * K * N)))) & ~1
+        x = torch.randn(M, K, device=dev).mul_(0.5).half()
+        wts = [torch.randn(K, N, device=dev).mul_(K ** -0.5).half() for _ in range(n)]
+        y = torch.empty(M, 2, N, dtype=torch.float16, device=dev)
+        ld = 2 * N if pair else 0
+
+        def step(i):
+            if pair:
+                capi.linear_pair(x, wts[(2 * i) % n], wts[(2 * i + 1) % n], y, y.view(-1)[N:], ldy=ld, workspace=ws)
+            else:
+                capi.linear(x, wts[i % n], y.view(-1)[:M * N].view(M, N), workspace=ws)
+
+        res = {}
+        for label, knob in (("hipblaslt", 0), ("tuned", -1)):
+            capi.tune_set("gemm_skinny", knob)
+            (capi.linear_pair_tune if pair else capi.linear_tune)(capi.FP16, M, K, N, ldy=ld, workspace=ws)
+            ms = time_steps_graph(step, per_graph=2 * n, replays=max(steps // (2 * n), 5))
+            res[label] = (ms, path_names.get(capi.gemm_lib().onellm_linear_last_path(), "?"))
+        capi.tune_set("gemm_skinny", -1)
+        e = entry(res["tuned"][0], w_bytes)
+        e["path"] = res["tuned"][1]
+        e["us_hipblaslt_alone"] = round(res["hipblaslt"][0] * 1e3, 2)
+        e["weight_sets"] = n
+        out["linear_m16_%s_%dx%d" % (name, K, N)] = e
+        del wts
+        torch.cuda.empty_cache()
+    return out
+
+
 def ceilings_section(dev, steps, warmup):
     """What this GPU's memory system delivers for the access mix of each product kernel: bare kernels with the same
     access shapes and no arithmetic (tests/cpp/access_ceilings.hip), timed exactly like the kernels themselves -
@@ -510,6 +551,7 @@ def extras_section(capi, dev, args, with_cpu):
     del rk, rv, kc, vc, qkv, bias, qkv_r, ws
     torch.cuda.empty_cache()
 
+    ex.update(projections_section(capi, dev, args.steps))
     ex.update(decoder_layer_section(capi, dev, args))
     torch.cuda.empty_cache()
 
