@@ -33,7 +33,7 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 constexpr int kSuperBlock = 64;              // rows of W one wave multiplies per step
-constexpr int kCounterSets = 32;             // workspaces that can run sliced at the same time
+constexpr int kCounterSets = 128;            // workspaces that can run sliced at the same time
 constexpr int kCounterPanels = 2048;         // column panels per call
 __device__ unsigned g_slice_arrivals[kCounterSets * kCounterPanels];
 
@@ -268,18 +268,29 @@ bool config_fits(const Variant& v, int splits, int M, int K, int N, size_t ws_by
     return need <= ws_bytes && need < (1u << 30);
 }
 
-// the counter set of a workspace; -1: none left
+// The counter set of a workspace.  A set belongs to the workspace that used it last; when all are taken the one unused
+// for longest changes hands - its counters are zero between calls, and the workspace it served would have to be in the
+// middle of a call while kCounterSets others take their turn for that to matter.
 int counter_set_of(const void* workspace)
 {
     static std::mutex m;
     static const void* owner[kCounterSets];
+    static unsigned long long last_use[kCounterSets];
+    static unsigned long long clock = 0;
     static int used = 0;
     std::lock_guard<std::mutex> lock(m);
-    for (int i = 0; i < used; ++i)
-        if (owner[i] == workspace) return i;
-    if (used == kCounterSets) return -1;
-    owner[used] = workspace;
-    return used++;
+    int set = -1;
+    for (int i = 0; i < used && set < 0; ++i)
+        if (owner[i] == workspace) set = i;
+    if (set < 0 && used < kCounterSets) set = used++;
+    if (set < 0) {
+        set = 0;
+        for (int i = 1; i < kCounterSets; ++i)
+            if (last_use[i] < last_use[set]) set = i;
+    }
+    owner[set] = workspace;
+    last_use[set] = ++clock;
+    return set;
 }
 
 // this device's copy of the counters (every device has its own, at its own address)
@@ -372,7 +383,6 @@ int skinny_launch(SkinnyConfig c, const void* x, const void* w, void* y, const v
     if (c.splits > 1) {
         if (!aligned(workspace, 16)) return ONELLM_EUNSUPPORTED;
         const int set = counter_set_of(workspace);
-        if (set < 0) return ONELLM_EUNSUPPORTED;
         unsigned* counters = nullptr;
         const int rc = device_counters(&counters);
         if (rc != 0) return rc;

@@ -27,7 +27,7 @@ int skinny_candidates(int M, int K, int N, size_t with_workspace_bytes, int prob
 SkinnyConfig skinny_default(int M, int K, int N, size_t with_workspace_bytes, int problems);
 
 // Queues the multiplication.  0, ONELLM_EUNSUPPORTED (this kernel does not take the problem as given: alignment,
-// workspace too small, no counter set left for a sliced run - the caller goes on to the library) or a hipError_t.
+// workspace too small for a sliced run - the caller goes on to the library) or a hipError_t.
 // A sliced run (splits > 1) uses `workspace` for partial sums; calls that share a workspace must not overlap, which
 // is the library's rule for the same buffer as well.
 // With w_second / y_second the launch also computes y_second = x . w_second (same shape and row stride): the gate and
