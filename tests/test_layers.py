@@ -238,6 +238,57 @@ def test_pair_of_projections_in_one_launch_matches_two_calls_and_the_oracle(G, r
 
 
 @pytest.mark.gpu
+def test_few_row_kernel_cut_runs_back_to_back_on_one_workspace(G, ref):
+    """300 cut runs of mixed shapes and configurations queued back to back on one workspace (its partial sums and
+    arrival counters are reused from launch to launch with nothing in between but stream order), then every output
+    compared bit for bit with what the same (shape, configuration) gave when it ran alone, which in turn matches the
+    oracle."""
+    import torch
+    from onellm_amd import capi
+    announce("few-row linear, back to back")
+    rng = np.random.default_rng(11)
+    dev = torch.device("cuda:0")
+    ws = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dev)
+    shapes = [(16, 1024, 512), (8, 2048, 1024), (16, 4096, 4096), (32, 512, 256), (3, 4096, 1536)]
+    ops = []
+    for M, K, N in shapes:
+        x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
+        w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+        ops.append((M, K, N, _dev(torch, x), _dev(torch, w), ref.linear(x, w).astype(np.float64)))
+    capi.tune_set("gemm_skinny", 1)
+    try:
+        alone = {}
+        for si, (M, K, N, dx, dw, want) in enumerate(ops):
+            for variant in range(7):
+                for splits in (2, 3, 4, 8):
+                    capi.tune_set("gemm_skinny_config", 100 * variant + splits)
+                    y = torch.zeros((M, N), dtype=torch.float16, device=dev)
+                    capi.linear(dx, dw, y, workspace=ws)
+                    torch.cuda.synchronize()
+                    if G.onellm_linear_last_path() != 2:
+                        continue
+                    got = y.cpu().numpy()
+                    np.testing.assert_allclose(got.astype(np.float64), want, **TOL[np.float16])
+                    alone[(si, variant, splits)] = got
+        keys = sorted(alone)
+        assert len(keys) >= 40, len(keys)
+        order = [keys[i] for i in rng.integers(0, len(keys), size=300)]
+        outs = []
+        for si, variant, splits in order:
+            M, K, N, dx, dw, _ = ops[si]
+            capi.tune_set("gemm_skinny_config", 100 * variant + splits)
+            y = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+            capi.linear(dx, dw, y, workspace=ws)
+            outs.append(y)
+        torch.cuda.synchronize()
+        for k, y in zip(order, outs):
+            assert np.array_equal(y.cpu().numpy(), alone[k]), k
+    finally:
+        capi.tune_set("gemm_skinny", -1)
+        capi.tune_set("gemm_skinny_config", -1)
+
+
+@pytest.mark.gpu
 def test_few_row_kernel_declines_what_it_is_not_built_for(G, ref):
     """Forced or not, a problem outside the kernel's rules (fp32, W as [N, K], too many rows, K not in whole
     64-row blocks, N or the row stride not in whole pieces, a misaligned operand) runs the library as before."""
