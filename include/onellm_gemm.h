@@ -3,10 +3,10 @@
  * Replaces launchLinearGemm (src/kernels/qkv_linear.cu:8-66, declared src/kernels/qkv_linear.h:9-14) and the
  * cublasWrapper::Gemm call under it (src/kernels/cublas_wrapper.cc:33-85).  The multiplication itself is a library
  * GEMM (hipBLASLt, fp32 accumulation); this entry point adds what the reference re-creates on every call: a handle
- * per device and a cached plan per (dtype, M, K, N, layout).  For the few rows of a decode step (fp16, W as [K, N],
- * M <= 32, K a multiple of 64, N of 8) the library also holds a kernel of its own that streams the weights once
- * through the matrix cores; onellm_linear_tune times it beside the library's algorithms and onellm_linear runs
- * whichever won.  Small shapes the library has no kernel for (unit-test and example-driver sizes, up to 2^24
+ * per device and a cached plan per (dtype, M, K, N, layout).  For the few rows of a decode step (fp16 or fp32, W as
+ * [K, N], M <= 32, K a multiple of 64, rows of W in whole 16-byte pieces) the library also holds a kernel of its own
+ * that streams the weights once through the matrix cores; onellm_linear_tune times it beside the library's
+ * algorithms and onellm_linear runs whichever won.  Small shapes the library has no kernel for (unit-test and example-driver sizes, up to 2^24
  * multiply-adds) run a plain kernel in this library; a larger one returns ONELLM_ENOGEMMKERNEL unless the caller has
  * allowed the plain kernel, which is about a hundred times slower.
  *

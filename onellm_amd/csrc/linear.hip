@@ -263,7 +263,7 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
     constexpr int kWantOwn = 64;
     SkinnyConfig own[kWantOwn];
     const int n_own = (tune_get("gemm_skinny") != 0 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk))
-                          ? skinny_candidates(M, K, N, workspace_bytes, 1, own, kWantOwn) : 0;
+                          ? skinny_candidates(dtype, M, K, N, workspace_bytes, 1, own, kWantOwn) : 0;
     if (n == 0 && n_own == 0) {
         destroy_plan(p);
         return ONELLM_EUNSUPPORTED;
@@ -292,7 +292,7 @@ extern "C" int onellm_linear_tune(int dtype, int M, int K, int N, int ldy, int w
                 if (i < n)
                     return hipblasLtMatmul(handle, p.desc, &alpha, wc, p.la, rig.x, p.lb, &beta, rig.y, p.lc, rig.y, p.lc, &cand[i].algo,
                                            workspace, workspace_bytes, st) == HIPBLAS_STATUS_SUCCESS;
-                return skinny_launch(own[i - n], rig.x, wc, rig.y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st) == 0;
+                return skinny_launch(own[i - n], dtype, rig.x, wc, rig.y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st) == 0;
             }, runs, st, rc);
             if (ms < 0.f) continue;
             if (i == 0) first_ms = ms;
@@ -348,7 +348,7 @@ extern "C" int onellm_linear_pair_tune(int dtype, int M, int K, int N, int ldy, 
     constexpr int kWantOwn = 64;
     SkinnyConfig own[kWantOwn];
     const int n_own = (tune_get("gemm_skinny") != 0 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk))
-                          ? skinny_candidates(M, K, N, workspace_bytes, 2, own, kWantOwn) : 0;
+                          ? skinny_candidates(dtype, M, K, N, workspace_bytes, 2, own, kWantOwn) : 0;
     const size_t esz = dtype == ONELLM_FP16 ? 2 : 4;
     float two_ms = -1.f, best_ms = -1.f;
     SkinnyConfig chosen;
@@ -369,7 +369,7 @@ extern "C" int onellm_linear_pair_tune(int dtype, int M, int K, int N, int ldy, 
         for (int i = 0; i < n_own && rc == 0; ++i) {
             const float ms = rig.time([&](int r) {
                 const void *w0 = rig.w[(2 * r) % rig.copies], *w1 = rig.w[(2 * r + 1) % rig.copies];
-                return skinny_launch(own[i], rig.x, w0, rig.y, w1, y_second, M, K, N, ldy, workspace, workspace_bytes, st) == 0;
+                return skinny_launch(own[i], dtype, rig.x, w0, rig.y, w1, y_second, M, K, N, ldy, workspace, workspace_bytes, st) == 0;
             }, runs, st, rc);
             if (ms >= 0.f && ms < 0.97f * two_ms && ms < best_ms) {
                 best_ms = ms;
@@ -438,10 +438,10 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
         else if (want == 1 && skinny_shape_ok(dtype, M, K, N, ldy, w_is_nk)) {
             const int pick = tune_get("gemm_skinny_config");             // 100 * variant + slices along K (tests)
             if (pick >= 0) c = SkinnyConfig{pick / 100, pick % 100};
-            else if (c.variant < 0) c = skinny_default(M, K, N, workspace_bytes, 1);
+            else if (c.variant < 0) c = skinny_default(dtype, M, K, N, workspace_bytes, 1);
         }
         if (c.variant >= 0) {
-            const int rc = skinny_launch(c, x, w, y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st);
+            const int rc = skinny_launch(c, dtype, x, w, y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st);
             if (rc == 0) {
                 t_last_path = 2;
                 return 0;
@@ -494,10 +494,10 @@ extern "C" int onellm_linear_pair(int dtype, const void* x, const void* w_first,
         if (want == 1) {
             const int pick = tune_get("gemm_skinny_config");
             if (pick >= 0) c = SkinnyConfig{pick / 100, pick % 100};
-            else if (c.variant < 0) c = skinny_default(M, K, N, workspace_bytes, 2);
+            else if (c.variant < 0) c = skinny_default(dtype, M, K, N, workspace_bytes, 2);
         }
         if (c.variant >= 0) {
-            const int rc = skinny_launch(c, x, w_first, y_first, w_second, y_second, M, K, N, ldy, workspace, workspace_bytes,
+            const int rc = skinny_launch(c, dtype, x, w_first, y_first, w_second, y_second, M, K, N, ldy, workspace, workspace_bytes,
                                          static_cast<hipStream_t>(stream));
             if (rc == 0) {
                 t_last_path = 3;

@@ -1,4 +1,5 @@
-// y[M, N] = x[M, K] . W[K, N] with M <= 32: the projections of a decode step.  fp16 operands, fp32 accumulation.
+// y[M, N] = x[M, K] . W[K, N] with M <= 32: the projections of a decode step.  fp16 operands (fp32 ones further
+// down), fp32 accumulation.
 //
 // With so few rows the multiplication is a stream over the weights: every byte of W is read once and meets all M rows
 // of x, so the kernel is bound by how fast the compute units can pull W, and everything else is arranged around that.
@@ -70,6 +71,89 @@ template <> struct WeightPiece<8> {
     __device__ __forceinline__ unsigned pair(int i) const { return v[i]; }
 };
 
+// What follows the waves' tiles in LDS (lds[wave][row][column], ROWS x NT floats per wave): their sum, the hand-over
+// between the slices of a cut run, and the rows of y.  OUT is the element type of y.
+template <typename OUT, int ROWS, int NT, int NW>
+__device__ __forceinline__ void finish_tile(const SkinnyArgs& a, const float* lds, int tid, int n0, int slot, int split, bool second)
+{
+    constexpr int NTHR = NW * kWave;
+    __syncthreads();
+    // a thread owns pieces of four consecutive columns of one row
+    constexpr int PIECES = ROWS * NT / 4, PER = (PIECES + NTHR - 1) / NTHR;
+    f32x4 sum[PER];
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+        const int piece = p * NTHR + tid;
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        if (piece < PIECES) {
+#pragma unroll
+            for (int wv = 0; wv < NW; ++wv) s = s + *reinterpret_cast<const f32x4*>(&lds[wv * ROWS * NT + piece * 4]);
+        }
+        sum[p] = s;
+    }
+
+    if (a.splits > 1) {
+        // Every slice writes its sums with device-scope stores, waits until they are acknowledged and adds one to the
+        // panel's counter; the one that finds all others there reads them back with device-scope loads.  The stores
+        // are written through to memory before the wait ends and the add executes at memory, so the reader's loads
+        // come after every other slice's sums; nobody waits for anybody.
+        __shared__ int s_last;
+        const __amdgpu_buffer_rsrc_t rp = window(a.partial, 0x7FFFFFFFu);
+        const unsigned panel_bytes = (unsigned)(ROWS * NT * 4);
+        const unsigned mine = ((unsigned)slot * a.splits + split) * panel_bytes;
+#pragma unroll
+        for (int p = 0; p < PER; ++p) {
+            const int piece = p * NTHR + tid;
+            if (piece < PIECES)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sum[p]), rp, mine + piece * 16, 0, kDeviceScope);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned before = __hip_atomic_fetch_add(&a.counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = before == (unsigned)(a.splits - 1);
+            if (last) __hip_atomic_store(&a.counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
+            s_last = last;
+        }
+        __syncthreads();
+        if (!s_last) return;
+        const unsigned all = (unsigned)slot * a.splits * panel_bytes;
+#pragma unroll
+        for (int p = 0; p < PER; ++p) {
+            const int piece = p * NTHR + tid;
+            f32x4 s = {0.f, 0.f, 0.f, 0.f};
+            if (piece < PIECES) {
+                for (int s0 = 0; s0 < a.splits; s0 += 4) {
+                    f32x4 t[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int sp = min(s0 + j, a.splits - 1);
+                        t[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, all + sp * panel_bytes + piece * 16, 0, kDeviceScope));
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (s0 + j < a.splits) s = s + t[j];
+                }
+            }
+            sum[p] = s;
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+        const int piece = p * NTHR + tid;
+        const int m = piece / (NT / 4), n = n0 + 4 * (piece % (NT / 4));
+        if (piece < PIECES && m < a.M && n < a.N) {
+            void* y = second ? a.y_second : a.y;
+            if constexpr (sizeof(OUT) == 2) {
+                const f16x4 o = {(_Float16)sum[p][0], (_Float16)sum[p][1], (_Float16)sum[p][2], (_Float16)sum[p][3]};
+                *reinterpret_cast<f16x4*>(static_cast<_Float16*>(y) + (size_t)m * a.ldy + n) = o;
+            } else {
+                *reinterpret_cast<f32x4*>(static_cast<float*>(y) + (size_t)m * a.ldy + n) = sum[p];
+            }
+        }
+    }
+}
+
 // MT: tiles of 16 rows of x; U: super-blocks a wave has in flight; NW: waves; CPL: columns per lane
 template <int MT, int U, int NW, int CPL>
 __global__ __launch_bounds__(NW * kWave)
@@ -78,7 +162,6 @@ void skinny_gemm_kernel(const SkinnyArgs a)
     extern __shared__ float lds[];
     constexpr int NT = 16 * CPL;
     constexpr int ROWS = MT * 16;
-    constexpr int NTHR = NW * kWave;
     const int panel = blockIdx.x, split = blockIdx.y;
     const bool second = blockIdx.z != 0;
     const int slot = second ? gridDim.x + panel : panel;         // where this panel's partial sums and counter are
@@ -161,80 +244,112 @@ void skinny_gemm_kernel(const SkinnyArgs a)
                 const f32x4 v = {acc[mt][4 * c4 + 0][r], acc[mt][4 * c4 + 1][r], acc[mt][4 * c4 + 2][r], acc[mt][4 * c4 + 3][r]};
                 *reinterpret_cast<f32x4*>(&lds[(wave * ROWS + mt * 16 + 4 * kg + r) * NT + CPL * nl + 4 * c4]) = v;
             }
-    __syncthreads();
-    // a thread owns pieces of four consecutive columns of one row
-    constexpr int PIECES = ROWS * NT / 4, PER = (PIECES + NTHR - 1) / NTHR;
-    f32x4 sum[PER];
-#pragma unroll
-    for (int p = 0; p < PER; ++p) {
-        const int piece = p * NTHR + tid;
-        f32x4 s = {0.f, 0.f, 0.f, 0.f};
-        if (piece < PIECES) {
-#pragma unroll
-            for (int wv = 0; wv < NW; ++wv) s = s + *reinterpret_cast<const f32x4*>(&lds[wv * ROWS * NT + piece * 4]);
-        }
-        sum[p] = s;
-    }
+    finish_tile<_Float16, ROWS, NT, NW>(a, lds, tid, n0, slot, split, second);
+}
 
-    if (a.splits > 1) {
-        // Every slice writes its sums with device-scope stores, waits until they are acknowledged and adds one to the
-        // panel's counter; the one that finds all others there reads them back with device-scope loads.  The stores
-        // are written through to memory before the wait ends and the add executes at memory, so the reader's loads
-        // come after every other slice's sums; nobody waits for anybody.
-        __shared__ int s_last;
-        const __amdgpu_buffer_rsrc_t rp = window(a.partial, 0x7FFFFFFFu);
-        const unsigned panel_bytes = (unsigned)(ROWS * NT * 4);
-        const unsigned mine = ((unsigned)slot * a.splits + split) * panel_bytes;
+// The same stream for fp32 weights (the reference's own element type) on v_mfma_f32_16x16x4_f32.  A lane loads CPL = 2
+// or 4 consecutive fp32 columns of the rows 16 kg .. 16 kg + 15 of a 64-row super-block (panels of 32 or 64 columns,
+// 128 or 256 contiguous bytes per row group); product t of a super-block takes row 16 kg + t from every row group as
+// its four k-values, so both operands are registers as loaded - x comes as row nl, columns 16 kg .. 16 kg + 15 - and
+// no gather is needed.  Sums, hand-over and output are the fp16 kernel's.
+// (The loaded registers are kept as float vectors and indexed as such: bit-casting one element of an integer vector to
+// float - __builtin_bit_cast(float, v[i]) - gave element 0 for every i with this compiler.)
+template <int CPL> struct WeightPiece32;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+template <> struct WeightPiece32<2> {
+    f32x2 v;
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off)
+    {
+        v = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, kStream));
+    }
+    __device__ __forceinline__ float column(int i) const { return v[i]; }
+};
+template <> struct WeightPiece32<4> {
+    f32x4 v;
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off)
+    {
+        v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, kStream));
+    }
+    __device__ __forceinline__ float column(int i) const { return v[i]; }
+};
+
+template <int MT, int U, int NW, int CPL>
+__global__ __launch_bounds__(NW * kWave)
+void skinny_gemm_f32_kernel(const SkinnyArgs a)
+{
+    extern __shared__ float lds[];
+    constexpr int NT = 16 * CPL;
+    constexpr int ROWS = MT * 16;
+    const int panel = blockIdx.x, split = blockIdx.y;
+    const bool second = blockIdx.z != 0;
+    const int slot = second ? gridDim.x + panel : panel;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int nl = lane & 15, kg = lane >> 4;
+    const int n0 = panel * NT;
+    const int nsb = a.K / kSuperBlock;
+    const int sb0 = (int)((long long)nsb * split / a.splits), sb1 = (int)((long long)nsb * (split + 1) / a.splits);
+    const __amdgpu_buffer_rsrc_t rw = window(second ? a.w_second : a.w, (unsigned)((size_t)a.K * a.N * 4));
+    const __amdgpu_buffer_rsrc_t rx = window(a.x, (unsigned)((size_t)a.M * a.K * 4));
+    const unsigned w_lane = (unsigned)((16 * kg) * a.N + n0 + CPL * nl) * 4u;
+    const unsigned w_row = (unsigned)a.N * 4u, w_sb = (unsigned)a.N * (4u * kSuperBlock);
+    const unsigned x_lane = (unsigned)(nl * a.K + 16 * kg) * 4u, x_tile = (unsigned)a.K * 64u;
+
+    f32x4 acc[MT][CPL];
 #pragma unroll
-        for (int p = 0; p < PER; ++p) {
-            const int piece = p * NTHR + tid;
-            if (piece < PIECES)
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sum[p]), rp, mine + piece * 16, 0, kDeviceScope);
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (tid == 0) {
-            const unsigned before = __hip_atomic_fetch_add(&a.counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int last = before == (unsigned)(a.splits - 1);
-            if (last) __hip_atomic_store(&a.counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
-            s_last = last;
-        }
-        __syncthreads();
-        if (!s_last) return;
-        const unsigned all = (unsigned)slot * a.splits * panel_bytes;
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int p = 0; p < PER; ++p) {
-            const int piece = p * NTHR + tid;
-            f32x4 s = {0.f, 0.f, 0.f, 0.f};
-            if (piece < PIECES) {
-                for (int s0 = 0; s0 < a.splits; s0 += 4) {
-                    f32x4 t[4];
+        for (int c = 0; c < CPL; ++c) acc[mt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    WeightPiece32<CPL> wr[U][16];
+    f32x4 xr[U][MT][4];
+    auto request = [&](int u, int sb) {
+        const bool in = sb < sb1;
+        const unsigned wo = w_lane + (unsigned)sb * w_sb;
+        const unsigned xo = x_lane + (unsigned)sb * (4u * kSuperBlock);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int sp = min(s0 + j, a.splits - 1);
-                        t[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, all + sp * panel_bytes + piece * 16, 0, kDeviceScope));
-                    }
+        for (int t = 0; t < 16; ++t) wr[u][t].load(rw, in ? wo + t * w_row : kNowhere);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (s0 + j < a.splits) s = s + t[j];
-                }
-            }
-            sum[p] = s;
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                xr[u][mt][q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, in ? xo + mt * x_tile + q * 16 : kNowhere, 0, 0));
+    };
+    int sb = sb0 + wave;
+#pragma unroll
+    for (int u = 0; u < U; ++u) request(u, sb + NW * u);
+    for (; sb < sb1; sb += NW * U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            WeightPiece32<CPL> wc[16];
+            f32x4 xc[MT][4];
+#pragma unroll
+            for (int t = 0; t < 16; ++t) wc[t] = wr[u][t];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) xc[mt][q] = xr[u][mt][q];
+            request(u, sb + NW * u + NW * U);
+#pragma unroll
+            for (int t = 0; t < 16; ++t)
+#pragma unroll
+                for (int c = 0; c < CPL; ++c)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(xc[mt][t / 4][t % 4], wc[t].column(c), acc[mt][c], 0, 0, 0);
         }
     }
 #pragma unroll
-    for (int p = 0; p < PER; ++p) {
-        const int piece = p * NTHR + tid;
-        const int m = piece / (NT / 4), n = n0 + 4 * (piece % (NT / 4));
-        if (piece < PIECES && m < a.M && n < a.N) {
-            const f16x4 o = {(_Float16)sum[p][0], (_Float16)sum[p][1], (_Float16)sum[p][2], (_Float16)sum[p][3]};
-            *reinterpret_cast<f16x4*>(reinterpret_cast<_Float16*>(second ? a.y_second : a.y) + (size_t)m * a.ldy + n) = o;
-        }
-    }
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) lds[(wave * ROWS + mt * 16 + 4 * kg + r) * NT + CPL * nl + c] = acc[mt][c][r];
+    finish_tile<float, ROWS, NT, NW>(a, lds, tid, n0, slot, split, second);
 }
 
 struct Variant {
-    int mt, nt, nw;
+    int dtype, mt, nt, nw;
     void (*launch)(const SkinnyArgs&, dim3, hipStream_t);
 };
 
@@ -245,12 +360,24 @@ void launch_variant(const SkinnyArgs& a, dim3 grid, hipStream_t st)
     hipLaunchKernelGGL((skinny_gemm_kernel<MT, U, NW, CPL>), grid, dim3(NW * kWave), lds_bytes, st, a);
 }
 
+template <int MT, int U, int NW, int CPL>
+void launch_variant_f32(const SkinnyArgs& a, dim3 grid, hipStream_t st)
+{
+    constexpr size_t lds_bytes = sizeof(float) * NW * MT * 16 * 16 * CPL;
+    hipLaunchKernelGGL((skinny_gemm_f32_kernel<MT, U, NW, CPL>), grid, dim3(NW * kWave), lds_bytes, st, a);
+}
+
 // up to 16 rows: 64-column panels with two super-blocks in flight or one, 128-column panels with one or two;
 // 17..32 rows: the same panels with two row tiles
+// fp32: 64-column panels with one super-block in flight, 32-column panels with two or one; the same with two row tiles
 const Variant g_variants[] = {
-    {1, 64, 4, launch_variant<1, 2, 4, 4>},  {1, 128, 4, launch_variant<1, 1, 4, 8>}, {1, 64, 4, launch_variant<1, 1, 4, 4>},
-    {1, 128, 4, launch_variant<1, 2, 4, 8>}, {2, 64, 4, launch_variant<2, 2, 4, 4>},  {2, 128, 4, launch_variant<2, 1, 4, 8>},
-    {2, 64, 4, launch_variant<2, 1, 4, 4>},
+    {ONELLM_FP16, 1, 64, 4, launch_variant<1, 2, 4, 4>},  {ONELLM_FP16, 1, 128, 4, launch_variant<1, 1, 4, 8>},
+    {ONELLM_FP16, 1, 64, 4, launch_variant<1, 1, 4, 4>},  {ONELLM_FP16, 1, 128, 4, launch_variant<1, 2, 4, 8>},
+    {ONELLM_FP16, 2, 64, 4, launch_variant<2, 2, 4, 4>},  {ONELLM_FP16, 2, 128, 4, launch_variant<2, 1, 4, 8>},
+    {ONELLM_FP16, 2, 64, 4, launch_variant<2, 1, 4, 4>},
+    {ONELLM_FP32, 1, 64, 4, launch_variant_f32<1, 1, 4, 4>}, {ONELLM_FP32, 1, 32, 4, launch_variant_f32<1, 2, 4, 2>},
+    {ONELLM_FP32, 1, 32, 4, launch_variant_f32<1, 1, 4, 2>}, {ONELLM_FP32, 2, 64, 4, launch_variant_f32<2, 1, 4, 4>},
+    {ONELLM_FP32, 2, 32, 4, launch_variant_f32<2, 2, 4, 2>},
 };
 constexpr int kVariants = (int)(sizeof(g_variants) / sizeof(g_variants[0]));
 
@@ -259,8 +386,9 @@ size_t partial_bytes(const Variant& v, int splits, int N, int problems)
 {
     return splits > 1 ? (size_t)problems * panels_of(v, N) * splits * v.mt * 16 * v.nt * sizeof(float) : 0;
 }
-bool config_fits(const Variant& v, int splits, int M, int K, int N, size_t ws_bytes, int problems)
+bool config_fits(const Variant& v, int dtype, int splits, int M, int K, int N, size_t ws_bytes, int problems)
 {
+    if (v.dtype != dtype) return false;
     if (M > v.mt * 16 || (v.mt == 2 && M <= 16)) return false;
     if (splits < 1 || splits > K / kSuperBlock) return false;
     if (problems * panels_of(v, N) > kCounterPanels) return false;
@@ -321,23 +449,24 @@ bool aligned(const void* p, size_t a) { return (reinterpret_cast<size_t>(p) & (a
 
 bool skinny_shape_ok(int dtype, int M, int K, int N, int ldy, int w_is_nk)
 {
-    if (dtype != ONELLM_FP16 || w_is_nk) return false;
+    if ((dtype != ONELLM_FP16 && dtype != ONELLM_FP32) || w_is_nk) return false;
+    const unsigned long long esz = dtype == ONELLM_FP16 ? 2 : 4;
     if (M < 1 || M > kSkinnyMaxRows) return false;
     if (K < kSuperBlock || K % kSuperBlock != 0) return false;       // whole super-blocks (a ragged one would multiply stray x by zero)
-    if (N < 8 || N % 8 != 0) return false;                           // 16-byte pieces of a weight row start aligned
+    if (N < 8 || (N * esz) % 16 != 0) return false;                  // 16-byte pieces of a weight row start aligned
     if (ldy == 0) ldy = N;
     if (ldy < N || ldy % 4 != 0) return false;                       // y is stored four columns at a time
-    if ((unsigned long long)K * N * 2 >= (1ull << 32) || (unsigned long long)M * K * 2 >= (1ull << 32)) return false;
+    if ((unsigned long long)K * N * esz >= (1ull << 32) || (unsigned long long)M * K * esz >= (1ull << 32)) return false;
     return true;
 }
 
-int skinny_candidates(int M, int K, int N, size_t ws_bytes, int problems, SkinnyConfig* out, int max)
+int skinny_candidates(int dtype, int M, int K, int N, size_t ws_bytes, int problems, SkinnyConfig* out, int max)
 {
     static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16};
     int n = 0;
     for (int v = 0; v < kVariants; ++v)
         for (int s : kSplits) {
-            if (!config_fits(g_variants[v], s, M, K, N, ws_bytes, problems)) continue;
+            if (!config_fits(g_variants[v], dtype, s, M, K, N, ws_bytes, problems)) continue;
             const long long panels = (long long)problems * panels_of(g_variants[v], N);
             if (s > 1 && (panels * s > 2048 || panels >= 1024)) continue;   // slicing is for problems that do not fill the chip
             if (n < max) out[n++] = SkinnyConfig{v, s};
@@ -345,15 +474,15 @@ int skinny_candidates(int M, int K, int N, size_t ws_bytes, int problems, Skinny
     return n;
 }
 
-SkinnyConfig skinny_default(int M, int K, int N, size_t ws_bytes, int problems)
+SkinnyConfig skinny_default(int dtype, int M, int K, int N, size_t ws_bytes, int problems)
 {
     SkinnyConfig best;
     long long best_gap = 0;
-    SkinnyConfig cand[64];
-    const int n = skinny_candidates(M, K, N, ws_bytes, problems, cand, 64);
+    SkinnyConfig cand[96];
+    const int n = skinny_candidates(dtype, M, K, N, ws_bytes, problems, cand, 96);
     for (int i = 0; i < n; ++i) {
         const Variant& v = g_variants[cand[i].variant];
-        if (v.nt != 64 || (cand[i].variant != 0 && cand[i].variant != 4)) continue;       // the 64-column, two-stage form
+        if (v.nt != 64) continue;                                        // the 64-column forms
         long long gap = (long long)problems * panels_of(v, N) * cand[i].splits - 256;
         if (gap < 0) gap = -gap;
         if (best.variant < 0 || gap < best_gap) {
@@ -365,17 +494,18 @@ SkinnyConfig skinny_default(int M, int K, int N, size_t ws_bytes, int problems)
     return best;
 }
 
-int skinny_launch(SkinnyConfig c, const void* x, const void* w, void* y, const void* w_second, void* y_second, int M, int K, int N,
-                  int ldy, void* workspace, size_t workspace_bytes, hipStream_t stream)
+int skinny_launch(SkinnyConfig c, int dtype, const void* x, const void* w, void* y, const void* w_second, void* y_second, int M, int K,
+                  int N, int ldy, void* workspace, size_t workspace_bytes, hipStream_t stream)
 {
     if (ldy == 0) ldy = N;
-    if (c.variant < 0 || c.variant >= kVariants || !skinny_shape_ok(ONELLM_FP16, M, K, N, ldy, 0)) return ONELLM_EUNSUPPORTED;
+    if (c.variant < 0 || c.variant >= kVariants || !skinny_shape_ok(dtype, M, K, N, ldy, 0)) return ONELLM_EUNSUPPORTED;
     const Variant& v = g_variants[c.variant];
     const int problems = w_second ? 2 : 1;
     if (!workspace) workspace_bytes = 0;
-    if (!config_fits(v, c.splits, M, K, N, workspace_bytes, problems)) return ONELLM_EUNSUPPORTED;
-    if (!aligned(x, 16) || !aligned(w, 16) || !aligned(y, 8)) return ONELLM_EUNSUPPORTED;
-    if (w_second && (!y_second || !aligned(w_second, 16) || !aligned(y_second, 8))) return ONELLM_EUNSUPPORTED;
+    if (!config_fits(v, dtype, c.splits, M, K, N, workspace_bytes, problems)) return ONELLM_EUNSUPPORTED;
+    const size_t y_align = dtype == ONELLM_FP16 ? 8 : 16;                 // four columns per store
+    if (!aligned(x, 16) || !aligned(w, 16) || !aligned(y, y_align)) return ONELLM_EUNSUPPORTED;
+    if (w_second && (!y_second || !aligned(w_second, 16) || !aligned(y_second, y_align))) return ONELLM_EUNSUPPORTED;
     SkinnyArgs a{};
     a.x = x; a.w = w; a.y = y;
     a.w_second = w_second; a.y_second = y_second;

@@ -1,5 +1,5 @@
-// y[M, N] = x[M, K] . W[K, N] for a handful of rows (a decode step's batch): fp16 operands, fp32 accumulation on the
-// matrix cores, the weights streamed once.  Host interface; the kernel is in skinny_gemm.hip.
+// y[M, N] = x[M, K] . W[K, N] for a handful of rows (a decode step's batch): fp16 or fp32 operands, fp32 accumulation
+// on the matrix cores, the weights streamed once.  Host interface; the kernel is in skinny_gemm.hip.
 // (internal to libonellm_gemm.so: onellm_linear and onellm_linear_tune are its callers)
 #pragma once
 #include <stddef.h>
@@ -21,10 +21,10 @@ bool skinny_shape_ok(int dtype, int M, int K, int N, int ldy, int w_is_nk);
 // Configurations worth timing for a problem - or for `problems` = 2 of them that share x and shape and go out in one
 // launch - `max` at most; with_workspace_bytes bounds the slices along K (a sliced run keeps its partial sums in the
 // caller's workspace).  Returns how many were written.
-int skinny_candidates(int M, int K, int N, size_t with_workspace_bytes, int problems, SkinnyConfig* out, int max);
+int skinny_candidates(int dtype, int M, int K, int N, size_t with_workspace_bytes, int problems, SkinnyConfig* out, int max);
 
 // A reasonable configuration without timing anything (what a forced run uses); variant -1 if there is none.
-SkinnyConfig skinny_default(int M, int K, int N, size_t with_workspace_bytes, int problems);
+SkinnyConfig skinny_default(int dtype, int M, int K, int N, size_t with_workspace_bytes, int problems);
 
 // Queues the multiplication.  0, ONELLM_EUNSUPPORTED (this kernel does not take the problem as given: alignment,
 // workspace too small for a sliced run - the caller goes on to the library) or a hipError_t.
@@ -32,7 +32,7 @@ SkinnyConfig skinny_default(int M, int K, int N, size_t with_workspace_bytes, in
 // is the library's rule for the same buffer as well.
 // With w_second / y_second the launch also computes y_second = x . w_second (same shape and row stride): the gate and
 // up projections of a feed-forward block in one go.
-int skinny_launch(SkinnyConfig c, const void* x, const void* w, void* y, const void* w_second, void* y_second, int M, int K, int N,
-                  int ldy, void* workspace, size_t workspace_bytes, hipStream_t stream);
+int skinny_launch(SkinnyConfig c, int dtype, const void* x, const void* w, void* y, const void* w_second, void* y_second, int M, int K,
+                  int N, int ldy, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 }  // namespace onellm

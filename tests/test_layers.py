@@ -142,19 +142,23 @@ def test_linear_matches_the_oracle(H, G, ref, dtype, M, K, N):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,K,N,ldy", [(1, 64, 8, 0), (3, 128, 72, 0), (16, 4096, 4096, 0), (16, 11008, 4096, 0), (7, 4096, 12288, 0),
-                                       (16, 4096, 11008, 22016), (32, 4096, 4096, 0), (17, 256, 136, 140), (16, 1024, 200, 0),
-                                       (4, 4096, 32000, 0)])
-def test_few_row_kernel_matches_the_oracle_in_every_configuration(G, ref, M, K, N, ldy):
+@pytest.mark.parametrize("dtype,M,K,N,ldy", [
+    (np.float16, 1, 64, 8, 0), (np.float16, 3, 128, 72, 0), (np.float16, 16, 4096, 4096, 0), (np.float16, 16, 11008, 4096, 0),
+    (np.float16, 7, 4096, 12288, 0), (np.float16, 16, 4096, 11008, 22016), (np.float16, 32, 4096, 4096, 0),
+    (np.float16, 17, 256, 136, 140), (np.float16, 16, 1024, 200, 0), (np.float16, 4, 4096, 32000, 0),
+    (np.float32, 1, 64, 8, 0), (np.float32, 5, 128, 36, 40), (np.float32, 16, 4096, 4096, 0), (np.float32, 16, 11008, 4096, 0),
+    (np.float32, 9, 4096, 11008, 22016), (np.float32, 32, 1024, 520, 0), (np.float32, 20, 256, 100, 0)])
+def test_few_row_kernel_matches_the_oracle_in_every_configuration(G, ref, dtype, M, K, N, ldy):
     """onellm_linear's own kernel for a decode step's rows, forced (tuning key gemm_skinny = 1) through every kernel
-    variant and every number of slices along K that takes the problem: fp16 parity with the oracle, untouched
-    padding columns, the same bits on a second call (the sliced runs reuse one workspace and its arrival counters)."""
+    variant and every number of slices along K that takes the problem: parity with the oracle at the element type's
+    bar, untouched padding columns, the same bits on a second call (the sliced runs reuse one workspace and its
+    arrival counters)."""
     import torch
     from onellm_amd import capi
-    announce("few-row linear", M, K, N, ldy)
+    announce("few-row linear", dtype.__name__, M, K, N, ldy)
     rng = np.random.default_rng(M * 131 + N)
-    x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
-    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    x = (rng.standard_normal((M, K)) * 0.5).astype(dtype)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(dtype)
     want = ref.linear(x, w).astype(np.float64)
     dx, dw = _dev(torch, x), _dev(torch, w)
     ld = ldy or N
@@ -162,12 +166,12 @@ def test_few_row_kernel_matches_the_oracle_in_every_configuration(G, ref, M, K, 
     ran = []
     capi.tune_set("gemm_skinny", 1)
     try:
-        for variant in range(8):
+        for variant in range(13):
             for splits in (1, 2, 3, 4, 6, 8, 16):
                 capi.tune_set("gemm_skinny_config", 100 * variant + splits)
                 outs = []
                 for rep in range(2):
-                    y = torch.full((M, ld), float("nan"), dtype=torch.float16, device=dx.device)
+                    y = torch.full((M, ld), float("nan"), dtype=dx.dtype, device=dx.device)
                     capi.linear(dx, dw, y, ldy=ld, workspace=ws)
                     torch.cuda.synchronize()
                     outs.append(y.cpu().numpy())
@@ -175,7 +179,7 @@ def test_few_row_kernel_matches_the_oracle_in_every_configuration(G, ref, M, K, 
                     continue                               # (this configuration does not take the problem: the library ran)
                 ran.append((variant, splits))
                 got = outs[0]
-                np.testing.assert_allclose(got[:, :N].astype(np.float64), want, err_msg=str((variant, splits)), **TOL[np.float16])
+                np.testing.assert_allclose(got[:, :N].astype(np.float64), want, err_msg=str((variant, splits)), **TOL[dtype])
                 assert np.isnan(got[:, N:]).all(), (variant, splits)
                 assert np.array_equal(outs[0][:, :N], outs[1][:, :N]), (variant, splits)
     finally:
@@ -186,24 +190,25 @@ def test_few_row_kernel_matches_the_oracle_in_every_configuration(G, ref, M, K, 
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,K,N", [(16, 4096, 11008), (5, 256, 72), (20, 512, 200)])
-def test_pair_of_projections_in_one_launch_matches_two_calls_and_the_oracle(G, ref, M, K, N):
+@pytest.mark.parametrize("dtype,M,K,N", [(np.float16, 16, 4096, 11008), (np.float16, 5, 256, 72), (np.float16, 20, 512, 200),
+                                         (np.float32, 16, 4096, 1408), (np.float32, 3, 256, 36)])
+def test_pair_of_projections_in_one_launch_matches_two_calls_and_the_oracle(G, ref, dtype, M, K, N):
     """onellm_linear_pair (the gate / up projections into the [M, 2, N] buffer the SwiGLU kernel reads): forced through
     the one-launch configurations, both halves match the oracle and are bit-identical to two onellm_linear calls
     with the same configuration; after a tuning run the chosen form still matches."""
     import torch
     from onellm_amd import capi
-    announce("linear pair", M, K, N)
+    announce("linear pair", dtype.__name__, M, K, N)
     rng = np.random.default_rng(N + M)
-    x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
-    w0 = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
-    w1 = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    x = (rng.standard_normal((M, K)) * 0.5).astype(dtype)
+    w0 = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(dtype)
+    w1 = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(dtype)
     want0, want1 = ref.linear(x, w0).astype(np.float64), ref.linear(x, w1).astype(np.float64)
     dx, d0, d1 = _dev(torch, x), _dev(torch, w0), _dev(torch, w1)
     ws = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dx.device)
 
     def run_pair():
-        pair = torch.full((M, 2, N), float("nan"), dtype=torch.float16, device=dx.device)
+        pair = torch.full((M, 2, N), float("nan"), dtype=dx.dtype, device=dx.device)
         capi.linear_pair(dx, d0, d1, pair, pair.view(-1)[N:], ldy=2 * N, workspace=ws)
         torch.cuda.synchronize()
         return pair.cpu().numpy()
@@ -211,16 +216,16 @@ def test_pair_of_projections_in_one_launch_matches_two_calls_and_the_oracle(G, r
     ran = 0
     capi.tune_set("gemm_skinny", 1)
     try:
-        for variant in range(7):
+        for variant in range(13):
             for splits in (1, 2, 4, 8):
                 capi.tune_set("gemm_skinny_config", 100 * variant + splits)
                 got = run_pair()
                 if G.onellm_linear_last_path() != 3:
                     continue
                 ran += 1
-                np.testing.assert_allclose(got[:, 0].astype(np.float64), want0, err_msg=str((variant, splits)), **TOL[np.float16])
-                np.testing.assert_allclose(got[:, 1].astype(np.float64), want1, err_msg=str((variant, splits)), **TOL[np.float16])
-                two = torch.full((M, 2, N), float("nan"), dtype=torch.float16, device=dx.device)
+                np.testing.assert_allclose(got[:, 0].astype(np.float64), want0, err_msg=str((variant, splits)), **TOL[dtype])
+                np.testing.assert_allclose(got[:, 1].astype(np.float64), want1, err_msg=str((variant, splits)), **TOL[dtype])
+                two = torch.full((M, 2, N), float("nan"), dtype=dx.dtype, device=dx.device)
                 capi.linear(dx, d0, two, ldy=2 * N, workspace=ws)
                 capi.linear(dx, d1, two.view(-1)[N:], ldy=2 * N, workspace=ws)
                 torch.cuda.synchronize()
@@ -230,11 +235,11 @@ def test_pair_of_projections_in_one_launch_matches_two_calls_and_the_oracle(G, r
         capi.tune_set("gemm_skinny", -1)
         capi.tune_set("gemm_skinny_config", -1)
     assert ran >= 3
-    best, two_calls = capi.linear_pair_tune(capi.FP16, M, K, N, ldy=2 * N, workspace=ws)
+    best, two_calls = capi.linear_pair_tune(capi.FP16 if dtype == np.float16 else capi.FP32, M, K, N, ldy=2 * N, workspace=ws)
     assert 0 < best <= two_calls
     got = run_pair()
-    np.testing.assert_allclose(got[:, 0].astype(np.float64), want0, **TOL[np.float16])
-    np.testing.assert_allclose(got[:, 1].astype(np.float64), want1, **TOL[np.float16])
+    np.testing.assert_allclose(got[:, 0].astype(np.float64), want0, **TOL[dtype])
+    np.testing.assert_allclose(got[:, 1].astype(np.float64), want1, **TOL[dtype])
 
 
 @pytest.mark.gpu
@@ -290,13 +295,13 @@ def test_few_row_kernel_cut_runs_back_to_back_on_one_workspace(G, ref):
 
 @pytest.mark.gpu
 def test_few_row_kernel_declines_what_it_is_not_built_for(G, ref):
-    """Forced or not, a problem outside the kernel's rules (fp32, W as [N, K], too many rows, K not in whole
-    64-row blocks, N or the row stride not in whole pieces, a misaligned operand) runs the library as before."""
+    """Forced or not, a problem outside the kernel's rules (rows of W that are not whole 16-byte pieces, W as [N, K],
+    too many rows, K not in whole 64-row blocks, a misaligned operand) runs the library as before."""
     import torch
     from onellm_amd import capi
     capi.tune_set("gemm_skinny", 1)
     try:
-        for dtype, M, K, N, nk, shift in [(np.float32, 4, 128, 64, False, 0), (np.float16, 4, 128, 64, True, 0), (np.float16, 33, 128, 64, False, 0),
+        for dtype, M, K, N, nk, shift in [(np.float32, 4, 128, 66, False, 0), (np.float16, 4, 128, 64, True, 0), (np.float16, 33, 128, 64, False, 0),
                                           (np.float16, 4, 96, 64, False, 0), (np.float16, 4, 128, 68, False, 0), (np.float16, 4, 128, 64, False, 1)]:
             announce("few-row linear declines", dtype.__name__, M, K, N, nk, shift)
             rng = np.random.default_rng(K + N)
