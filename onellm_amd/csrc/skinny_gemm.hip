@@ -398,7 +398,9 @@ bool config_fits(const Variant& v, int dtype, int splits, int M, int K, int N, s
 
 // The counter set of a workspace.  A set belongs to the workspace that used it last; when all are taken the one unused
 // for longest changes hands - its counters are zero between calls, and the workspace it served would have to be in the
-// middle of a call while kCounterSets others take their turn for that to matter.
+// middle of a call while kCounterSets others take their turn for that to matter.  (A launch captured into a graph
+// keeps the set it was given; after such a change of hands two workspaces share a set, which is harmless as long as
+// their calls do not run at the same time.)
 int counter_set_of(const void* workspace)
 {
     static std::mutex m;
