@@ -243,33 +243,34 @@ def cpu_norm(N, H, fused, budget_s):
     return time_cpu(lambda: ref.rmsnorm(x, g, 1e-5), budget_s)
 
 
-def decoder_layer_section(capi, dev, args):
-    """One whole decoder layer of the Llama-2-7B shape at batch 16, ctx 4096, as LlamaSelfDecoder sequences it:
+def decoder_layer_section(capi, dev, args, B=16, H=32, Hkv=32, S=4096, I=11008, key="decoder_layer_llama7b_b16_ctx4096"):
+    """One whole decoder layer of the Llama-2-7B shape at batch 16, ctx 4096 (or, with other arguments, of the same width
+    with grouped-query heads at batch 32, ctx 8192), as LlamaSelfDecoder sequences it:
     RMSNorm -> qkv projection -> fused masked attention -> output projection -> fused add-bias-residual-RMSNorm ->
     gate / up projections -> SwiGLU -> down projection -> fused add-bias-residual-RMSNorm.  The projections go through
     onellm_linear (hipBLASLt or this repository's few-row kernel, whichever its tuning run found faster); everything
     else is this repository's kernels.  Steps rotate over three sets of weights and of caches (1.2 GB and 3.2 GB), so
     that every step meets its weights cold, as a layer inside a 32-layer model does."""
     import torch
-    B, H, D, S, I, t = 16, 32, 128, 4096, 11008, 4096
-    hid = H * D
+    D, t = 128, S
+    hid, nqkv = H * D, (H + 2 * Hkv) * D
     g = torch.Generator(device=dev).manual_seed(7)
     rnd = lambda *shape, scale=1.0: (torch.randn(*shape, device=dev, generator=g) * scale).half()
     NSETS = 3
-    wsets = [dict(wqkv=rnd(hid, 3 * hid, scale=hid ** -0.5), wo=rnd(hid, hid, scale=hid ** -0.5), wgate=rnd(hid, I, scale=hid ** -0.5),
+    wsets = [dict(wqkv=rnd(hid, nqkv, scale=hid ** -0.5), wo=rnd(hid, hid, scale=hid ** -0.5), wgate=rnd(hid, I, scale=hid ** -0.5),
                   wup=rnd(hid, I, scale=hid ** -0.5), wdown=rnd(I, hid, scale=I ** -0.5)) for _ in range(NSETS)]
-    bqkv, bo, bd = rnd(3 * hid, scale=0.1), rnd(hid, scale=0.1), rnd(hid, scale=0.1)
+    bqkv, bo, bd = rnd(nqkv, scale=0.1), rnd(hid, scale=0.1), rnd(hid, scale=0.1)
     g1, g2, g3 = (torch.rand(hid, device=dev, generator=g) + 0.5).half(), (torch.rand(hid, device=dev, generator=g) + 0.5).half(), \
         (torch.rand(hid, device=dev, generator=g) + 0.5).half()
-    sets = [(rnd(1, B, H, S, D, scale=0.5), rnd(1, B, H, S, D, scale=0.5)) for _ in range(NSETS)]
+    sets = [(rnd(1, B, Hkv, S, D, scale=0.5), rnd(1, B, Hkv, S, D, scale=0.5)) for _ in range(NSETS)]
     x0 = rnd(B, hid)
     x, y = x0.clone(), torch.empty_like(x0)
-    qkv, att = torch.empty(B, 3 * H, D, dtype=torch.float16, device=dev), torch.empty(B, hid, dtype=torch.float16, device=dev)
+    qkv, att = torch.empty(B, H + 2 * Hkv, D, dtype=torch.float16, device=dev), torch.empty(B, hid, dtype=torch.float16, device=dev)
     pair, act = torch.empty(B, 2, I, dtype=torch.float16, device=dev), torch.empty(B, I, dtype=torch.float16, device=dev)
-    ws_attn = torch.empty(capi.decode_attn_workspace_bytes(B, H, H, D, t), dtype=torch.uint8, device=dev)
+    ws_attn = torch.empty(capi.decode_attn_workspace_bytes(B, H, Hkv, D, t), dtype=torch.uint8, device=dev)
     ws_gemm = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dev)
 
-    for (K_, N_, ld_) in ((hid, 3 * hid, 0), (hid, hid, 0), (I, hid, 0)):
+    for (K_, N_, ld_) in ((hid, nqkv, 0), (hid, hid, 0), (I, hid, 0)):
         capi.linear_tune(capi.FP16, B, K_, N_, ldy=ld_, workspace=ws_gemm)
     capi.linear_pair_tune(capi.FP16, B, hid, I, ldy=2 * I, workspace=ws_gemm)
 
@@ -278,7 +279,7 @@ def decoder_layer_section(capi, dev, args):
         capi.rmsnorm(y, g1, 1e-5)
 
     def proj_qkv(i):
-        capi.linear(y, wsets[i % NSETS]["wqkv"], qkv.view(B, 3 * hid), workspace=ws_gemm)
+        capi.linear(y, wsets[i % NSETS]["wqkv"], qkv.view(B, nqkv), workspace=ws_gemm)
 
     def attention(i):
         kc, vc = sets[i % len(sets)]
@@ -316,7 +317,7 @@ def decoder_layer_section(capi, dev, args):
     # the whole layer as the C++ LlamaSelfDecoder queues it (one call per step; its output-projection and down-projection
     # biases are applied by the fused norms, as above)
     def decoder(k, **kw):
-        return capi.SelfDecoder(capi.FP16, B, H, H, D, I, S, D, 10000.0, 1e-5,
+        return capi.SelfDecoder(capi.FP16, B, H, Hkv, D, I, S, D, 10000.0, 1e-5,
                                 [dict(attn_norm=g1, ffn_norm=g2, bqkv=bqkv, bo=bo, bdown=bd, **wsets[k])], g3, **kw)
 
     decs = [decoder(k) for k in range(NSETS)]
@@ -358,7 +359,7 @@ def decoder_layer_section(capi, dev, args):
         d.close()
     ms_py = time_steps(layer, steps, 3)
     weight_bytes = 2 * sum(w.numel() for w in wsets[0].values())
-    nb = weight_bytes + attn_bytes(B, H, H, D, [t] * B, 2)
+    nb = weight_bytes + attn_bytes(B, H, Hkv, D, [t] * B, 2)
     e = entry(ms, nb)
     e["parts_us"], e["gemm_path"] = {}, {}
     path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel", 3: "own few-row kernel, both in one launch"}
@@ -370,7 +371,7 @@ def decoder_layer_section(capi, dev, args):
     e["us_graph_replay"] = round(ms_graph * 1e3, 2)
     e["note"] = ("bytes = the five weight matrices (%d) + the attention step's algorithmic bytes; steps rotate over %d sets of "
                  "weights and caches; parts are timed one at a time, so their sum includes a launch gap per part" % (weight_bytes, NSETS))
-    return {"decoder_layer_llama7b_b16_ctx4096": e}
+    return {key: e}
 
 
 def projections_section(capi, dev, steps):
@@ -553,6 +554,10 @@ def extras_section(capi, dev, args, with_cpu):
 
     ex.update(projections_section(capi, dev, args.steps))
     ex.update(decoder_layer_section(capi, dev, args))
+    torch.cuda.empty_cache()
+    # the same layer width with grouped-query heads at BASELINE configs[2]'s batch and cache (32 sequences, 32 q / 8 kv
+    # heads, 8192 rows each: the layers take one step count for the whole batch): 32 rows through the projections
+    ex.update(decoder_layer_section(capi, dev, args, B=32, H=32, Hkv=8, S=8192, key="decoder_layer_gqa_b32_q32_kv8_ctx8192"))
     torch.cuda.empty_cache()
 
     for (N, Hd) in ((16, 4096), (512, 4096), (8192, 4096), (8192, 8192)):
