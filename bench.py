@@ -313,7 +313,7 @@ def decoder_layer_section(capi, dev, args, B=16, H=32, Hkv=32, S=4096, I=11008, 
         for _, fn in parts:
             fn(i)
 
-    steps = max(args.steps // 3, 10)
+    steps = args.steps
     # the whole layer as the C++ LlamaSelfDecoder queues it (one call per step; its output-projection and down-projection
     # biases are applied by the fused norms, as above)
     def decoder(k, **kw):
@@ -329,6 +329,13 @@ def decoder_layer_section(capi, dev, args, B=16, H=32, Hkv=32, S=4096, I=11008, 
         decs[i % NSETS].forward(t, x, y, kc, vc)
 
     ms = time_steps(layer_cpp, steps, max(args.warmup // 3, 3))
+    # the same step with every projection on the GEMM library, the division of labour the task statement names (this
+    # library's few-row projection kernel is an extension the tuning run may pick; tuning key gemm_skinny = 0 rules it out)
+    capi.tune_set("gemm_skinny", 0)
+    try:
+        ms_library = time_steps(layer_cpp, steps, max(args.warmup // 3, 3))
+    finally:
+        capi.tune_set("gemm_skinny", -1)
     for d in decs:
         d.close()
 
@@ -362,13 +369,15 @@ def decoder_layer_section(capi, dev, args, B=16, H=32, Hkv=32, S=4096, I=11008, 
     nb = weight_bytes + attn_bytes(B, H, Hkv, D, [t] * B, 2)
     e = entry(ms, nb)
     e["parts_us"], e["gemm_path"] = {}, {}
-    path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel", 3: "own few-row kernel, both in one launch"}
+    path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel", 3: "own few-row kernel, both in one launch",
+                  4: "own few-row kernel, uncut (no counter set free)", 5: "hipBLASLt (no counter set free)"}
     for name, fn in parts:
         e["parts_us"][name] = round(time_steps(fn, steps, 3) * 1e3, 2)
         if name.endswith("_proj"):
             e["gemm_path"][name] = path_names.get(capi.gemm_lib().onellm_linear_last_path(), "?")
     e["us_same_sequence_from_python"] = round(ms_py * 1e3, 2)
     e["us_graph_replay"] = round(ms_graph * 1e3, 2)
+    e["us_with_library_projections"] = round(ms_library * 1e3, 2)
     e["note"] = ("bytes = the five weight matrices (%d) + the attention step's algorithmic bytes; steps rotate over %d sets of "
                  "weights and caches; parts are timed one at a time, so their sum includes a launch gap per part" % (weight_bytes, NSETS))
     return {key: e}
@@ -382,7 +391,8 @@ def projections_section(capi, dev, steps):
     import torch
     M, hid, I = 16, 4096, 11008
     ws = torch.empty(capi.linear_workspace_bytes(), dtype=torch.uint8, device=dev)
-    path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel", 3: "own few-row kernel, both in one launch"}
+    path_names = {0: "plain kernel", 1: "hipBLASLt", 2: "own few-row kernel", 3: "own few-row kernel, both in one launch",
+                  4: "own few-row kernel, uncut (no counter set free)", 5: "hipBLASLt (no counter set free)"}
     out = {}
     for name, K, N, pair in (("qkv", hid, 3 * hid, False), ("out", hid, hid, False), ("gate_up_pair", hid, I, True), ("down", I, hid, False)):
         w_bytes = 2 * K * N * (2 if pair else 1)
@@ -506,7 +516,7 @@ def extras_section(capi, dev, args, with_cpu):
     tl = np.random.default_rng(3).integers(1024, 8193, size=B3).astype(np.int32)
     t_dev = torch.from_numpy(tl).to(dev)
     nb_fused = attn_bytes(B3, Hq3, Hkv3, D, tl.tolist(), 2)
-    steps3 = max(args.steps // 3, 10)
+    steps3 = args.steps          # (every extras line times the same number of launches per block: the label below)
     ms, (qkv, bias, (kc, vc), _) = bench_attention(capi, dev, steps3, args.warmup, B3, Hq3, Hkv3, D, S3, S3, nsets=3, t_dev=t_dev)
     cpu = cpu_attention(qkv, bias, kc, vc, Hq3, tl, D, 6.0)[0] if with_cpu else None
     ex["decode_attn_gqa_fused_b32_q32_kv8_len1024-8192"] = entry(ms, nb_fused, cpu)

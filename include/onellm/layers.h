@@ -63,6 +63,10 @@ void setLinearGemmAutotune(bool on);
 void setLinearGemmPlainFallback(bool allow);
 // Number of GEMM workspaces alive: one per (device, launch stream) that has run a projection.
 size_t linearGemmWorkspaceCount();
+// Before a stream that ran projections is destroyed: waits for the stream, frees the GEMM workspace the current
+// device keeps for it and gives the workspace's arrival-counter sets back (onellm_release_workspace).  Returns
+// whether there was one.  Graphs captured on that stream must not be replayed afterwards.
+bool releaseLinearGemmWorkspace(hipStream_t stream);
 
 class LLaMASelfAttentionLayer {
 public:

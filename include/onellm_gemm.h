@@ -60,7 +60,10 @@ int onellm_linear_pair_tune(int dtype, int M, int K, int N, int ldy, int w_is_nk
 size_t onellm_linear_workspace_bytes(void);
 
 /* what the last onellm_linear / onellm_linear_pair call on this thread ran: 1 the library GEMM, 2 this library's
- * few-row kernel, 3 that kernel for both projections of a pair in one launch, 0 the plain fallback kernel */
+ * few-row kernel, 3 that kernel for both projections of a pair in one launch, 0 the plain fallback kernel; and, when
+ * the tuned configuration cuts the problem along K but every arrival-counter set of this GPU belongs to another
+ * workspace (onellm_hip.h, onellm_release_workspace): 4 the few-row kernel uncut, 5 the library GEMM - same results,
+ * slower than the tuned form */
 int onellm_linear_last_path(void);
 
 /* allow != 0: problems of any size may run the plain kernel when the library declines them (process-wide; off by

@@ -119,8 +119,9 @@ size_t onellm_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int max
  * Same arguments, results and kernels as onellm_decode_attn, minus the workspace: split partials and
  * arrival counters live in a fixed device array inside the library,
  * ONELLM_DECODE_ATTN_STATIC_SCRATCH_BYTES (16 MiB) per GPU, held from library load to process exit.
- * The call allocates, frees and synchronises nothing.  The first call on a GPU also queues one small
- * kernel on `stream` that clears the counter region.  A step whose partials do not fit returns
+ * The call allocates, frees and synchronises nothing and launches only the attention kernel (the array is
+ * zero when the library is loaded and every call leaves its counters at zero), so it can be the first call
+ * on a stream that is being captured.  A step whose partials do not fit returns
  * ONELLM_ESCRATCH before anything is launched (onellm_decode_attn_workspace_bytes() is an upper bound
  * of what a step may need; steps that are not split need nothing).  All calls on one GPU share the
  * array, so calls that overlap in time on one GPU (two streams, two threads) race: serialise them.
@@ -190,11 +191,12 @@ int onellm_kv_repeat(int dtype, const void* k_cache, const void* v_cache,
  * (tests/unittests/test_beamsearch_topK.cu:33-35).
  * 1 <= K <= 8.  Slots with no candidate hold value -inf and id -1.
  * On a stream that is not being captured both stages run in one kernel launch (the workgroup of a batch entry that
- * stores its survivors last merges them), for up to 1024 batch entries and for the first 64 distinct workspace
- * pointers a process passes; beyond either limit, and on a stream under capture, stage 2 is a second launch (a
- * launch less is worth more to the host than the 1.5 us the longer kernel costs the device; a replayed graph has no
- * host in it).  Same results either way.  Two calls that may overlap in time need two workspaces, as in the
- * reference.
+ * stores its survivors last merges them), for up to 1024 batch entries, with arrival counters the library keeps per
+ * (GPU, workspace pointer): 64 sets per GPU, owned from a workspace's first call until onellm_release_workspace().
+ * Beyond either limit, and on a stream under capture, stage 2 is a second launch (a launch less is worth more to the
+ * host than the 1.5 us the longer kernel costs the device; a replayed graph has no host in it).  Same results either
+ * way; onellm_beam_topk_last_path() tells which ran and why.  Two calls that may overlap in time need two
+ * workspaces, as in the reference.
  */
 #define ONELLM_TOPK_BLOCKS_PER_ROW 8
 int onellm_beam_topk(const float* logits, int B, int beam, int V, int K,
@@ -203,6 +205,30 @@ size_t onellm_beam_topk_workspace_bytes(int B, int beam, int K);
 /* kernel launches the last onellm_beam_topk call of this thread queued: 1 or 2 (0 before the first call or after
  * a refused one).  No counterpart in the reference; for tests and profiles. */
 int onellm_beam_topk_last_launches(void);
+/* which form the last onellm_beam_topk call of this thread took (0 before the first call or after a refused one).
+ * No counterpart in the reference. */
+#define ONELLM_TOPK_PATH_ONE_LAUNCH     1 /* both stages in one launch                                            */
+#define ONELLM_TOPK_PATH_TWO_LAUNCHES   2 /* by design: stream under capture, more than 1024 batch entries, or the
+                                             topk_two_launches tuning key                                          */
+#define ONELLM_TOPK_PATH_NO_COUNTER_SET 3 /* two launches because every counter set of this GPU belongs to another
+                                             workspace: release the ones no longer used                            */
+int onellm_beam_topk_last_path(void);
+
+/*
+ * Arrival-counter sets.  Kernels that finish split work in one launch (the one-launch beam top-K here, the few-row
+ * projection kernel of onellm_gemm.h when it cuts a problem along K) count arrivals in static device memory of the
+ * library, one set of counters per (GPU, workspace pointer).  A set is owned from the first call that passes the
+ * workspace and is never handed to another workspace behind the caller's back - a launch recorded into a graph keeps
+ * its counters for as long as the graph lives.  A caller that frees or stops using a workspace gives its sets back:
+ *   onellm_release_workspace(ptr)  returns how many sets (over all GPUs and kernel families) were freed.  The caller
+ *       states that no launch that was handed `ptr` is queued, running, or recorded in a graph that will be replayed.
+ * When every set of a GPU is owned, a call with a new workspace runs the form that needs no counters (a second
+ * launch, an uncut run or the GEMM library): same results, slower, reported by the call's *_last_path query, counted
+ * process-wide by onellm_counter_set_fallbacks() and announced once on stderr.  No counterpart in the reference
+ * (its top-K always takes two launches, src/kernels/beamsearch_topK.cu:85-119).
+ */
+int onellm_release_workspace(const void* workspace);
+long onellm_counter_set_fallbacks(void);
 
 /* ------------------------------------------------------------------------------------------------
  * The callers either side of the decode path (built after the six entry points above).

@@ -24,6 +24,10 @@ int onellm_layers_linear(int dtype, void* x, void* w, void* y, int M, int K, int
  * exist (one per device and launch stream that has run a projection). */
 int onellm_layers_allow_plain_gemm(int allow);
 int onellm_layers_gemm_workspace_count(void);
+/* releaseLinearGemmWorkspace of onellm/layers.h: before a launch stream is destroyed, waits for it, frees the GEMM
+ * workspace the current device keeps for it and gives its arrival-counter sets back.  1: freed, 0: the stream had
+ * none, -1: error (onellm_layers_last_error). */
+int onellm_layers_release_gemm_workspace(onellm_stream_t stream);
 
 /* A LlamaSelfDecoder (src/layers/decoder/self_decoder.h:10-74) with its layer weights and an allocator.
  * The ten `void**` are host arrays of L device pointers, in the order of LlamaLayerWeight::loadWeights

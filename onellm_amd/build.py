@@ -38,7 +38,7 @@ DRIVER_SRC = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver.cpp")
 DRIVER_BIN = os.path.join(ROOT, "tests", "cpp", "self_decoder_driver")
 
 KERNEL_SOURCES = ["decode_attn.hip", "norms.hip", "kv_cache.hip", "beam_topk.hip", "prefill_rope.hip", "activation.hip", "sampling.hip",
-                  "tuning.cpp"]
+                  "tuning.cpp", "counter_sets.cpp"]
 LAUNCHER_SOURCES = ["launchers.cpp"]
 GEMM_SOURCES = ["linear.hip", "skinny_gemm.hip"]
 LAYER_SOURCES = ["layers.cpp", "layers_capi.cpp"]
@@ -146,7 +146,7 @@ def build(force=False, verbose=False):
               ["-L" + HERE, "-lonellm_hip", "-Wl,-rpath,$ORIGIN"]
         subprocess.run(cmd, check=True, capture_output=not verbose)
     if os.path.exists(HARNESS_SRC) and (force or _newer(LIB_HARNESS, [HARNESS_SRC, LIB_LAUNCH] + _headers())):
-        cmd = [HIPCC, "-shared", "-fPIC", "-O2", "-std=c++17", "-I" + INCLUDE, HARNESS_SRC, "-o", LIB_HARNESS,
+        cmd = [HIPCC, "-shared", "-fPIC", "-O2", "-std=c++17", "-I" + INCLUDE, "-I" + CSRC, HARNESS_SRC, "-o", LIB_HARNESS,
                "-L" + HERE, "-lonellm_launchers", "-lonellm_hip", "-Wl,-rpath,$ORIGIN/../../onellm_amd"]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:

@@ -5,6 +5,7 @@ fallback: if the library is not built, loading raises.
 """
 import ctypes
 import os
+import weakref
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libonellm_hip.so")
@@ -17,6 +18,7 @@ ATTN_NO_V_BIAS = 0x1
 ATTN_NO_CACHE_WRITE = 0x2
 ATTN_ZEROED_WORKSPACE = 0x4
 TOPK_BLOCKS_PER_ROW = 8
+TOPK_PATH_ONE_LAUNCH, TOPK_PATH_TWO_LAUNCHES, TOPK_PATH_NO_COUNTER_SET = 1, 2, 3
 
 # every symbol include/onellm_hip.h declares: name -> (restype, argtypes)
 _vp, _ci, _cf, _cu, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_uint, ctypes.c_size_t
@@ -36,6 +38,9 @@ SYMBOLS = {
     "onellm_beam_topk": (_ci, [_vp, _ci, _ci, _ci, _ci, _vp, _vp]),
     "onellm_beam_topk_workspace_bytes": (_sz, [_ci, _ci, _ci]),
     "onellm_beam_topk_last_launches": (_ci, []),
+    "onellm_beam_topk_last_path": (_ci, []),
+    "onellm_release_workspace": (_ci, [_vp]),
+    "onellm_counter_set_fallbacks": (ctypes.c_long, []),
     "onellm_qkv_bias_rope_transpose": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci,
                                              _cf, _vp]),
     "onellm_silu_and_mul": (_ci, [_ci, _vp, _vp, _ci, _ci, _vp]),
@@ -182,6 +187,20 @@ def beam_topk_last_launches():
     return lib().onellm_beam_topk_last_launches()
 
 
+def beam_topk_last_path():
+    return lib().onellm_beam_topk_last_path()
+
+
+def release_workspace(workspace):
+    """Give the arrival-counter sets of a workspace (a tensor or a raw pointer) back; returns how many were freed."""
+    ptr = workspace if isinstance(workspace, int) else workspace.data_ptr()
+    return lib().onellm_release_workspace(ptr)
+
+
+def counter_set_fallbacks():
+    return lib().onellm_counter_set_fallbacks()
+
+
 def beam_topk(logits, B, beam, K, workspace=None):
     """logits [B*beam, V] fp32.  Returns (workspace, round1_vals, round1_ids, final_vals, final_ids) as views."""
     import torch
@@ -189,6 +208,9 @@ def beam_topk(logits, B, beam, K, workspace=None):
     assert rows == B * beam and logits.dtype == torch.float32
     if workspace is None:
         workspace = torch.empty(beam_topk_workspace_bytes(B, beam, K) // 4, dtype=torch.float32, device=logits.device)
+        # a workspace made here gives its counter set back when the tensor dies (the caller of the C function does
+        # that itself, with onellm_release_workspace, when it frees a workspace)
+        weakref.finalize(workspace, lib().onellm_release_workspace, workspace.data_ptr())
     _check(lib().onellm_beam_topk(_ptr(logits), B, beam, V, K, _ptr(workspace), _stream()), "onellm_beam_topk")
     n1 = B * beam * TOPK_BLOCKS_PER_ROW * K
     vals = workspace[:n1].view(B * beam, TOPK_BLOCKS_PER_ROW, K)

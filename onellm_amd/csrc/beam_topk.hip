@@ -28,13 +28,16 @@
 // counter.  The caller's workspace has no room for counters and is not zeroed, so they live in a file-scope
 // device array (zero when the module is loaded; the workgroup that merges sets its counter back to zero, so
 // every launch leaves them zero).  Launches that may overlap need counters of their own: a launch uses the
-// set that belongs to its workspace pointer (a small host-side table, filled as workspaces are first seen) -
-// two launches that share a workspace may not overlap anyway, they would overwrite each other's survivors.
-// A workspace that finds the table full, or a batch beyond the set's size, takes the two-launch form.
+// set its (device, workspace pointer) owns (counter_sets.hpp: owned from the first launch until the caller
+// gives it back with onellm_release_workspace, never reassigned in between) - two launches that share a
+// workspace may not overlap anyway, they would overwrite each other's survivors.  A workspace that finds
+// every set owned, or a batch beyond the set's size, takes the two-launch form, and
+// onellm_beam_topk_last_path says which of the two it was.
 #include <limits.h>
 #include <math.h>
 #include <mutex>
 #include "common.hpp"
+#include "counter_sets.hpp"
 
 namespace onellm {
 int tune_get(const char* key);
@@ -47,20 +50,9 @@ constexpr int kArrivalEntries = 1024;   // batch entries per launch of the one-l
 __device__ unsigned g_arrivals[kArrivalSets * kArrivalEntries];
 
 thread_local int g_last_launches = 0;
+thread_local int g_last_path = 0;
 
-// the counter set of this workspace; -1: none left
-int arrival_set_of(const void* workspace)
-{
-    static std::mutex m;
-    static const void* owner[kArrivalSets];
-    static int used = 0;
-    std::lock_guard<std::mutex> lock(m);
-    for (int i = 0; i < used; ++i)
-        if (owner[i] == workspace) return i;
-    if (used == kArrivalSets) return -1;
-    owner[used] = workspace;
-    return used++;
-}
+CounterSets g_arrival_sets("onellm_beam_topk", kArrivalSets);
 
 __device__ __forceinline__ Key make_key(float v, int id)
 {
@@ -573,8 +565,17 @@ int launch_topk(const float* logits, int B, int beam, int V, int K, int nblk, fl
         }
         two = cs != hipStreamCaptureStatusNone;
     }
-    const int set = (B <= kArrivalEntries && !two) ? arrival_set_of(ws) : -1;
+    int set = -1;
+    g_last_path = ONELLM_TOPK_PATH_TWO_LAUNCHES;
+    if (B <= kArrivalEntries && !two) {
+        int dev = 0;
+        const hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return (int)e;
+        set = g_arrival_sets.acquire(dev, ws);
+        if (set < 0) g_last_path = ONELLM_TOPK_PATH_NO_COUNTER_SET;
+    }
     if (set >= 0) {
+        g_last_path = ONELLM_TOPK_PATH_ONE_LAUNCH;
         hipLaunchKernelGGL((topk_stage1_kernel<KP, true>), dim3(B * beam * nblk), dim3(256), 0, st, logits, V, nblk, vec_ok, K,
                            vals, ids, set, beam, fvals, fids);
         g_last_launches = 1;
@@ -604,6 +605,7 @@ extern "C" int onellm_beam_topk(const float* logits, int B, int beam, int V, int
 {
     using namespace onellm;
     g_last_launches = 0;
+    g_last_path = 0;
     if (!logits || !workspace || B <= 0 || beam <= 0 || V <= 0) return ONELLM_EINVAL;
     if (K < 1 || K > 8) return ONELLM_EUNSUPPORTED;
     if ((long)B * beam * V > (long)INT_MAX - 1) return ONELLM_EUNSUPPORTED;   // ids are int32 flat indices
@@ -616,3 +618,5 @@ extern "C" int onellm_beam_topk(const float* logits, int B, int beam, int V, int
 }
 
 extern "C" int onellm_beam_topk_last_launches(void) { return onellm::g_last_launches; }
+
+extern "C" int onellm_beam_topk_last_path(void) { return onellm::g_last_path; }

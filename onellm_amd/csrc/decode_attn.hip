@@ -25,8 +25,8 @@
 // vector-ALU kernels) and attn_mfma.hpp (the matrix-core kernels for grouped-query heads).  Here: the merge
 // kernels, the scalar kernel for any head size, the launch selection and the C entry points.
 #include <math.h>
-#include <mutex>
 #include "common.hpp"
+#include "device_symbol.hpp"
 #include "rope.hpp"
 #include "attn_schedule.hpp"
 #include "attn_finish.hpp"
@@ -479,41 +479,10 @@ static __device__ __align__(256) unsigned char scratch[ONELLM_DECODE_ATTN_STATIC
 namespace onellm {
 namespace {
 
-__global__ __launch_bounds__(256)
-void zero_words_kernel(int* p, int n)
-{
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < n) p[i] = 0;
-}
-
-constexpr int kMaxDevices = 64;
-std::mutex g_scratch_mutex;
-void* g_scratch_ptr[kMaxDevices];          // device address of `scratch` on each GPU, resolved on first use
-
-// Address of the current device's copy of `scratch`.  The first call on a device resolves the symbol there and
-// queues one fill of the counter region on `st` (a kernel, not a memset node, so that a capturing stream records
-// something it can replay); nothing is allocated.
-int static_scratch(hipStream_t st, void** out)
-{
-    int dev = -1;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return static_cast<int>(e);
-    if (dev < 0 || dev >= kMaxDevices) return ONELLM_EUNSUPPORTED;
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (!g_scratch_ptr[dev]) {
-        void* p = nullptr;
-        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-        if (e != hipSuccess) return static_cast<int>(e);
-        if (!p) return static_cast<int>(hipErrorInvalidSymbol);
-        constexpr int words = (int)(kCounterBytes / sizeof(int));
-        hipLaunchKernelGGL(zero_words_kernel, dim3((words + 255) / 256), dim3(256), 0, st, static_cast<int*>(p), words);
-        const int rc = launch_status();
-        if (rc != 0) return rc;
-        g_scratch_ptr[dev] = p;
-    }
-    *out = g_scratch_ptr[dev];
-    return 0;
-}
+// Address of the current device's copy of `scratch`, resolved once per device.  Nothing is launched or allocated:
+// the array is zero when the module is loaded and every call leaves its counter region at zero again.
+DeviceSymbol g_scratch_address;
+int static_scratch(void** out) { return g_scratch_address.address(HIP_SYMBOL(scratch), out); }
 
 }  // namespace
 }  // namespace onellm
@@ -735,7 +704,7 @@ extern "C" int onellm_decode_attn_static(int dtype, const void* qkv, const void*
                                          int rope_pos_offset, unsigned flags, onellm_stream_t stream)
 {
     void* ws = nullptr;
-    int rc = onellm::static_scratch(static_cast<hipStream_t>(stream), &ws);
+    int rc = onellm::static_scratch(&ws);
     if (rc != 0) return rc;
     // the library owns this buffer and nothing else writes it: its counters are zero between calls
     rc = onellm_decode_attn(dtype, qkv, qkv_bias, k_cache, v_cache, out, B, Hq, Hkv, D, S, layer, num_layers, t_host, t_dev,

@@ -71,6 +71,25 @@ struct GemmWorkspace {
         buffers[key] = b;
         return b;
     }
+    bool drop(hipStream_t stream)
+    {
+        int device = 0;
+        hip_ok(hipGetDevice(&device), "gemm workspace device");
+        Buffer b;
+        {
+            std::lock_guard<std::mutex> g(mu);
+            auto it = buffers.find(std::make_pair(device, stream));
+            if (it == buffers.end()) return false;
+            b = it->second;
+            buffers.erase(it);
+        }
+        if (b.ptr) {
+            hip_ok(hipStreamSynchronize(stream), "gemm workspace sync");
+            (void)onellm_release_workspace(b.ptr);
+            hip_ok(hipFree(b.ptr), "gemm workspace free");
+        }
+        return true;
+    }
     size_t count()
     {
         std::lock_guard<std::mutex> g(mu);
@@ -140,6 +159,8 @@ void setLinearGemmAutotune(bool on)
 void setLinearGemmPlainFallback(bool allow) { (void)onellm_linear_allow_plain(allow ? 1 : 0); }
 
 size_t linearGemmWorkspaceCount() { return g_gemm_ws.count(); }
+
+bool releaseLinearGemmWorkspace(hipStream_t stream) { return g_gemm_ws.drop(stream); }
 
 // src/kernels/qkv_linear.cu:8-66
 void launchLinearGemm(Tensor* input, BaseWeight& weight, Tensor* output, bool trans_a, bool trans_b, bool shared_out_buf)

@@ -64,6 +64,13 @@ int onellm_layers_allow_plain_gemm(int allow)
 
 int onellm_layers_gemm_workspace_count(void) { return (int)linearGemmWorkspaceCount(); }
 
+int onellm_layers_release_gemm_workspace(onellm_stream_t stream)
+{
+    int had = 0;
+    const int rc = guarded([&] { had = releaseLinearGemmWorkspace(static_cast<hipStream_t>(stream)) ? 1 : 0; });
+    return rc == 0 ? had : -1;
+}
+
 // per-layer pointer arrays of length L, in the argument order of LlamaLayerWeight::loadWeights
 void* onellm_decoder_create(int dtype, int B, int Hq, int Hkv, int D, int I, int L, int S, int rotary_dim, float rope_base,
                         float eps, int attn_bias, void** attn_norm, void** ffn_norm, void** wqkv, void** bqkv, void** wo,

@@ -221,7 +221,7 @@ struct TimingRig {
 
 // what runs the two projections of a feed-forward block that share their input: key (M, K, N, ldy, workspace or not);
 // variant -1: two ordinary calls
-std::map<std::tuple<int, int, int, int, int, int>, SkinnyConfig> g_pair_plans;      // (first element: device)
+std::map<std::tuple<int, int, int, int, int, int, int>, SkinnyConfig> g_pair_plans;      // (device, element type, M, K, N, ldy, workspace or not)
 
 bool stream_capturing(hipStream_t st)
 {
@@ -380,7 +380,7 @@ extern "C" int onellm_linear_pair_tune(int dtype, int M, int K, int N, int ldy, 
     }
     {
         std::lock_guard<std::mutex> g(g_mu);
-        g_pair_plans[std::make_tuple(dev, M, K, N, ldy, workspace_bytes ? 1 : 0)] = chosen;
+        g_pair_plans[std::make_tuple(dev, dtype, M, K, N, ldy, workspace_bytes ? 1 : 0)] = chosen;
     }
     if (best_us) *best_us = best_ms * 1e3f;
     if (two_calls_us) *two_calls_us = two_ms * 1e3f;
@@ -429,6 +429,7 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
         }
     }
     if (tune_get("gemm_no_library") == 1) plan.usable = false;
+    bool no_counter_set = false;
     // this library's few-row kernel: where the tuning run chose it (tuning key gemm_skinny = 0: never; 1: wherever it
     // takes the problem, with a default configuration if none was timed)
     {
@@ -441,10 +442,20 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
             else if (c.variant < 0) c = skinny_default(dtype, M, K, N, workspace_bytes, 1);
         }
         if (c.variant >= 0) {
-            const int rc = skinny_launch(c, dtype, x, w, y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st);
+            int rc = skinny_launch(c, dtype, x, w, y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st);
             if (rc == 0) {
                 t_last_path = 2;
                 return 0;
+            }
+            if (rc == kSkinnyNoCounterSet) {
+                // the cut run found no arrival-counter set free: the same variant uncut, else the library; either way
+                // the caller can see it (paths 4 and 5)
+                no_counter_set = true;
+                rc = skinny_launch(SkinnyConfig{c.variant, 1}, dtype, x, w, y, nullptr, nullptr, M, K, N, ldy, workspace, workspace_bytes, st);
+                if (rc == 0) {
+                    t_last_path = 4;
+                    return 0;
+                }
             }
             if (rc != ONELLM_EUNSUPPORTED) return rc;        // (declined as given - alignment, workspace: on to the library)
         }
@@ -454,7 +465,7 @@ extern "C" int onellm_linear(int dtype, const void* x, const void* w, void* y, i
         const hipblasStatus_t s = hipblasLtMatmul(handle, plan.desc, &alpha, w, plan.la, x, plan.lb, &beta, y, plan.lc, y,
                                                   plan.lc, &plan.heur.algo, workspace, workspace_bytes, st);
         if (s == HIPBLAS_STATUS_SUCCESS) {
-            t_last_path = 1;
+            t_last_path = no_counter_set ? 5 : 1;
             return 0;
         }
     }
@@ -488,7 +499,7 @@ extern "C" int onellm_linear_pair(int dtype, const void* x, const void* w_first,
         if (e != hipSuccess) return (int)e;
         {
             std::lock_guard<std::mutex> g(g_mu);
-            auto it = g_pair_plans.find(std::make_tuple(dev, M, K, N, ldy, workspace_bytes ? 1 : 0));
+            auto it = g_pair_plans.find(std::make_tuple(dev, dtype, M, K, N, ldy, workspace_bytes ? 1 : 0));
             if (it != g_pair_plans.end()) c = it->second;
         }
         if (want == 1) {
@@ -497,11 +508,19 @@ extern "C" int onellm_linear_pair(int dtype, const void* x, const void* w_first,
             else if (c.variant < 0) c = skinny_default(dtype, M, K, N, workspace_bytes, 2);
         }
         if (c.variant >= 0) {
-            const int rc = skinny_launch(c, dtype, x, w_first, y_first, w_second, y_second, M, K, N, ldy, workspace, workspace_bytes,
-                                         static_cast<hipStream_t>(stream));
+            int rc = skinny_launch(c, dtype, x, w_first, y_first, w_second, y_second, M, K, N, ldy, workspace, workspace_bytes,
+                                   static_cast<hipStream_t>(stream));
             if (rc == 0) {
                 t_last_path = 3;
                 return 0;
+            }
+            if (rc == kSkinnyNoCounterSet) {
+                rc = skinny_launch(SkinnyConfig{c.variant, 1}, dtype, x, w_first, y_first, w_second, y_second, M, K, N, ldy, workspace,
+                                   workspace_bytes, static_cast<hipStream_t>(stream));
+                if (rc == 0) {
+                    t_last_path = 4;
+                    return 0;
+                }
             }
             if (rc != ONELLM_EUNSUPPORTED) return rc;
         }

@@ -16,15 +16,18 @@
 //   * The waves' tiles meet in LDS.  A run cut along K writes its slice's sums to the workspace with device-scope
 //     stores and bumps the panel's arrival counter; the slice that finds all others there adds them up in slice order
 //     (the result does not depend on who came last) and writes y.  The counters live in this library (one set per
-//     workspace seen), are zero between calls and are reset by the slice that reads them last.
+//     (device, workspace), owned until the workspace is released), are zero between calls and are reset by the slice
+//     that reads them last.
 // Alignment and shape rules are in skinny_shape_ok / skinny_launch; whatever they decline goes to the library GEMM.
-#include <mutex>
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include "onellm_gemm.h"
+#include "counter_sets.hpp"
+#include "device_symbol.hpp"
 #include "skinny_gemm.hpp"
 
 namespace onellm {
+int tune_get(const char* key);
 namespace {
 
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
@@ -51,6 +54,7 @@ struct SkinnyArgs {
     float* partial;                          // [panels][splits][rows][NT]
     unsigned* counters;                      // [panels]
     int M, K, N, ldy, splits;
+    int ordered;                             // 1: the counter add is a release and the reading slice takes an acquire fence
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t window(const void* p, unsigned bytes)
@@ -110,9 +114,17 @@ __device__ __forceinline__ void finish_tile(const SkinnyArgs& a, const float* ld
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0) {
-            const unsigned before = __hip_atomic_fetch_add(&a.counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // (the formally ordered form - tuning key gemm_ordered_finish - makes the add a release and has the reading
+            // slice take an acquire fence: the compiler then adds the write-back / invalidate of this chip quarter's L2,
+            // which the written-through stores and the memory-served loads do not need; kept for the soak test)
+            const unsigned before = a.ordered
+                ? __hip_atomic_fetch_add(&a.counters[slot], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT)
+                : __hip_atomic_fetch_add(&a.counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const int last = before == (unsigned)(a.splits - 1);
-            if (last) __hip_atomic_store(&a.counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
+            if (last) {
+                __hip_atomic_store(&a.counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero for the next call
+                if (a.ordered) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            }
             s_last = last;
         }
         __syncthreads();
@@ -396,54 +408,12 @@ bool config_fits(const Variant& v, int dtype, int splits, int M, int K, int N, s
     return need <= ws_bytes && need < (1u << 30);
 }
 
-// The counter set of a workspace.  A set belongs to the workspace that used it last; when all are taken the one unused
-// for longest changes hands - its counters are zero between calls, and the workspace it served would have to be in the
-// middle of a call while kCounterSets others take their turn for that to matter.  (A launch captured into a graph
-// keeps the set it was given; after such a change of hands two workspaces share a set, which is harmless as long as
-// their calls do not run at the same time.)
-int counter_set_of(const void* workspace)
-{
-    static std::mutex m;
-    static const void* owner[kCounterSets];
-    static unsigned long long last_use[kCounterSets];
-    static unsigned long long clock = 0;
-    static int used = 0;
-    std::lock_guard<std::mutex> lock(m);
-    int set = -1;
-    for (int i = 0; i < used && set < 0; ++i)
-        if (owner[i] == workspace) set = i;
-    if (set < 0 && used < kCounterSets) set = used++;
-    if (set < 0) {
-        set = 0;
-        for (int i = 1; i < kCounterSets; ++i)
-            if (last_use[i] < last_use[set]) set = i;
-    }
-    owner[set] = workspace;
-    last_use[set] = ++clock;
-    return set;
-}
+// The counter set of a (device, workspace): owned from the workspace's first cut run until the caller releases
+// the workspace, never handed to another one in between (counter_sets.hpp).
+CounterSets g_slice_sets("onellm_linear (few-row kernel cut along K)", kCounterSets);
 
 // this device's copy of the counters (every device has its own, at its own address)
-int device_counters(unsigned** out)
-{
-    constexpr int kDevices = 64;
-    static std::mutex m;
-    static unsigned* known[kDevices];
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
-    if (dev < 0 || dev >= kDevices) return ONELLM_EUNSUPPORTED;
-    std::lock_guard<std::mutex> lock(m);
-    if (!known[dev]) {
-        e = hipGetSymbolAddress(reinterpret_cast<void**>(&known[dev]), HIP_SYMBOL(g_slice_arrivals));
-        if (e != hipSuccess) {
-            known[dev] = nullptr;
-            return (int)e;
-        }
-    }
-    *out = known[dev];
-    return 0;
-}
+DeviceSymbol g_slice_arrivals_address;
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<size_t>(p) & (a - 1)) == 0; }
 
@@ -514,12 +484,22 @@ int skinny_launch(SkinnyConfig c, int dtype, const void* x, const void* w, void*
     a.M = M; a.K = K; a.N = N; a.ldy = ldy; a.splits = c.splits;
     if (c.splits > 1) {
         if (!aligned(workspace, 16)) return ONELLM_EUNSUPPORTED;
-        const int set = counter_set_of(workspace);
-        unsigned* counters = nullptr;
-        const int rc = device_counters(&counters);
+        int dev = 0;
+        const hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return (int)e;
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+            (void)hipGetLastError();
+            capturing = hipStreamCaptureStatusNone;
+        }
+        const int set = g_slice_sets.acquire(dev, workspace, capturing != hipStreamCaptureStatusNone);
+        if (set < 0) return kSkinnyNoCounterSet;
+        void* counters = nullptr;
+        const int rc = g_slice_arrivals_address.address(HIP_SYMBOL(g_slice_arrivals), &counters);
         if (rc != 0) return rc;
         a.partial = static_cast<float*>(workspace);
-        a.counters = counters + (size_t)set * kCounterPanels;
+        a.counters = static_cast<unsigned*>(counters) + (size_t)set * kCounterPanels;
+        a.ordered = tune_get("gemm_ordered_finish") == 1;
     }
     v.launch(a, dim3(panels_of(v, N), c.splits, problems), stream);
     return (int)hipGetLastError();

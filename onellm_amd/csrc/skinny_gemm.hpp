@@ -26,8 +26,12 @@ int skinny_candidates(int dtype, int M, int K, int N, size_t with_workspace_byte
 // A reasonable configuration without timing anything (what a forced run uses); variant -1 if there is none.
 SkinnyConfig skinny_default(int dtype, int M, int K, int N, size_t with_workspace_bytes, int problems);
 
+// skinny_launch: a run cut along K found every arrival-counter set of the device owned by other workspaces; nothing
+// was launched.  The caller runs the same variant uncut, or the library.
+constexpr int kSkinnyNoCounterSet = -1000;
+
 // Queues the multiplication.  0, ONELLM_EUNSUPPORTED (this kernel does not take the problem as given: alignment,
-// workspace too small for a sliced run - the caller goes on to the library) or a hipError_t.
+// workspace too small for a sliced run - the caller goes on to the library), kSkinnyNoCounterSet or a hipError_t.
 // A sliced run (splits > 1) uses `workspace` for partial sums; calls that share a workspace must not overlap, which
 // is the library's rule for the same buffer as well.
 // With w_second / y_second the launch also computes y_second = x . w_second (same shape and row stride): the gate and

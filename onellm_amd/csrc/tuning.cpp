@@ -28,6 +28,7 @@ Knob g_knobs[] = {
     {"attn_ordered_finish", {-1}}, // 1: release on the fused finish's counter add + acquire fence in the merging piece
     {"attn_early_look", {-1}},   // 1 / 0: a piece that finds the unit's other pieces arrived merges it from its registers / never looks
     {"topk_two_launches", {-1}}, // beam top-K: 1 = always a second launch for the merge of the survivors, 0 = one launch wherever it can be (also under capture)
+    {"gemm_ordered_finish", {-1}}, // 1: release on the few-row projection kernel's counter add + acquire fence in the slice that reads the sums back
     {"attn_turns", {-1}},        // 0: co-resident attention workgroups do not take turns at wave priority
 };
 }  // namespace
@@ -43,7 +44,8 @@ int tune_get(const char* key)
 
 // 1.1: ONELLM_ATTN_ZEROED_WORKSPACE, 64 KiB of arrival counters at the front of the attention workspace
 // 1.2: onellm_decode_attn_static
-extern "C" int onellm_hip_version(void) { return 1002; }
+// 1.3: onellm_release_workspace, onellm_counter_set_fallbacks, onellm_beam_topk_last_path
+extern "C" int onellm_hip_version(void) { return 1003; }
 
 extern "C" int onellm_tune_set(const char* key, int value)
 {

@@ -6,6 +6,7 @@
 #include <string>
 #include "onellm/kernels.h"
 #include "onellm/tensor_map.h"
+#include "counter_sets.hpp"
 
 namespace {
 std::string g_last_error;
@@ -237,6 +238,22 @@ int h_layer_weight_checks(int head_num, int kv_head_num, int head_size, int inte
     ok |= (attn_bias ? biases : none) << 5;
     ok |= (lw.self_attn_weight.qkv.type == WeightType::FP16_W && lw.ffn_weight.down.type == WeightType::FP16_W) << 6;
     return ok;
+}
+
+// ---- the table of arrival-counter sets (csrc/counter_sets.hpp): plain host logic, driven from Python
+void* h_counter_table_new(int sets_per_device, int listed) { return new onellm::CounterSets("test table", sets_per_device, listed != 0); }
+void h_counter_table_delete(void* t) { delete static_cast<onellm::CounterSets*>(t); }
+int h_counter_table_acquire(void* t, int device, void* workspace, int capturing)
+{
+    return static_cast<onellm::CounterSets*>(t)->acquire(device, workspace, capturing != 0);
+}
+int h_counter_table_release(void* t, void* workspace) { return static_cast<onellm::CounterSets*>(t)->release(workspace); }
+void h_counter_table_stats(void* t, int device, int* owned, int* captured, long* fallbacks)
+{
+    const onellm::CounterSets::Stats s = static_cast<onellm::CounterSets*>(t)->stats(device);
+    *owned = s.owned;
+    *captured = s.captured;
+    *fallbacks = s.fallbacks;
 }
 
 }  // extern "C"

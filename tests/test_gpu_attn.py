@@ -202,11 +202,16 @@ def test_config2_llama7b_full_size(capi, ref, dev):
         assert torch.equal(out, out2)
 
 
-def test_config3_gqa_fused_equals_repeat_path(capi, ref, dev):
+@pytest.mark.parametrize("finish", ["merge_launch", "fused_finish"])
+def test_config3_gqa_fused_equals_repeat_path(capi, ref, dev, finish):
     # BASELINE config 3: fp16, B32, 32 q heads over 8 kv heads x 128, S 8192, lengths U[1024, 8192].
     # (i) reference-style: concat the new row, repeat KV to 32 heads, attend with Hkv == Hq;
     # (ii) fused: attend straight from the [B, 8, S, 128] cache.  Both against the oracle.
-    announce("attn config3 setup")
+    # `fused_finish` hands the library a zero-filled workspace with ONELLM_ATTN_ZEROED_WORKSPACE: the form the
+    # launcher shim always uses and bench.py times (balanced schedule, one workgroup per compute unit, the piece that
+    # arrives last merges its unit inside the attention kernel); `merge_launch` is the plain call (a second launch).
+    announce("attn config3 setup", finish)
+    flags = capi.ATTN_ZEROED_WORKSPACE if finish == "fused_finish" else 0
     torch.manual_seed(3)
     B, Hq, Hkv, D, S = 32, 32, 8, 128, 8192
     G = Hq // Hkv
@@ -224,9 +229,19 @@ def test_config3_gqa_fused_equals_repeat_path(capi, ref, dev):
     announce("attn config3 fused")
     f_kc, f_vc = d_kc.clone(), d_vc.clone()
     out_f = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
-    capi.decode_attn(d_qkv, d_bias, f_kc, f_vc, out_f, Hq, int(t.max()), D, 10000.0, t_dev=d_t, max_t=int(t.max()))
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    capi.decode_attn(d_qkv, d_bias, f_kc, f_vc, out_f, Hq, int(t.max()), D, 10000.0, t_dev=d_t, max_t=int(t.max()),
+                     flags=flags, workspace=ws)
     np.testing.assert_allclose(out_f.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[np.float16])
     assert np.array_equal(_bits(f_kc.cpu().numpy()), _bits(r_kc)) and np.array_equal(_bits(f_vc.cpu().numpy()), _bits(r_vc))
+    if flags:
+        # the fused finish leaves its arrival counters (the first 64 KiB of the workspace) at zero, and a second
+        # step on the same workspace gives the same bits
+        assert int(ws[:64 * 1024].view(torch.int32).abs().max().item()) == 0
+        out_f2 = torch.zeros_like(out_f)
+        capi.decode_attn(d_qkv, d_bias, f_kc, f_vc, out_f2, Hq, int(t.max()), D, 10000.0, t_dev=d_t, max_t=int(t.max()),
+                         flags=flags, workspace=ws)
+        assert torch.equal(out_f, out_f2)
     # (i) repeat path on the cache that already holds the new rows: broadcast to 32 heads, then a
     # 32-head attention that re-derives the same new row (written again, same bits)
     announce("attn config3 repeat path")
@@ -239,7 +254,9 @@ def test_config3_gqa_fused_equals_repeat_path(capi, ref, dev):
     b3 = d_bias.view(Hq + 2 * Hkv, D)
     bias_r = torch.cat([b3[:Hq], b3[Hq:Hq + Hkv].repeat_interleave(G, 0), b3[Hq + Hkv:].repeat_interleave(G, 0)], 0).contiguous().view(-1)
     out_r = torch.zeros_like(out_f)
-    capi.decode_attn(qkv_r, bias_r, rk, rv, out_r, Hq, int(t.max()), D, 10000.0, t_dev=d_t, max_t=int(t.max()))
+    ws_r = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hq, D, S), dtype=torch.uint8, device=dev)
+    capi.decode_attn(qkv_r, bias_r, rk, rv, out_r, Hq, int(t.max()), D, 10000.0, t_dev=d_t, max_t=int(t.max()),
+                     flags=flags, workspace=ws_r)
     np.testing.assert_allclose(out_r.cpu().numpy().astype(np.float64), want.astype(np.float64), **TOL[np.float16])
     # same rows, same arithmetic per row group => the two paths agree far inside the tolerance
     assert (out_r.float() - out_f.float()).abs().max().item() <= 2e-3

@@ -284,18 +284,43 @@ def test_topk_one_launch_repeats_on_one_workspace_and_falls_back_past_its_limits
         np.testing.assert_array_equal(fi.cpu().numpy(), want[3], err_msg="call %d" % it)
         np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), want[2].view(np.uint32), err_msg="call %d" % it)
     assert launches == {1}, launches
+    assert capi.beam_topk_last_path() == capi.TOPK_PATH_ONE_LAUNCH
+    # More workspaces alive than the library has counter sets (64 per GPU): the ones that come too late take two
+    # launches and say why; nobody's set is taken from it; released sets are handed out again.
     B, beam, K, d, want = cases[0]
     held = [torch.empty(capi.beam_topk_workspace_bytes(B, beam, K) // 4, dtype=torch.float32, device=dev) for _ in range(80)]
+    fallbacks = capi.counter_set_fallbacks()
     seen = []
-    for w in held:
-        _, _, _, fv, fi = capi.beam_topk(d, B, beam, K, workspace=w)
-        seen.append(capi.beam_topk_last_launches())
-        np.testing.assert_array_equal(fi.cpu().numpy(), want[3])
-        np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), want[2].view(np.uint32))
-    assert seen[-1] == 2 and set(seen) == {1, 2}, seen
-    # a workspace the table knows keeps its one-launch form
-    capi.beam_topk(d, B, beam, K, workspace=big)
-    assert capi.beam_topk_last_launches() == 1
+    try:
+        for w in held:
+            _, _, _, fv, fi = capi.beam_topk(d, B, beam, K, workspace=w)
+            seen.append((capi.beam_topk_last_launches(), capi.beam_topk_last_path()))
+            np.testing.assert_array_equal(fi.cpu().numpy(), want[3])
+            np.testing.assert_array_equal(fv.cpu().numpy().view(np.uint32), want[2].view(np.uint32))
+        served = seen.count((1, capi.TOPK_PATH_ONE_LAUNCH))
+        assert 1 <= served <= 63, seen                     # (`big` holds a set as well)
+        assert seen == [(1, capi.TOPK_PATH_ONE_LAUNCH)] * served + [(2, capi.TOPK_PATH_NO_COUNTER_SET)] * (80 - served), seen
+        assert capi.counter_set_fallbacks() == fallbacks + 80 - served
+        # workspaces the table knows keep their one-launch form
+        for w in (big, held[0], held[served - 1]):
+            capi.beam_topk(d, B, beam, K, workspace=w)
+            assert capi.beam_topk_last_path() == capi.TOPK_PATH_ONE_LAUNCH
+        # one set given back serves exactly one newcomer
+        assert capi.release_workspace(held[0]) == 1 and capi.release_workspace(held[0]) == 0
+        for w, path in ((held[79], capi.TOPK_PATH_ONE_LAUNCH), (held[78], capi.TOPK_PATH_NO_COUNTER_SET),
+                        (held[0], capi.TOPK_PATH_NO_COUNTER_SET)):
+            _, _, _, fv, fi = capi.beam_topk(d, B, beam, K, workspace=w)
+            assert capi.beam_topk_last_path() == path
+            np.testing.assert_array_equal(fi.cpu().numpy(), want[3])
+        # a stream under capture never needs a set
+        capi.tune_set("topk_two_launches", 1)
+        capi.beam_topk(d, B, beam, K, workspace=held[77])
+        assert capi.beam_topk_last_path() == capi.TOPK_PATH_TWO_LAUNCHES
+    finally:
+        capi.tune_set("topk_two_launches", -1)
+        torch.cuda.synchronize()
+        for w in held:
+            capi.release_workspace(w)
 
 
 @pytest.mark.parametrize("forced_one_launch", [False, True])
@@ -334,3 +359,6 @@ def test_topk_graph_replays(capi, ref, dev, forced_one_launch):
         np.testing.assert_array_equal(fv.view(np.uint32), want[2].view(np.uint32), err_msg="replay %d" % rep)
         _, _, _, _, fi2 = capi.beam_topk(d, B, beam, K, workspace=ws)      # eager, same counters
         np.testing.assert_array_equal(fi2.cpu().numpy(), want[3])
+    torch.cuda.synchronize()
+    del g
+    assert capi.release_workspace(ws) == 1

@@ -72,7 +72,8 @@ def test_layers_library_exports_its_c_surface(H):
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = sorted(set(re.findall(r"\b(onellm_[a-z0-9_]+)\s*\(", text)))
     assert names == ["onellm_decoder_create", "onellm_decoder_destroy", "onellm_decoder_forward", "onellm_layers_allow_plain_gemm",
-                     "onellm_layers_gemm_workspace_count", "onellm_layers_last_error", "onellm_layers_linear"]
+                     "onellm_layers_gemm_workspace_count", "onellm_layers_last_error", "onellm_layers_linear",
+                     "onellm_layers_release_gemm_workspace"]
     for n in names:
         assert hasattr(H, n)
 
@@ -279,9 +280,13 @@ def test_few_row_kernel_cut_runs_back_to_back_on_one_workspace(G, ref):
         assert len(keys) >= 40, len(keys)
         order = [keys[i] for i in rng.integers(0, len(keys), size=300)]
         outs = []
-        for si, variant, splits in order:
+        for n, (si, variant, splits) in enumerate(order):
             M, K, N, dx, dw, _ = ops[si]
             capi.tune_set("gemm_skinny_config", 100 * variant + splits)
+            # every fifth call hands its sums over in the formally ordered way (release on the counter add, acquire
+            # fence in the slice that reads them back); the default relies on written-through stores and an add
+            # executed at memory.  Same sums in the same order: same bits.
+            capi.tune_set("gemm_ordered_finish", 1 if n % 5 == 4 else -1)
             y = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
             capi.linear(dx, dw, y, workspace=ws)
             outs.append(y)
@@ -291,6 +296,57 @@ def test_few_row_kernel_cut_runs_back_to_back_on_one_workspace(G, ref):
     finally:
         capi.tune_set("gemm_skinny", -1)
         capi.tune_set("gemm_skinny_config", -1)
+        capi.tune_set("gemm_ordered_finish", -1)
+
+
+@pytest.mark.gpu
+def test_few_row_kernel_without_a_free_counter_set_runs_uncut_and_says_so(G, ref):
+    """A run cut along K counts its slices in one of the library's 128 counter sets per GPU, owned by the workspace
+    from its first cut run on.  The 129th workspace gets none: the call runs the same kernel uncut (path 4), with the
+    same result to the tolerance, never with somebody else's counters; after onellm_release_workspace of one owner
+    the next workspace is served again."""
+    import torch
+    from onellm_amd import capi
+    announce("few-row linear, counter sets exhausted")
+    rng = np.random.default_rng(12)
+    dev = torch.device("cuda:0")
+    M, K, N = 16, 1024, 512
+    x = (rng.standard_normal((M, K)) * 0.5).astype(np.float16)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+    want = ref.linear(x, w).astype(np.float64)
+    dx, dw = _dev(torch, x), _dev(torch, w)
+    # one allocation cut into 1 MiB workspaces: distinct pointers, all alive (what the kernel needs here is 256 KiB)
+    pool = torch.empty(140 << 20, dtype=torch.uint8, device=dev)
+    spaces = [pool[i << 20:(i + 1) << 20] for i in range(140)]
+    capi.tune_set("gemm_skinny", 1)
+    capi.tune_set("gemm_skinny_config", 100 * 0 + 4)
+    fallbacks = capi.counter_set_fallbacks()
+    try:
+        paths = []
+        for ws in spaces[:132]:
+            y = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+            capi.linear(dx, dw, y, workspace=ws)
+            paths.append(G.onellm_linear_last_path())
+            np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), want, **TOL[np.float16])
+        owners = paths.count(2)
+        assert 1 <= owners <= 128 and paths[:owners] == [2] * owners and set(paths[owners:]) == {4}, paths
+        assert capi.counter_set_fallbacks() == fallbacks + (132 - owners)
+        # an owner keeps being served while strangers are turned away
+        y = torch.zeros((M, N), dtype=torch.float16, device=dev)
+        capi.linear(dx, dw, y, workspace=spaces[0])
+        assert G.onellm_linear_last_path() == 2
+        # give one set back: exactly one more workspace can run cut
+        assert capi.release_workspace(spaces[1]) == 1
+        for ws, expect in ((spaces[135], 2), (spaces[136], 4), (spaces[1], 4)):
+            y = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+            capi.linear(dx, dw, y, workspace=ws)
+            assert G.onellm_linear_last_path() == expect
+            np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), want, **TOL[np.float16])
+    finally:
+        capi.tune_set("gemm_skinny", -1)
+        capi.tune_set("gemm_skinny_config", -1)
+        for ws in spaces:
+            capi.release_workspace(ws)
 
 
 @pytest.mark.gpu
@@ -400,9 +456,21 @@ STEP_TOL = {np.float32: dict(rtol=2e-4, atol=2e-4), np.float16: dict(rtol=3e-2, 
     (np.float16, 2, 32, 32, 128, 1408, 1, 64, 64, 128),
     (np.float16, 1, 4, 4, 64, 96, 3, 16, 1, 64),
 ])
-def test_decoder_step_matches_the_oracle(H, ref, dtype, B, Hq, Hkv, D, I, L, S, t, rotary):
+@pytest.mark.parametrize("projections", ["tuned", "library_only"])
+def test_decoder_step_matches_the_oracle(H, ref, dtype, B, Hq, Hkv, D, I, L, S, t, rotary, projections):
+    """`library_only` (tuning key gemm_skinny = 0) is the path the task statement names: every projection on hipBLASLt.
+    `tuned` lets the tuning run pick this library's few-row kernel where it measured faster (an extension)."""
     import torch
-    announce("decoder step", dtype.__name__, B, Hq, Hkv, D, I, L, S, "t", t)
+    from onellm_amd import capi
+    announce("decoder step", dtype.__name__, B, Hq, Hkv, D, I, L, S, "t", t, projections)
+    capi.tune_set("gemm_skinny", 0 if projections == "library_only" else -1)
+    try:
+        _decoder_step_case(H, ref, torch, dtype, B, Hq, Hkv, D, I, L, S, t, rotary)
+    finally:
+        capi.tune_set("gemm_skinny", -1)
+
+
+def _decoder_step_case(H, ref, torch, dtype, B, Hq, Hkv, D, I, L, S, t, rotary):
     rng = np.random.default_rng(B * 1000 + Hq * 10 + t)
     hidden, eps = Hq * D, 1e-5
     layers = _random_layers(rng, dtype, Hq, Hkv, D, I, L)
@@ -651,5 +719,15 @@ def test_gemm_workspace_is_per_launch_stream_and_never_created_under_capture(H):
         assert run() == 0                                            # an ordinary call afterwards is fine
         torch.cuda.synchronize()
         assert torch.equal(y, want)
+        # a stream that is about to be destroyed gives its workspace (and that workspace's counter sets) back
+        count = H.onellm_layers_gemm_workspace_count()
+        assert H.onellm_layers_release_gemm_workspace(ctypes.c_void_p(s1.cuda_stream)) == 1
+        assert H.onellm_layers_release_gemm_workspace(ctypes.c_void_p(s1.cuda_stream)) == 0
+        assert H.onellm_layers_gemm_workspace_count() == count - 1
+        harness.h_set_launch_stream(s1.cuda_stream)                  # ... and gets a new one if it is used again after all
+        assert run() == 0, H.onellm_layers_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)
+        assert H.onellm_layers_gemm_workspace_count() == count
     finally:
         harness.h_set_launch_stream(None)
