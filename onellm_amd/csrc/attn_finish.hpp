@@ -7,75 +7,142 @@
 namespace onellm {
 namespace {
 
-// q of the tile's heads (and, in the last split, the new k/v row): bias, RoPE, staging in LDS; the
-// last split also stores the new row to the cache and leaves its scores in snew.  Ends with the
-// whole workgroup synchronised on sq / sk / sv (snew is ready after the caller's next barrier).
-template <typename T, int D, int GT, int NTHR>
-__device__ __forceinline__ void stage_q_and_new_row(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, T* kc, T* vc,
-                                                    float* sq, float* sk, float* sv, float* snew)
+// Two consecutive elements of a row fetched with one access, and one element fetched into a register of its own.
+// (Two fp16 loads that fill the two halves of one register depend on each other - the second has to wait for the first
+// to land - so element-by-element loads of a pair cost a memory round trip each; a 32-bit load of the pair, and a
+// zero-extending 16-bit load of a single element, keep every load of the set-up independent of the others.)
+template <typename T> struct RawPair;
+template <> struct RawPair<__half> {
+    unsigned w = 0;
+    __device__ __forceinline__ float first() const { return __half2float(__ushort_as_half((unsigned short)(w & 0xFFFFu))); }
+    __device__ __forceinline__ float second() const { return __half2float(__ushort_as_half((unsigned short)(w >> 16))); }
+};
+template <> struct RawPair<float> {
+    float a = 0.f, b = 0.f;
+    __device__ __forceinline__ float first() const { return a; }
+    __device__ __forceinline__ float second() const { return b; }
+};
+__device__ __forceinline__ RawPair<__half> load_pair(const __half* p)
 {
+    RawPair<__half> r;
+    r.w = *reinterpret_cast<const unsigned*>(p);
+    return r;
+}
+__device__ __forceinline__ RawPair<float> load_pair(const float* p)
+{
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const f32x2 v = *reinterpret_cast<const f32x2*>(p);
+    RawPair<float> r;
+    r.a = v[0];
+    r.b = v[1];
+    return r;
+}
+template <typename T> struct RawOne;
+template <> struct RawOne<__half> {
+    unsigned w = 0;
+    __device__ __forceinline__ float value() const { return __half2float(__ushort_as_half((unsigned short)w)); }
+};
+template <> struct RawOne<float> {
+    float v = 0.f;
+    __device__ __forceinline__ float value() const { return v; }
+};
+__device__ __forceinline__ RawOne<__half> load_one(const __half* p)
+{
+    RawOne<__half> r;
+    r.w = *reinterpret_cast<const unsigned short*>(p);
+    return r;
+}
+__device__ __forceinline__ RawOne<float> load_one(const float* p)
+{
+    RawOne<float> r;
+    r.v = *p;
+    return r;
+}
+
+// What a unit's set-up reads from memory - q of the tile's heads and, in the unit's last piece, the new k and v row,
+// each with its bias - as it sits in registers between the request and the use.  Everything is requested before
+// any of it is used or anything is stored: one memory round trip instead of three in a row (q; then k behind the
+// stores of q's results; then v), which every workgroup pays before its first score (5.0 -> 2.4 us after entry
+// with cold caches at 32 heads x 128).  The matrix-core kernels request the next unit's rows while the current
+// unit is still being finished, so that round trip disappears from a change of unit altogether.
+// (qkv and bias must be aligned to a pair of elements: the tiled kernels are only taken for such pointers)
+template <typename T, int D, int GT, int NTHR>
+struct SetupRows {
+    static constexpr int QI = (GT * (D / 2) + NTHR - 1) / NTHR;      // q pairs per thread
+    static constexpr int KI = (D / 2 + NTHR - 1) / NTHR;             // k pairs per thread
+    static constexpr int VI = (D + NTHR - 1) / NTHR;                 // v elements per thread
+    RawPair<T> q[QI], qb[QI], k[KI], kb[KI];
+    RawOne<T> v[VI], vb[VI];
+};
+
+template <typename T, int D, int GT, int NTHR>
+__device__ __forceinline__ void request_setup_rows(const AttnArgs& a, const Unit& u, SetupRows<T, D, GT, NTHR>& r)
+{
+    using R = SetupRows<T, D, GT, NTHR>;
     const int tid = lane_id_per_unit();
     const T* qkv = static_cast<const T*>(a.qkv) + (size_t)u.b * (a.Hq + 2 * a.Hkv) * D;
     const T* bias = static_cast<const T*>(a.bias);
-    // Everything this set-up reads from memory - q, the new k and v row, their biases - is requested before any
-    // of it is used or anything is stored: one memory round trip instead of three in a row (q; then k behind the
-    // stores of q's results; then v), which every workgroup pays before its first score (5.0 -> 2.4 us after
-    // entry with cold caches at 32 heads x 128).
-    constexpr int QI = (GT * (D / 2) + NTHR - 1) / NTHR;      // q pairs per thread
-    constexpr int KI = (D / 2 + NTHR - 1) / NTHR;             // k pairs per thread
-    constexpr int VI = (D + NTHR - 1) / NTHR;                 // v elements per thread
-    T q0[QI], q1[QI], qb0[QI], qb1[QI], k0[KI], k1[KI], kb0[KI], kb1[KI], v0[VI], vb0[VI];
     const bool v_bias = bias && !(a.flags & ONELLM_ATTN_NO_V_BIAS);
 #pragma unroll
-    for (int k = 0; k < QI; ++k) {
+    for (int k = 0; k < R::QI; ++k) {
         const int i = tid + k * NTHR;
         const int g = i / (D / 2), p = i % (D / 2);
-        q0[k] = q1[k] = qb0[k] = qb1[k] = from_f32<T>(0.f);
+        r.q[k] = RawPair<T>();
+        r.qb[k] = RawPair<T>();
         if (i < GT * (D / 2) && u.g0 + g < a.G) {
             const int o = (u.kvh * a.G + u.g0 + g) * D + 2 * p;
-            q0[k] = qkv[o];
-            q1[k] = qkv[o + 1];
-            if (bias) {
-                qb0[k] = bias[o];
-                qb1[k] = bias[o + 1];
-            }
+            r.q[k] = load_pair(qkv + o);
+            if (bias) r.qb[k] = load_pair(bias + o);
         }
     }
     if (u.is_last) {
 #pragma unroll
-        for (int k = 0; k < KI; ++k) {
+        for (int k = 0; k < R::KI; ++k) {
             const int p = tid + k * NTHR;
-            k0[k] = k1[k] = kb0[k] = kb1[k] = from_f32<T>(0.f);
+            r.k[k] = RawPair<T>();
+            r.kb[k] = RawPair<T>();
             if (p < D / 2) {
                 const int o = (a.Hq + u.kvh) * D + 2 * p;
-                k0[k] = qkv[o];
-                k1[k] = qkv[o + 1];
-                if (bias) {
-                    kb0[k] = bias[o];
-                    kb1[k] = bias[o + 1];
-                }
+                r.k[k] = load_pair(qkv + o);
+                if (bias) r.kb[k] = load_pair(bias + o);
             }
         }
 #pragma unroll
-        for (int k = 0; k < VI; ++k) {
+        for (int k = 0; k < R::VI; ++k) {
             const int d = tid + k * NTHR;
-            v0[k] = vb0[k] = from_f32<T>(0.f);
+            r.v[k] = RawOne<T>();
+            r.vb[k] = RawOne<T>();
             if (d < D) {
                 const int o = (a.Hq + a.Hkv + u.kvh) * D + d;
-                v0[k] = qkv[o];
-                if (v_bias) vb0[k] = bias[o];
+                r.v[k] = load_one(qkv + o);
+                if (v_bias) r.vb[k] = load_one(bias + o);
             }
         }
     }
+    // (the requests stay here: the compiler may not move a load past this point towards its use)
+    asm volatile("" ::: "memory");
+}
+
+// The set-up proper, from the requested rows: bias, RoPE, staging in LDS; the last piece also stores the new row
+// to the cache and leaves its scores in snew.  Ends with the whole workgroup synchronised on sq / sk / sv (snew is
+// ready after the caller's next barrier).
+template <typename T, int D, int GT, int NTHR>
+__device__ __forceinline__ void stage_setup_rows(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, const SetupRows<T, D, GT, NTHR>& r,
+                                                 T* kc, T* vc, float* sq, float* sk, float* sv, float* snew)
+{
+    using R = SetupRows<T, D, GT, NTHR>;
+    const int tid = lane_id_per_unit();
+    const T* bias = static_cast<const T*>(a.bias);
+    const bool v_bias = bias && !(a.flags & ONELLM_ATTN_NO_V_BIAS);
 #pragma unroll
-    for (int k = 0; k < QI; ++k) {
+    for (int k = 0; k < R::QI; ++k) {
         const int i = tid + k * NTHR;
         if (i < GT * (D / 2)) {
             const int g = i / (D / 2), p = i % (D / 2);
-            float x0 = to_f32(q0[k]), x1 = to_f32(q1[k]);     // (zeros for a head past the group's end)
+            float x0 = r.q[k].first(), x1 = r.q[k].second();     // (zeros for a head past the group's end)
             if (bias) {
-                x0 += to_f32(qb0[k]);
-                x1 += to_f32(qb1[k]);
+                x0 += r.qb[k].first();
+                x1 += r.qb[k].second();
             }
             if (u.g0 + g < a.G && 2 * p < a.rotary_dim) rope_pair(x0, x1, p, u.pos, fr);
             sq[g * D + 2 * p] = x0 * a.qscale;
@@ -85,13 +152,13 @@ __device__ __forceinline__ void stage_q_and_new_row(const AttnArgs& a, const Rop
     if (u.is_last) {
         const bool store = u.g0 == 0 && !(a.flags & ONELLM_ATTN_NO_CACHE_WRITE);
 #pragma unroll
-        for (int k = 0; k < KI; ++k) {
+        for (int k = 0; k < R::KI; ++k) {
             const int p = tid + k * NTHR;
             if (p < D / 2) {
-                float x0 = to_f32(k0[k]), x1 = to_f32(k1[k]);
+                float x0 = r.k[k].first(), x1 = r.k[k].second();
                 if (bias) {
-                    x0 += to_f32(kb0[k]);
-                    x1 += to_f32(kb1[k]);
+                    x0 += r.kb[k].first();
+                    x1 += r.kb[k].second();
                 }
                 if (2 * p < a.rotary_dim) rope_pair(x0, x1, p, u.pos, fr);
                 const T r0 = from_f32<T>(x0), r1 = from_f32<T>(x1);
@@ -104,11 +171,11 @@ __device__ __forceinline__ void stage_q_and_new_row(const AttnArgs& a, const Rop
             }
         }
 #pragma unroll
-        for (int k = 0; k < VI; ++k) {
+        for (int k = 0; k < R::VI; ++k) {
             const int d = tid + k * NTHR;
             if (d < D) {
-                float x = to_f32(v0[k]);
-                if (v_bias) x += to_f32(vb0[k]);
+                float x = r.v[k].value();
+                if (v_bias) x += r.vb[k].value();
                 const T v = from_f32<T>(x);
                 sv[d] = to_f32(v);
                 if (store) vc[(size_t)(u.t - 1) * D + d] = v;
@@ -116,16 +183,27 @@ __device__ __forceinline__ void stage_q_and_new_row(const AttnArgs& a, const Rop
         }
     }
     __syncthreads();
-    if (u.is_last && tid < kWave) {
-        const int lane = tid;
-#pragma unroll
-        for (int g = 0; g < GT; ++g) {
+    if (u.is_last) {
+        // the new row's score with each head of the tile: the heads are dealt to the waves (one wave doing them all
+        // in turn started its rows a microsecond after the others, and the unit's finish waits for the last wave)
+        const int lane = tid & (kWave - 1);
+        for (int g = tid / kWave; g < GT; g += NTHR / kWave) {
             float part = 0.f;
             for (int d = lane; d < D; d += kWave) part = fmaf(sq[g * D + d], sk[d], part);
             part = wave_sum(part);
             if (lane == 0) snew[g] = part;
         }
     }
+}
+
+// request + set-up in one go (the kernels that do not look ahead to their next unit)
+template <typename T, int D, int GT, int NTHR>
+__device__ __forceinline__ void stage_q_and_new_row(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, T* kc, T* vc,
+                                                    float* sq, float* sk, float* sv, float* snew)
+{
+    SetupRows<T, D, GT, NTHR> rows;
+    request_setup_rows<T, D, GT, NTHR>(a, u, rows);
+    stage_setup_rows<T, D, GT, NTHR>(a, fr, u, rows, kc, vc, sq, sk, sv, snew);
 }
 
 // device-scope accesses for data that workgroups on different chip quarters hand to each other

@@ -33,8 +33,9 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 template <int D, int GT, int NW, bool DOUBLE_BUFFER>
-__device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds)
+__device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds, int& ev)
 {
+    stamp_event(a, ev);
     using T = __half;
     static_assert(GT == 4 || GT == 8 || GT == 16, "heads per tile");
     static_assert(D == 64 || D == 128 || D == 256, "head size");
@@ -100,6 +101,7 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
                 }
     }
 
+    stamp_event(a, ev);
     // per lane: head (lane % GT); m is the same in every lane of a head, l is this lane's share
     float m = -INFINITY, l = 0.f;
     f32x4 o[CG * VEC];                          // o[cg*8 + c][r]: head (4*grp + r) % GT, column (cg*16 + slot)*8 + c
@@ -214,6 +216,7 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
         }
     }
 
+    stamp_event(a, ev);
     // ---- one state per wave: l is summed over the four row quarters, o is already complete
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
@@ -232,6 +235,288 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
     }
     __syncthreads();
     finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv, look);
+    stamp_event(a, ev);
+}
+
+// ---- the unit of the grid schedule with two register buffers (D = 64, 128): one unit per workgroup.
+//
+// Differences from gqa_mfma_unit above, each measured on MI355X:
+//   * a unit's last, partial batch of rows (read from the last valid row where it reaches past the end, and masked)
+//     goes through the same two buffers as the full ones instead of being asked for after the last full batch was
+//     consumed - a memory round trip with nothing else in flight at the end of every unit;
+//   * the second batch sets out right behind the set-up instead of inside the loop;
+//   * while two more full batches lie ahead, the loop holds nothing conditional, so the compiler waits for exactly
+//     the loads a product needs (with a conditional request in the loop it waits for all loads: both buffers).
+// 4 sequences x 8 kv heads of 8192 rows in eight pieces each 28.1 -> 26.8 us; 8 sequences of 256..2048 rows 16.4 ->
+// 15.4; 64 q / 8 kv heads x 16 sequences x 8192 rows 85.4 -> 83.7; 32 sequences x 8 kv heads x 8192 rows 153.6 -> 152.0.
+// The balanced schedule keeps gqa_mfma_unit: the same loop inside its walk over several units measured 0.5-2.5 us
+// slower there (config 3 ragged 93.3 -> 93.9, 96 sequences of 256..2048 rows 80.9 -> 83.3) - the schedule state of two
+// units no longer fits the scalar registers.  Also built and measured there, and not kept: asking for the next piece's
+// rows before the current piece is finished, at the end of its streaming loop or right behind the counter add of a
+// piece that is handed over.  A piece's finish waits for its stores to be acknowledged with `s_waitcnt vmcnt(0)`,
+// which also waits for every load in flight (64 KiB per workgroup: the finish went from 2.5 to 4.7-5.8 us and ate what
+// the set-up saved), and the registers that stay live across the finish cost the second wave per SIMD (96 sequences
+// of 256..2048 rows: 80 -> 105 us).
+template <int D>
+struct KvBatch {
+    static constexpr int NKJ = D / 32;
+    static constexpr int CG = D > 128 ? D / 128 : 1;
+    Vec16<__half> k[NKJ], v[CG * 4];
+};
+
+// A lane's place in a unit's K and V rows: K, lane (slot, grp): row `slot` of the wave's 16, 16-byte pieces
+// grp + 4 * j; V, lane (slot, grp): rows 4 * grp + e, columns (cg * 16 + slot) * 8 .. + 7.  Worked out once per unit.
+template <int D>
+struct KvLane {
+    const __half* kp;       // row `wave * 16 + slot` of the unit's K rows, piece grp
+    const __half* vp;       // row `wave * 16 + 4 * grp` of its V rows, this lane's columns
+    int row0;               // wave * 16
+    int slot, grp;
+};
+
+template <int D>
+__device__ __forceinline__ KvLane<D> kv_lane(const __half* kc, const __half* vc)
+{
+    constexpr int VEC = 8, VSLOTS = D / VEC < 16 ? D / VEC : 16;
+    const int tid = lane_id_per_unit();
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    KvLane<D> p;
+    p.slot = lane & 15;
+    p.grp = lane >> 4;
+    p.row0 = wave * 16;
+    p.kp = kc + (size_t)(p.row0 + p.slot) * D + p.grp * VEC;
+    p.vp = vc + (size_t)(p.row0 + 4 * p.grp) * D + (p.slot % VSLOTS) * VEC;
+    return p;
+}
+
+// rows [rbase, rbase + NW * 16) of a unit whose rows end at r1, into `r`; a batch that reaches past r1 reads the last
+// valid row instead (the caller masks those scores)
+template <int D>
+__device__ __forceinline__ void issue_full_batch(KvBatch<D>& r, const KvLane<D>& p, int rbase)
+{
+    constexpr int NKJ = D / 32, CG = D > 128 ? D / 128 : 1;
+    const __half* kp = p.kp + (size_t)rbase * D;
+    const __half* vp = p.vp + (size_t)rbase * D;
+#pragma unroll
+    for (int j = 0; j < NKJ; ++j) r.k[j] = load16_stream(kp + j * 32);
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r.v[cg * 4 + e] = load16_stream(vp + (size_t)e * D + cg * 128);
+}
+
+template <int D, int NW>
+__device__ __forceinline__ void issue_batch(KvBatch<D>& r, const KvLane<D>& p, int rbase, int r1)
+{
+    constexpr int NKJ = D / 32, CG = D > 128 ? D / 128 : 1;
+    if (rbase + NW * 16 <= r1) {
+        issue_full_batch<D>(r, p, rbase);
+    } else {
+        // (p.kp / p.vp point at rows row0 + slot / row0 + 4 * grp of the unit: step back or forth to the clamped row)
+        const int krow = min(rbase + p.row0 + p.slot, r1 - 1) - (p.row0 + p.slot);
+#pragma unroll
+        for (int j = 0; j < NKJ; ++j) r.k[j] = load16_stream(p.kp + (ptrdiff_t)krow * D + j * 32);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int vrow = min(rbase + p.row0 + 4 * p.grp + e, r1 - 1) - (p.row0 + 4 * p.grp);
+#pragma unroll
+            for (int cg = 0; cg < CG; ++cg) r.v[cg * 4 + e] = load16_stream(p.vp + (ptrdiff_t)vrow * D + cg * 128);
+        }
+    }
+}
+
+template <int D, int GT, int NW>
+__device__ __forceinline__ void gqa_mfma_grid_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds, int& ev)
+{
+    using T = __half;
+    static_assert(GT == 4 || GT == 8 || GT == 16, "heads per tile");
+    static_assert(D == 64 || D == 128, "head size (two register buffers)");
+    constexpr int VEC = 8;
+    constexpr int NKB = D / 16;                 // k-blocks of the score product
+    constexpr int NKJ = D / 32;                 // 16-byte pieces of a K row per lane
+    constexpr int CG = 1;
+    constexpr int VSLOTS = D / VEC < 16 ? D / VEC : 16;
+    constexpr int NTHR = NW * kWave;
+    constexpr int RPI = NW * 16;                // rows per batch
+
+    float* sq = lds;                            // [GT][D]
+    float* sk = sq + GT * D;                    // [D]
+    float* sv = sk + D;                         // [D]
+    float* snew = sv + D;                       // [GT]
+    float* st_ml = snew + GT;                   // [NW][GT][2]
+    float* st_acc = st_ml + NW * GT * 2;        // [NW][GT][D]
+
+    auto cache_of = [&](const Unit& x, T*& kc, T*& vc) {
+        const size_t head_off = a.slab + ((size_t)x.b * a.Hkv + x.kvh) * (size_t)a.S * D;
+        kc = static_cast<T*>(a.k_cache) + head_off;
+        vc = static_cast<T*>(a.v_cache) + head_off;
+    };
+    auto batches_of = [](const Unit& x) { return x.r1 > x.r0 ? (x.r1 - x.r0 + RPI - 1) / RPI : 0; };
+
+    KvBatch<D> ba, bb;
+    {
+        stamp_event(a, ev);
+        const int tid = lane_id_per_unit();
+        const int lane = tid & (kWave - 1);
+        const int wave = tid / kWave;
+        const int slot = lane & 15;
+        const int grp = lane >> 4;
+        const int r0 = u.r0, r1 = u.r1;
+        T *kc, *vc;
+        cache_of(u, kc, vc);
+        const KvLane<D> at = kv_lane<D>(kc, vc);
+        const int nb = batches_of(u);
+        const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
+
+        // the first batch of rows sets out before the set-up's own loads, the second behind them (the set-up then
+        // waits for one batch, not two)
+        if (nb > 0) issue_batch<D, NW>(ba, at, r0, r1);
+        {
+            SetupRows<T, D, GT, NTHR> rows;
+            request_setup_rows<T, D, GT, NTHR>(a, u, rows);
+            stage_setup_rows<T, D, GT, NTHR>(a, fr, u, rows, kc, vc, sq, sk, sv, snew);
+        }
+        if (nb > 1) issue_batch<D, NW>(bb, at, r0 + RPI, r1);
+
+        // B operand of the score product: column (lane % 16) is head (lane % GT); k slots 4*grp + e of
+        // k-block (jp, h) are the columns grp*8 + jp*32 + 4*h + e - the ones the K registers hold there
+        f16x4 qhi[NKB], qlo[NKB];
+        {
+            const float* qh = sq + (lane % GT) * D + grp * VEC;
+#pragma unroll
+            for (int jp = 0; jp < NKJ; ++jp)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float v = qh[jp * 32 + 4 * h + e];
+                        const _Float16 hi = (_Float16)v;
+                        qhi[jp * 2 + h][e] = hi;
+                        qlo[jp * 2 + h][e] = (_Float16)(v - (float)hi);
+                    }
+        }
+
+        stamp_event(a, ev);
+        float m = -INFINITY, l = 0.f;           // per lane: head (lane % GT); m is the same in every lane of a head, l this lane's share
+        f32x4 o[CG * VEC];                      // o[c][r]: head (4*grp + r) % GT, column slot*8 + c
+#pragma unroll
+        for (int c = 0; c < CG * VEC; ++c) o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        auto consume = [&](const KvBatch<D>& kv, int rbase, auto masked_tag) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
+            f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int jp = 0; jp < NKJ; ++jp) {
+                const f16x4 k0 = __builtin_shufflevector(kv.k[jp].raw, kv.k[jp].raw, 0, 1, 2, 3);
+                const f16x4 k1 = __builtin_shufflevector(kv.k[jp].raw, kv.k[jp].raw, 4, 5, 6, 7);
+                s0 = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qhi[jp * 2], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qlo[jp * 2], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qhi[jp * 2 + 1], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qlo[jp * 2 + 1], s1, 0, 0, 0);
+            }
+            // (rows past the unit's end - only in its last, partial batch - were read from the last valid row: masked here)
+            float s[4];
+            float bm = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                s[r] = s0[r] + s1[r];           // score of row 4*grp + r of the batch, head lane % GT
+                if constexpr (MASKED) s[r] = (rbase + wave * 16 + 4 * grp + r < r1) ? s[r] : -INFINITY;
+                bm = fmaxf(bm, s[r]);
+            }
+            if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+                bm = fmaxf(bm, __shfl_xor(bm, 16, kWave));
+                bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
+                const float mnew = fmaxf(m, bm);    // finite: some row of the wave's batch is valid
+                const float alpha = __builtin_amdgcn_exp2f(m - mnew);
+                l *= alpha;
+                // accumulator register r belongs to head (4*grp + r) % GT: fetch that head's factor from a
+                // lane that tracks it (lane % GT == head)
+                float al[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, (lane & 48) | ((4 * grp + r) % GT), kWave);
+#pragma unroll
+                for (int c = 0; c < CG * VEC; ++c)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[c][r] *= al[r];
+                m = mnew;
+            }
+            f16x4 phi, plo;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float p = __builtin_amdgcn_exp2f(s[r] - m);
+                l += p;
+                const _Float16 hi = (_Float16)p;
+                phi[r] = hi;
+                plo[r] = (_Float16)(p - (float)hi);
+            }
+            u32x4 vw[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vw[e] = __builtin_bit_cast(u32x4, kv.v[e].raw);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+                // column c of the four rows: one byte-permute per pair of rows
+                constexpr unsigned kLow = 0x05040100u, kHigh = 0x07060302u;
+                const unsigned sel = (c & 1) ? kHigh : kLow;
+                const u32x2 packed = {__builtin_amdgcn_perm(vw[1][c / 2], vw[0][c / 2], sel),
+                                      __builtin_amdgcn_perm(vw[3][c / 2], vw[2][c / 2], sel)};
+                const f16x4 vcol = __builtin_bit_cast(f16x4, packed);
+                o[c] = __builtin_amdgcn_mfma_f32_16x16x16f16(phi, vcol, o[c], 0, 0, 0);
+                o[c] = __builtin_amdgcn_mfma_f32_16x16x16f16(plo, vcol, o[c], 0, 0, 0);
+            }
+        };
+        // Batch k sits in buffer k % 2 (the first two were requested before this unit's set-up).  Full batches go in
+        // pairs; the last batch of a piece may be partial: a wave whose rows of it are all past the end must not touch
+        // its state (its scores would all be -inf).
+        int look = -1;                          // (fused finish: the other pieces' arrivals, asked near the end)
+        if (nfull == 0) look = first_look(a, u);
+        int k = 0;
+        // (while the two batches after the pair in flight are full ones, nothing in the loop is conditional: the
+        // compiler then waits for exactly the loads a product needs and leaves the other buffer's on their way)
+        for (; k + 4 <= nfull; k += 2) {
+            take_turns(a);
+            const int rbase = r0 + k * RPI;
+            consume(ba, rbase, std::false_type{});
+            issue_full_batch<D>(ba, at, rbase + 2 * RPI);
+            consume(bb, rbase + RPI, std::false_type{});
+            issue_full_batch<D>(bb, at, rbase + 3 * RPI);
+        }
+        for (; k < nfull; k += 2) {
+            take_turns(a);
+            if (k + 2 >= nfull) look = first_look(a, u);
+            const int rbase = r0 + k * RPI;
+            consume(ba, rbase, std::false_type{});
+            if (k + 2 < nb) issue_batch<D, NW>(ba, at, rbase + 2 * RPI, r1);
+            if (k + 1 < nfull) {
+                consume(bb, rbase + RPI, std::false_type{});
+                if (k + 3 < nb) issue_batch<D, NW>(bb, at, rbase + 3 * RPI, r1);
+            }
+        }
+        if (nb > nfull) {
+            const int rbase = r0 + nfull * RPI;
+            if (rbase + wave * 16 < r1) {
+                if (nfull & 1) consume(bb, rbase, std::true_type{});
+                else consume(ba, rbase, std::true_type{});
+            }
+        }
+
+        stamp_event(a, ev);
+        // ---- one state per wave: l is summed over the four row quarters, o is already complete
+        l += __shfl_xor(l, 16, kWave);
+        l += __shfl_xor(l, 32, kWave);
+        if (grp == 0 && slot < GT) {
+            st_ml[(wave * GT + slot) * 2] = m;
+            st_ml[(wave * GT + slot) * 2 + 1] = l;
+        }
+        if (4 * grp < GT && slot < VSLOTS) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) st_acc[(size_t)(wave * GT + 4 * grp + r) * D + slot * VEC + c] = o[c][r];
+        }
+        __syncthreads();
+        finish_unit<T, D, GT, NW, NTHR>(a, u, st_ml, st_acc, snew, sv, look);
+        stamp_event(a, ev);
+    }
 }
 
 template <int D, int GT, int NW, bool DOUBLE_BUFFER, bool BALANCED>
@@ -240,7 +525,13 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
 {
     extern __shared__ float lds[];
     stamp_entry(a);
-    for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_unit<D, GT, NW, DOUBLE_BUFFER>(a, fr, u, lds); });
+    int ev = 0;
+    if constexpr (DOUBLE_BUFFER && !BALANCED) {
+        Unit u;
+        if (locate_unit<GT>(a, u)) gqa_mfma_grid_unit<D, GT, NW>(a, fr, u, lds, ev);
+    } else {
+        for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_unit<D, GT, NW, DOUBLE_BUFFER>(a, fr, u, lds, ev); });
+    }
     stamp_end(a);
 }
 

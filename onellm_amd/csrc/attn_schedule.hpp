@@ -68,9 +68,22 @@ __device__ __forceinline__ void stamp_end(const AttnArgs& a)
         a.stamps[wg * 4 + 1] = wall_clock64();
     }
 }
+// phase stamps of the matrix-core kernels: behind the four words per workgroup, kStampEvents words per workgroup -
+// four per unit piece in the order it meets them (piece begun, set-up done, last row consumed, piece finished)
+constexpr int kStampEvents = 16;
+__device__ __forceinline__ void stamp_event(const AttnArgs& a, int& next)
+{
+    if (a.stamps && threadIdx.x == 0 && next < kStampEvents) {
+        const long long total = (long long)gridDim.x * gridDim.y * gridDim.z;
+        const long long wg = ((long long)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        a.stamps[total * 4 + wg * kStampEvents + next] = wall_clock64();
+    }
+    ++next;
+}
 #else
 __device__ __forceinline__ void stamp_entry(const AttnArgs&) {}
 __device__ __forceinline__ void stamp_end(const AttnArgs&) {}
+__device__ __forceinline__ void stamp_event(const AttnArgs&, int&) {}
 #endif
 
 // What one workgroup works on: a chunk of the history of one (sequence, kv-head) for up to GT query heads.
@@ -145,12 +158,7 @@ __device__ __forceinline__ int seq_items(const AttnArgs& a, int t)
 // The schedule is the same in every lane; saying so keeps it in scalar registers (the kernels that
 // walk it are short of vector registers).
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
-__device__ __forceinline__ long long uniform(long long v)
-{
-    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(unsigned long long)v);
-    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)((unsigned long long)v >> 32));
-    return (long long)(((unsigned long long)hi << 32) | lo);
-}
+__device__ __forceinline__ unsigned uniform(unsigned v) { return (unsigned)__builtin_amdgcn_readfirstlane((int)v); }
 
 // Thread index as a value the compiler takes as new each time it is asked for: everything a unit
 // derives from it (addresses, masks, lane roles) is then recomputed per unit instead of being
@@ -162,37 +170,57 @@ __device__ __forceinline__ int lane_id_per_unit()
     return tid;
 }
 
-__device__ __forceinline__ long long wave_sum_i64(long long v)
+// Item numbers are 32-bit: the host takes the balanced schedule only for steps whose item count, times the
+// workgroups that share it, stays below 2^31 (kBalancedMaxItemsTimesWorkgroups), so every product below fits.
+// The walk sits on every workgroup's path before its first load (and again at each change of unit), which is why it
+// is written for latency: one load of the lengths, sums across the wave on the DPP row operations (no trips
+// through the LDS crossbar), 32-bit divisions.
+constexpr unsigned kBalancedMaxItemsTimesWorkgroups = 0x7FFFFFFFu;
+
+// inclusive prefix sum over the wave's 64 lanes; lane 63 ends up with the total
+__device__ __forceinline__ unsigned wave_inclusive_scan(unsigned v)
 {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118, kRowBcast15 = 0x142, kRowBcast31 = 0x143;
+    int x = (int)v;
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr1, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr2, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr4, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowShr8, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, kRowBcast15, 0xA, 0xF, false);     // rows 1 and 3 take the total of the row before
+    x += __builtin_amdgcn_update_dpp(0, x, kRowBcast31, 0xC, 0xF, false);     // rows 2 and 3 take the total of the first half
+    return (unsigned)x;
 }
+__device__ __forceinline__ unsigned lane_value(unsigned v, int lane) { return (unsigned)__builtin_amdgcn_readlane((int)v, lane); }
 
 // items of all sequences, and of the sequences before `before` (every lane gets both)
-__device__ __forceinline__ void count_items(const AttnArgs& a, int before, long long& total, long long& prefix)
+__device__ __forceinline__ void count_items(const AttnArgs& a, int before, unsigned& total, unsigned& prefix)
 {
     if (!a.t_dev) {
-        const int it = seq_items(a, a.t_host);
-        total = (long long)a.B * it;
-        prefix = (long long)before * it;
+        const unsigned it = (unsigned)seq_items(a, a.t_host);
+        total = (unsigned)a.B * it;
+        prefix = (unsigned)before * it;
         return;
     }
     const int lane = threadIdx.x & (kWave - 1);
-    long long tot = 0, pre = 0;
-    for (int bb = lane; bb < a.B; bb += kWave) {
-        const int it = seq_items(a, a.t_dev[bb]);
-        tot += it;
-        if (bb < before) pre += it;
+    unsigned tot = 0, pre = 0;
+    for (int c = 0; c < a.B; c += kWave) {
+        const int bb = c + lane;
+        const unsigned it = bb < a.B ? (unsigned)seq_items(a, a.t_dev[bb]) : 0u;
+        const unsigned inc = wave_inclusive_scan(it);
+        tot += lane_value(inc, kWave - 1);
+        // sequences of this block before `before`: the inclusive sum of lane before - c - 1
+        const int last = before - c - 1;
+        if (last >= kWave - 1) pre += lane_value(inc, kWave - 1);
+        else if (last >= 0) pre += lane_value(inc, uniform(last));
     }
-    total = uniform(wave_sum_i64(tot));
-    prefix = uniform(wave_sum_i64(pre));
+    total = tot;
+    prefix = pre;
 }
 
 // workgroup that owns item x when W items are dealt to N workgroups as [i*W/N, (i+1)*W/N)
-__device__ __forceinline__ int item_owner(long long x, long long W, int N)
+__device__ __forceinline__ int item_owner(unsigned x, unsigned W, int N)
 {
-    return (int)(((x + 1) * N - 1) / W);
+    return (int)(((x + 1u) * (unsigned)N - 1u) / W);
 }
 
 // Workgroups that take part: never more than there are items, so that no share is empty and the
@@ -201,19 +229,19 @@ __device__ __forceinline__ int item_owner(long long x, long long W, int N)
 // not between one and two workgroups per compute unit (some units would get two shares, the rest one:
 // better one larger share each).  The launch has one workgroup per compute unit or two (or what a sweep
 // asked for, taken as it is).
-__device__ __forceinline__ int balanced_workgroups(const AttnArgs& a, long long W)
+__device__ __forceinline__ int balanced_workgroups(const AttnArgs& a, unsigned W)
 {
-    long long n = (W + 3) / 4;
-    if (n > a.bal_nwg) n = a.bal_nwg;
+    unsigned n = (W + 3u) / 4u;
+    if (n > (unsigned)a.bal_nwg) n = (unsigned)a.bal_nwg;
     if (a.bal_nwg == kBalancedWorkgroups && n > kBalancedWorkgroups / 2 && n < kBalancedWorkgroups) n = kBalancedWorkgroups / 2;
     return (int)n;
 }
 
 struct Walk {
-    long long W;           // items of the whole step
+    unsigned W;            // items of the whole step
     int N;                 // workgroups that share them
-    long long cur, hi;     // next item of this workgroup, end of its share
-    long long base;        // first item of sequence b
+    unsigned cur, hi;      // next item of this workgroup, end of its share
+    unsigned base;         // first item of sequence b
     int b, items;          // current sequence and its items per unit
     int nunits;            // units per sequence
 };
@@ -222,43 +250,56 @@ struct Walk {
 __device__ __forceinline__ bool walk_begin(const AttnArgs& a, int nunits, Walk& w)
 {
     const int lane = threadIdx.x & (kWave - 1);
-    long long total, unused;
-    count_items(a, 0, total, unused);
-    const long long W = total * nunits;
-    const int N = balanced_workgroups(a, W);
-    if ((int)blockIdx.x >= N) return false;
     w.nunits = nunits;
-    w.W = W;
-    w.N = N;
-    w.cur = uniform((long long)blockIdx.x * W / N);
-    w.hi = uniform((long long)(blockIdx.x + 1) * W / N);         // > cur, because N <= W
-    const long long target = w.cur / nunits;       // the sequence that holds item `cur` holds per-unit item `target`
     if (!a.t_dev) {
         w.items = seq_items(a, a.t_host);
-        w.b = uniform((int)(target / w.items));
-        w.base = (long long)w.b * w.items * nunits;
+        const unsigned W = (unsigned)a.B * (unsigned)w.items * (unsigned)nunits;
+        const int N = balanced_workgroups(a, W);
+        if ((int)blockIdx.x >= N) return false;
+        w.W = W;
+        w.N = N;
+        w.cur = uniform(blockIdx.x * W / (unsigned)N);
+        w.hi = uniform((blockIdx.x + 1u) * W / (unsigned)N);       // > cur, because N <= W
+        w.b = uniform((int)(w.cur / ((unsigned)w.items * (unsigned)nunits)));
+        w.base = (unsigned)w.b * (unsigned)w.items * (unsigned)nunits;
         return true;
     }
-    long long run = 0;
-    for (int c = 0; c < a.B; c += kWave) {
+    // up to 64 sequences (the usual case): their lengths are loaded once and stay in the lanes
+    const int first_bb = lane;
+    const unsigned it0 = first_bb < a.B ? (unsigned)seq_items(a, a.t_dev[first_bb]) : 0u;
+    const unsigned inc0 = wave_inclusive_scan(it0);
+    unsigned total = lane_value(inc0, kWave - 1);
+    for (int c = kWave; c < a.B; c += kWave) {
         const int bb = c + lane;
-        const int it = bb < a.B ? seq_items(a, a.t_dev[bb]) : 0;
-        long long inc = it;
-#pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
-            const long long v = __shfl_up(inc, off, kWave);
-            if (lane >= off) inc += v;
+        const unsigned it = bb < a.B ? (unsigned)seq_items(a, a.t_dev[bb]) : 0u;
+        total += lane_value(wave_inclusive_scan(it), kWave - 1);
+    }
+    const unsigned W = total * (unsigned)nunits;
+    const int N = balanced_workgroups(a, W);
+    if ((int)blockIdx.x >= N) return false;
+    w.W = W;
+    w.N = N;
+    w.cur = uniform(blockIdx.x * W / (unsigned)N);
+    w.hi = uniform((blockIdx.x + 1u) * W / (unsigned)N);           // > cur, because N <= W
+    const unsigned target = w.cur / (unsigned)nunits;   // the sequence that holds item `cur` holds per-unit item `target`
+    unsigned run = 0;
+    for (int c = 0; c < a.B; c += kWave) {
+        unsigned it = it0, inc = inc0;
+        if (c > 0) {
+            const int bb = c + lane;
+            it = bb < a.B ? (unsigned)seq_items(a, a.t_dev[bb]) : 0u;
+            inc = wave_inclusive_scan(it);
         }
-        const long long tot = __shfl(inc, kWave - 1, kWave);
+        const unsigned tot = lane_value(inc, kWave - 1);
         if (run + tot > target) {
             const unsigned long long hit = __builtin_amdgcn_ballot_w64(run + inc > target);
             const int f = __builtin_ctzll(hit);
             w.b = c + f;
-            w.items = uniform(__shfl(it, f, kWave));
-            w.base = (run + uniform(__shfl(inc, f, kWave)) - w.items) * nunits;
+            w.items = (int)lane_value(it, f);
+            w.base = (run + lane_value(inc, f) - (unsigned)w.items) * (unsigned)nunits;
             return true;
         }
-        run += uniform(tot);
+        run += tot;
     }
     return false;                                   // not reached: target < total
 }
@@ -269,12 +310,12 @@ template <int GT>
 __device__ __forceinline__ bool walk_unit(const AttnArgs& a, const Walk& w, Unit& u, int& nitems)
 {
     const int ngt = (a.G + GT - 1) / GT;
-    const long long rel = w.cur - w.base;
-    const int uib = uniform((int)(rel / w.items));
-    const int item = uniform((int)(rel - (long long)uib * w.items));
-    const long long left = w.hi - w.cur;
+    const unsigned rel = w.cur - w.base;
+    const int uib = uniform((int)(rel / (unsigned)w.items));
+    const int item = uniform((int)(rel - (unsigned)uib * (unsigned)w.items));
+    const unsigned left = w.hi - w.cur;
     nitems = w.items - item;
-    if (left < nitems) nitems = (int)left;
+    if (left < (unsigned)nitems) nitems = (int)left;
     nitems = uniform(nitems);
     u.b = w.b;
     u.kvh = uib / ngt;
@@ -297,8 +338,8 @@ __device__ __forceinline__ bool walk_unit(const AttnArgs& a, const Walk& w, Unit
     u.npieces = 1;
     u.counter = (int)unit_index;
     if (!u.direct && a.counters) {
-        const long long first = w.base + (long long)uib * w.items;
-        const int i0 = uniform(item_owner(first + c0, w.W, w.N)), i1 = uniform(item_owner(first + w.items - 1, w.W, w.N));
+        const unsigned first = w.base + (unsigned)uib * (unsigned)w.items;
+        const int i0 = uniform(item_owner(first + (unsigned)c0, w.W, w.N)), i1 = uniform(item_owner(first + (unsigned)w.items - 1u, w.W, w.N));
         u.p0 = ((size_t)i0 + unit_index) * GT;
         u.npieces = i1 - i0 + 1;
     }
@@ -308,9 +349,9 @@ __device__ __forceinline__ bool walk_unit(const AttnArgs& a, const Walk& w, Unit
 // Moves past nitems items; steps to the next sequence that has work when the current one is done.
 __device__ __forceinline__ void walk_advance(const AttnArgs& a, Walk& w, int nitems)
 {
-    w.cur += nitems;
+    w.cur += (unsigned)nitems;
     if (w.cur >= w.hi) return;
-    if (w.cur == w.base + (long long)w.items * w.nunits) {
+    if (w.cur == w.base + (unsigned)w.items * (unsigned)w.nunits) {
         w.base = w.cur;
         do {
             if (++w.b >= a.B) {                      // lengths changed under the kernel (out of contract): stop

@@ -105,17 +105,17 @@ void decode_attn_merge_balanced_kernel(const AttnArgs a, int D)
     const int t = a.t_dev ? a.t_dev[b] : a.t_host;
     const int items = seq_items(a, t);
     if (items == 0) return;
-    long long total, before;
+    unsigned total, before;
     count_items(a, b, total, before);
     const int ngt = (a.G + a.gt - 1) / a.gt;
     const int nunits = a.Hkv * ngt;
     const int gi = h % a.G;
     const int uib = (h / a.G) * ngt + gi / a.gt;
     const int g = gi % a.gt;
-    const long long W = total * nunits;
-    const long long first = before * nunits + (long long)uib * items;
+    const unsigned W = total * (unsigned)nunits;
+    const unsigned first = before * (unsigned)nunits + (unsigned)uib * (unsigned)items;
     const int N = balanced_workgroups(a, W);
-    const int i0 = item_owner(first + a.unit_cost, W, N), i1 = item_owner(first + items - 1, W, N);   // (the items that hold rows)
+    const int i0 = item_owner(first + (unsigned)a.unit_cost, W, N), i1 = item_owner(first + (unsigned)items - 1u, W, N);   // (the items that hold rows)
     if (i0 == i1) return;
     const int n = i1 - i0 + 1;
     // entry of workgroup i0 + s: (i0 + s + global unit) * gt + g
@@ -527,8 +527,11 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // 160, 192, ... in fp16) - in 16-byte aligned caches take the tiled kernels; any other head size or alignment
     // takes the scalar kernel
     const bool padded = row_bytes % 16 == 0 && padded_pieces(row_bytes / 16);
+    // (... and qkv / bias aligned to a pair of elements: the set-up reads them a pair at a time)
+    const uintptr_t pair_mask = (uintptr_t)(2 * esz - 1);
+    const bool pairs_aligned = !(reinterpret_cast<uintptr_t>(qkv) & pair_mask) && !(reinterpret_cast<uintptr_t>(qkv_bias) & pair_mask);
     const bool tiled = row_bytes >= 16 && row_bytes <= 1024 && (!(row_bytes & (row_bytes - 1)) || padded)
-                       && aligned16(k_cache) && aligned16(v_cache);
+                       && aligned16(k_cache) && aligned16(v_cache) && pairs_aligned;
     const int lpr = row_bytes / 16;
 
     AttnArgs a{};
@@ -613,7 +616,12 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // rounds ends with part of the chip idle: 576 units 227 -> 190 us, 640 units 265 -> 212, 768 units 284 -> 249)
     const bool uneven_grid = !t_dev && wmax >= 2048 && grid_wgs > 256
                              && (mfma_kernel ? (grid_wgs % 512 != 0 && grid_wgs < 4096) : grid_wgs < 384);
-    if (forced <= 0 && !padded && (bal == 1 || (bal != 0 && (uneven_grid || balanced_by_default(t_dev != nullptr, mfma_kernel, G, wmax))))) {
+    // (the walk counts items in 32 bits: a step of more items than that allows - hundreds of millions of rows -
+    // stays on the grid schedule)
+    const int cost_bound = tune_get("attn_balanced_cost") > 6 ? tune_get("attn_balanced_cost") : 6;
+    const bool walk_fits = (wmax + (long long)B * nunits * cost_bound) * (kBalancedWorkgroups * 2) < (long long)kBalancedMaxItemsTimesWorkgroups;
+    if (forced <= 0 && !padded && walk_fits
+        && (bal == 1 || (bal != 0 && (uneven_grid || balanced_by_default(t_dev != nullptr, mfma_kernel, G, wmax))))) {
         a.item_rows = item_rows;
         // (what a change of unit costs a workgroup, in items: measured on the matrix-core kernel, where workgroups whose
         // equal-row shares held one / two / three units finished at 82 / 90 / 94 us of a 101 us step)
