@@ -53,9 +53,24 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
             vv[u_] = load16_stream(vp + (size_t)row * D);
         }
     };
+    // the same for the chunk's last, partial iteration: rows past the end are read from the last valid row (and
+    // masked when they are consumed)
+    auto issue_any = [&](Vec16<T> (&kv)[U], Vec16<T> (&vv)[U], int rbase) {
+        if (rbase + RPI <= r1) {
+            issue(kv, vv, rbase);
+        } else {
+#pragma unroll
+            for (int u_ = 0; u_ < U; ++u_) {
+                const int row = min(rbase + u_ * NRG + rg, r1 - 1);
+                kv[u_] = load16_stream(kp + (size_t)row * D);
+                vv[u_] = load16_stream(vp + (size_t)row * D);
+            }
+        }
+    };
     const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
+    const int nb = r1 > r0 ? (r1 - r0 + RPI - 1) / RPI : 0;     // iterations, the partial one included
     Vec16<T> ka[U], va[U], kb[U], vb[U];
-    if (nfull > 0) issue(ka, va, r0);
+    if (nb > 0) issue_any(ka, va, r0);
 
     stage_q_and_new_row<T, D, GT, NTHR>(a, fr, u, kc, vc, sq, sk, sv, snew);
 
@@ -120,34 +135,39 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
 
     int look = -1;                              // (fused finish: the other pieces' arrivals, asked near the end)
     if (nfull == 0) look = first_look(a, u);
-    if (r1 > r0) {
-        // Full iterations are software-pipelined over two register buffers: the loads of the next
-        // iteration are in flight while the current one is consumed, so a wave never sits with an
-        // empty memory queue.  The (at most one) partial iteration at the end is masked.
+    if (nb > 0) {
+        // Iterations are software-pipelined over two register buffers - iteration k in buffer k % 2, the loads of
+        // the next one in flight while the current one is consumed - the chunk's last, partial iteration included
+        // (asked for after the last full one was consumed, it was a memory round trip with nothing else in flight
+        // at the end of every chunk: Llama-7B shape at 512 rows 24.9 -> us).  While two more full iterations lie
+        // ahead the loop holds nothing conditional, so the compiler waits for exactly the loads a product needs.
         const bool none[U] = {};
-        int rbase = r0;
-        for (int it = 0; it < nfull; it += 2) {
-            if (it + 2 >= nfull) look = first_look(a, u);
-            if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
+        if (nb > 1) issue_any(kb, vb, r0 + RPI);
+        int k = 0;
+        for (; k + 4 <= nfull; k += 2) {
+            const int rbase = r0 + k * RPI;
             consume(ka, va, none, std::false_type{});
-            if (it + 1 < nfull) {
-                if (it + 2 < nfull) issue(ka, va, rbase + 2 * RPI);
-                consume(kb, vb, none, std::false_type{});
-            }
-            rbase += 2 * RPI;
+            issue(ka, va, rbase + 2 * RPI);
+            consume(kb, vb, none, std::false_type{});
+            issue(kb, vb, rbase + 3 * RPI);
         }
-        rbase = r0 + nfull * RPI;
-        if (rbase < r1) {
+        for (; k < nfull; k += 2) {
+            if (k + 2 >= nfull) look = first_look(a, u);
+            const int rbase = r0 + k * RPI;
+            consume(ka, va, none, std::false_type{});
+            if (k + 2 < nb) issue_any(ka, va, rbase + 2 * RPI);
+            if (k + 1 < nfull) {
+                consume(kb, vb, none, std::false_type{});
+                if (k + 3 < nb) issue_any(kb, vb, rbase + 3 * RPI);
+            }
+        }
+        if (nb > nfull) {
+            const int rbase = r0 + nfull * RPI;
             bool valid[U];
 #pragma unroll
-            for (int u_ = 0; u_ < U; ++u_) {
-                int row = rbase + u_ * NRG + rg;
-                valid[u_] = row < r1;
-                row = min(row, r1 - 1);
-                ka[u_] = load16_stream(kp + (size_t)row * D);
-                va[u_] = load16_stream(vp + (size_t)row * D);
-            }
-            consume(ka, va, valid, std::true_type{});
+            for (int u_ = 0; u_ < U; ++u_) valid[u_] = rbase + u_ * NRG + rg < r1;
+            if (nfull & 1) consume(kb, vb, valid, std::true_type{});
+            else consume(ka, va, valid, std::true_type{});
         }
     }
 
@@ -167,8 +187,10 @@ __device__ __forceinline__ void split_unit(const AttnArgs& a, const RopeFreqs& f
     finish_unit<T, D, GT, NRG, NTHR>(a, u, st_ml, st_acc, snew, sv, look);
 }
 
+// (the single-head fp16 kernel at D = 128 - the Llama-7B shape - is held to the registers of four waves per SIMD: it
+// sits within two or three registers of that bound, and the fourth resident workgroup per compute unit is worth more)
 template <typename T, int LPR, int GT, int U, int NW, bool BALANCED>
-__global__ __launch_bounds__(NW * kWave)
+__global__ __launch_bounds__(NW * kWave, (GT == 1 && LPR == 16 && sizeof(T) == 2) ? 4 : 1)
 void decode_attn_split_kernel(const AttnArgs a, const RopeFreqs fr)
 {
     extern __shared__ float lds[];

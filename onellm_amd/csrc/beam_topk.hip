@@ -339,8 +339,8 @@ struct WaveTop {
     }
 };
 
-// workgroup of 256 lanes, `t` the finished list of each wave -> the lanes of wave 0 return the workgroup's KP best
-template <int KP>
+// workgroup of NWV waves, `t` the finished list of each wave -> the lanes of wave 0 return the workgroup's KP best
+template <int KP, int NWV>
 __device__ __forceinline__ void block_merge(TopList<KP>& t, Key* skey)
 {
     const int tid = threadIdx.x, wave = tid / kWave;
@@ -350,7 +350,7 @@ __device__ __forceinline__ void block_merge(TopList<KP>& t, Key* skey)
     }
     __syncthreads();
     if (wave == 0) {
-        for (int w = 1; w < 4; ++w) {
+        for (int w = 1; w < NWV; ++w) {
             TopList<KP> o;
 #pragma unroll
             for (int i = 0; i < KP; ++i) o.k[i] = skey[w * KP + i];
@@ -420,13 +420,17 @@ __device__ __forceinline__ void merge_survivors(const float* __restrict__ logits
 // workgroup's survivors, then adds to the counter with release order at device scope; the add of the last
 // arriver has acquire order and the barrier after it extends that to the workgroup, whose loads of the
 // survivors are device-scope loads (they do not take a line an earlier launch left in this compute unit's cache).
-template <int KP, bool FUSED>
-__global__ __launch_bounds__(256)
+//
+// NWV waves per workgroup: four take a row slice's chunks in turns of four, eight in turns of eight (every SIMD then
+// has a second chain of dependent instructions to run while the first waits, and each chain has half the values to
+// look at; it pays for long rows only, see launch_topk).
+template <int KP, bool FUSED, int NWV>
+__global__ __launch_bounds__(NWV * kWave)
 void topk_stage1_kernel(const float* __restrict__ logits, int V, int nblk, int vec_ok, int K,
                         float* __restrict__ vals, int* __restrict__ ids, int set, int beam,
                         float* __restrict__ fvals, int* __restrict__ fids)
 {
-    __shared__ Key skey[4 * KP];
+    __shared__ Key skey[NWV * KP];
     __shared__ int s_last;
     const int row = blockIdx.x / nblk, lane_blk = blockIdx.x % nblk;
     const float* p = logits + (size_t)row * V;
@@ -434,15 +438,15 @@ void topk_stage1_kernel(const float* __restrict__ logits, int V, int nblk, int v
     WaveTop<KP> w;
     w.clear();
     if (vec_ok) {
-        constexpr int PASSES = 4;
+        constexpr int PASSES = NWV == 4 ? 4 : 2;                  // (a 32000-token row is one batch per wave either way)
         const int nchunks = (V + 255) / 256;
         const int sub = threadIdx.x / 64, l4 = (threadIdx.x % 64) * 4;
-        for (int c0 = lane_blk + nblk * sub; c0 < nchunks; c0 += nblk * 4 * PASSES) {
+        for (int c0 = lane_blk + nblk * sub; c0 < nchunks; c0 += nblk * NWV * PASSES) {
             f32x4 v[PASSES];
             int tok[PASSES];
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) {
-                tok[q] = (c0 + nblk * 4 * q) * 256 + l4;
+                tok[q] = (c0 + nblk * NWV * q) * 256 + l4;
                 v[q] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
                 if (tok[q] < V) v[q] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + tok[q]));
             }
@@ -469,16 +473,19 @@ void topk_stage1_kernel(const float* __restrict__ logits, int V, int nblk, int v
                 }
             }
             w.raise_floor(lane_max);
-            w.template take<4 * PASSES, 4>(x, valid, flat0 + tok[0], nblk * 4 * 256);
+            w.template take<4 * PASSES, 4>(x, valid, flat0 + tok[0], nblk * NWV * 256);
         }
     } else {
+        // (a thread looks at token `threadIdx.x % 256` of the 256-token chunks lane_blk + nblk * (threadIdx.x / 256 + j * NWV / 4))
         constexpr int PASSES = 8;
-        for (int tok0 = threadIdx.x + lane_blk * 256; tok0 - (int)threadIdx.x < V; tok0 += nblk * 256 * PASSES) {
+        constexpr int STEP = NWV / 4;                               // chunks of the slice the workgroup covers at a time
+        const int first = (int)(threadIdx.x % 256) + (lane_blk + nblk * (int)(threadIdx.x / 256)) * 256;
+        for (int tok0 = first; tok0 - (int)(threadIdx.x % 256) < V; tok0 += nblk * 256 * STEP * PASSES) {
             float x[PASSES];
             unsigned valid = 0;
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) {
-                const int tok = tok0 + q * nblk * 256;
+                const int tok = tok0 + q * nblk * 256 * STEP;
                 x[q] = -INFINITY;
                 if (tok < V) {
                     x[q] = p[tok];
@@ -488,19 +495,19 @@ void topk_stage1_kernel(const float* __restrict__ logits, int V, int nblk, int v
             if (w.per_lane_road()) {
 #pragma unroll
                 for (int q = 0; q < PASSES; ++q)
-                    if ((valid >> q) & 1) w.lanes.insert(make_key(x[q], flat0 + tok0 + q * nblk * 256));
+                    if ((valid >> q) & 1) w.lanes.insert(make_key(x[q], flat0 + tok0 + q * nblk * 256 * STEP));
                 continue;
             }
             float lane_max = -INFINITY;
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) lane_max = fmaxf(lane_max, x[q]);
             w.raise_floor(lane_max);
-            w.template take<PASSES, 1>(x, valid, flat0 + tok0, nblk * 256);
+            w.template take<PASSES, 1>(x, valid, flat0 + tok0, nblk * 256 * STEP);
         }
     }
     w.finish();
     TopList<KP>& t = w.top;
-    block_merge<KP>(t, skey);
+    block_merge<KP, NWV>(t, skey);
     if (threadIdx.x == 0) {
 #pragma unroll
         for (int i = 0; i < KP; ++i) {
@@ -565,6 +572,13 @@ int launch_topk(const float* logits, int B, int beam, int V, int K, int nblk, fl
         }
         two = cs != hipStreamCaptureStatusNone;
     }
+    // Eight waves per workgroup for long rows (four chunks or more per wave) while the launch leaves room for them (up
+    // to two workgroups per compute unit): measured on MI355X, graph replay, batch 8 x beam 4, K = 4: V = 128256
+    // 14.1 -> 13.5 us; V = 32000 7.6 -> 8.2 us (a wave's fixed work - floor, marks, ranking - does not shrink with its
+    // share of the row, and the workgroup merges eight lists instead of four), so short rows keep four.  Tuning key
+    // topk_waves = 4 / 8 forces either.
+    const int want_waves = tune_get("topk_waves");
+    const bool eight = want_waves == 8 || (want_waves != 4 && (long)B * beam * nblk <= 512 && V >= nblk * 8 * 256 * 4);
     int set = -1;
     g_last_path = ONELLM_TOPK_PATH_TWO_LAUNCHES;
     if (B <= kArrivalEntries && !two) {
@@ -576,13 +590,17 @@ int launch_topk(const float* logits, int B, int beam, int V, int K, int nblk, fl
     }
     if (set >= 0) {
         g_last_path = ONELLM_TOPK_PATH_ONE_LAUNCH;
-        hipLaunchKernelGGL((topk_stage1_kernel<KP, true>), dim3(B * beam * nblk), dim3(256), 0, st, logits, V, nblk, vec_ok, K,
-                           vals, ids, set, beam, fvals, fids);
+        if (eight) hipLaunchKernelGGL((topk_stage1_kernel<KP, true, 8>), dim3(B * beam * nblk), dim3(512), 0, st, logits, V, nblk, vec_ok, K,
+                                      vals, ids, set, beam, fvals, fids);
+        else hipLaunchKernelGGL((topk_stage1_kernel<KP, true, 4>), dim3(B * beam * nblk), dim3(256), 0, st, logits, V, nblk, vec_ok, K,
+                                vals, ids, set, beam, fvals, fids);
         g_last_launches = 1;
         return launch_status();
     }
-    hipLaunchKernelGGL((topk_stage1_kernel<KP, false>), dim3(B * beam * nblk), dim3(256), 0, st, logits, V, nblk, vec_ok, K,
-                       vals, ids, -1, beam, fvals, fids);
+    if (eight) hipLaunchKernelGGL((topk_stage1_kernel<KP, false, 8>), dim3(B * beam * nblk), dim3(512), 0, st, logits, V, nblk, vec_ok, K,
+                                  vals, ids, -1, beam, fvals, fids);
+    else hipLaunchKernelGGL((topk_stage1_kernel<KP, false, 4>), dim3(B * beam * nblk), dim3(256), 0, st, logits, V, nblk, vec_ok, K,
+                            vals, ids, -1, beam, fvals, fids);
     int rc = launch_status();
     if (rc) return rc;
     hipLaunchKernelGGL((topk_stage2_kernel<KP>), dim3(B), dim3(kWave), 0, st, logits, vals, ids, beam * nblk * K, K, fvals, fids);

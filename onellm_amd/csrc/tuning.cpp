@@ -29,6 +29,7 @@ Knob g_knobs[] = {
     {"attn_early_look", {-1}},   // 1 / 0: a piece that finds the unit's other pieces arrived merges it from its registers / never looks
     {"topk_two_launches", {-1}}, // beam top-K: 1 = always a second launch for the merge of the survivors, 0 = one launch wherever it can be (also under capture)
     {"gemm_ordered_finish", {-1}}, // 1: release on the few-row projection kernel's counter add + acquire fence in the slice that reads the sums back
+    {"topk_waves", {-1}},        // beam top-K: 4 / 8 waves per stage-1 workgroup instead of the launcher's choice
     {"attn_turns", {-1}},        // 0: co-resident attention workgroups do not take turns at wave priority
 };
 }  // namespace

@@ -101,12 +101,16 @@ def test_repeat_matches_oracle(capi, ref, dev, dtype, Hq, Hkv, D):
 
 # ---------------------------------------------------------------- beam top-K
 
-@pytest.fixture(params=["one_launch", "two_launches"])
+@pytest.fixture(params=["one_launch-4waves", "two_launches-4waves", "one_launch-8waves", "two_launches-8waves"])
 def topk_form(request, capi):
-    """Both forms of the second stage: merged by the last stage-1 workgroup of a batch entry, or by a second launch."""
-    capi.tune_set("topk_two_launches", 1 if request.param == "two_launches" else 0)
+    """Both forms of the second stage - merged by the last stage-1 workgroup of a batch entry, or by a second launch -
+    with four and with eight waves per stage-1 workgroup (the launcher picks by shape; here both run on every shape)."""
+    form, waves = request.param.split("-")
+    capi.tune_set("topk_two_launches", 1 if form == "two_launches" else 0)
+    capi.tune_set("topk_waves", 8 if waves == "8waves" else 4)
     yield request.param
     capi.tune_set("topk_two_launches", -1)
+    capi.tune_set("topk_waves", -1)
 
 
 def _lexsort_topk(flat_vals, flat_ids, K):
