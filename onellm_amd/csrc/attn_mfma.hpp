@@ -526,9 +526,8 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
     extern __shared__ float lds[];
     stamp_entry(a);
     int ev = 0;
-    if constexpr (DOUBLE_BUFFER && !BALANCED) {
-        Unit u;
-        if (locate_unit<GT>(a, u)) gqa_mfma_grid_unit<D, GT, NW>(a, fr, u, lds, ev);
+    if constexpr (DOUBLE_BUFFER) {
+        for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_grid_unit<D, GT, NW>(a, fr, u, lds, ev); });
     } else {
         for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_unit<D, GT, NW, DOUBLE_BUFFER>(a, fr, u, lds, ev); });
     }
