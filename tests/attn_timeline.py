@@ -1,12 +1,16 @@
 """Per-workgroup timeline of a decode-attention launch: when each workgroup ended and on which XCD it ran.
 
     python -m onellm_amd.build --stamps          # builds tests/cpp/libonellm_hip_stamps.so (once)
-    python tests/attn_timeline.py [config2|config2_ctx512|config2_ctx16|config3|config3_full] [knob=value ...]
+    python tests/attn_timeline.py [config2|config2_ctx512|config2_ctx16|config3|config3_full] [phases] [knob=value ...]
 
 Runs the kernel library built with -DONELLM_ATTN_STAMPS (the product sources plus two clock stamps per workgroup and
 the XCC id register) on synthetic inputs of the named BASELINE shape and prints, per XCD and per dispatch half
 (workgroups i and i + 256 land on the same compute unit), the mean / min / max end time in microseconds after the
-first workgroup's entry, over eight launches on rotating cache sets.  A measurement aid, not a test."""
+first workgroup's entry, over eight launches on rotating cache sets.  With `phases` (matrix-core kernels: config3,
+config3_full) it also prints, for the workgroups grouped by the number of unit pieces in their share, when each piece
+was begun, how long its set-up, its streaming loop and its finish took, and how long a change of unit takes from the
+last row of one piece to the first score of the next.  A measurement aid for the tables under profiles/, not a test:
+pytest does not collect it."""
 import ctypes
 import os
 import sys
@@ -36,7 +40,8 @@ def main():
     L = capi.lib()
     L.onellm_attn_set_stamp_buffer.argtypes = [ctypes.c_void_p]
     L.onellm_attn_set_stamp_buffer.restype = None
-    for kv in sys.argv[2:]:                      # internal tuning knobs, e.g. attn_balanced_wgs=512
+    phases = "phases" in sys.argv[2:]
+    for kv in [x for x in sys.argv[2:] if x != "phases"]:      # internal tuning knobs, e.g. attn_balanced_wgs=512
         key, value = kv.split("=")
         capi.tune_set(key, int(value))
         print("knob", key, "=", value)
@@ -53,7 +58,8 @@ def main():
     if c["ragged"]:
         t_dev = torch.from_numpy(np.random.default_rng(3).integers(1024, S + 1, size=B).astype(np.int32)).to(dev)
     ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
-    stamps = torch.zeros(8192 * 4, dtype=torch.int64, device=dev)
+    EVENTS = 16                                                # phase stamps per workgroup, behind the four words of each
+    stamps = torch.zeros(8192 * (4 + EVENTS), dtype=torch.int64, device=dev)
 
     def step(i):
         kc, vc = sets[i % len(sets)]
@@ -70,7 +76,7 @@ def main():
     ev1.record()
     torch.cuda.synchronize()
     print("%s: %.1f us per step (HIP events, 50 steps, stamps off)" % (name, ev0.elapsed_time(ev1) / 50 * 1e3))
-    ends, xcc, cu, alone = [], None, None, []
+    ends, xcc, cu, alone, phase_runs = [], None, None, [], []
     for rep in range(8):
         stamps.zero_()
         torch.cuda.synchronize()
@@ -81,9 +87,14 @@ def main():
         torch.cuda.synchronize()
         alone.append(ev0.elapsed_time(ev1) * 1e3)
         L.onellm_attn_set_stamp_buffer(None)
-        d = stamps.cpu().numpy().reshape(-1, 4)
+        raw = stamps.cpu().numpy()
+        d = raw[:8192 * 4].reshape(-1, 4)
         used = d[:, 0] != 0
         n = int(used.sum())
+        if phases:
+            ev = raw[n * 4:n * 4 + n * EVENTS].reshape(n, EVENTS).astype(np.float64)
+            t0 = d[:n, 0].min()
+            phase_runs.append(((d[:n, 0] - t0) / 100.0, (d[:n, 1] - t0) / 100.0, np.where(ev > 0, (ev - t0) / 100.0, np.nan)))
         st, en = d[:n, 0], d[:n, 1]
         xcc = d[:n, 2] & 0xF
         cu = ((d[:n, 3] >> 8) & 0xFF) | (xcc << 8)      # (XCD, shader engine, array, unit)
@@ -103,6 +114,34 @@ def main():
             line += " | %d..%d end mean %.1f (min %.1f, max %.1f)" % (half, n - 1, b.mean(), b.min(), b.max())
         print(line)
     by_compute_unit(ends[-1], cu)
+    if phases:
+        phase_table(phase_runs)
+
+
+def phase_table(runs):
+    """Four stamps per unit piece (begun, set-up done, last row consumed, finished), averaged over the launches, for the
+    workgroups grouped by how many pieces their share holds."""
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        entry = np.mean([r[0] for r in runs], 0)
+        end = np.mean([r[1] for r in runs], 0)
+        ev = np.nanmean([r[2] for r in runs], 0)
+    npieces = (~np.isnan(ev)).sum(1) // 4
+    print("workgroups by number of pieces in their share:", {int(k): int(v) for k, v in zip(*np.unique(npieces, return_counts=True))})
+    for n in sorted(set(npieces)):
+        if n == 0:
+            continue
+        sel = npieces == n
+        e = ev[sel]
+        print("-- %d piece(s), %d workgroups: end mean %.1f us; entry -> first piece begun %.2f us"
+              % (n, sel.sum(), end[sel].mean(), np.nanmean(e[:, 0] - entry[sel])))
+        for p in range(n):
+            b, s, l, f = e[:, 4 * p], e[:, 4 * p + 1], e[:, 4 * p + 2], e[:, 4 * p + 3]
+            line = "   piece %d: begun at %5.1f; set-up %.2f; streaming %.2f; finish %.2f" % (p, np.nanmean(b), np.nanmean(s - b), np.nanmean(l - s), np.nanmean(f - l))
+            if p + 1 < n:
+                line += "; last row -> next piece's first score %.2f" % np.nanmean(e[:, 4 * (p + 1) + 1] - l)
+            print(line)
 
 
 
