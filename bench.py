@@ -21,13 +21,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0   # MI355X, published
+HEADLINE_SETTLE_S = 0.1  # the headline step runs untimed for this long before its --warmup launches (see settle())
 
 # HBM bytes per launch of the headline kernel as counted by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
-# each scaled by the same counter's reading for a 1 GiB device copy: x1.99994 and x1.0000), keyed by context, and
+# each scaled by the same counter's reading for a 1 GiB device copy: x1.99995 and x1.0000), keyed by context, and
 # the digest of the attention sources the counted kernel was built from: when the sources change the figure is
 # withheld (traffic: null) until the counter runs are repeated and both are updated together.
-MEASURED_TRAFFIC_BYTES = {4096: 1074438341}
-MEASURED_TRAFFIC_SOURCES = "449cb23c0c63426a"
+MEASURED_TRAFFIC_BYTES = {4096: 1074483396}
+MEASURED_TRAFFIC_SOURCES = "d27cca355c292130"
 ATTENTION_SOURCES = ["decode_attn.hip", "attn_schedule.hpp", "attn_finish.hpp", "attn_valu.hpp", "attn_mfma.hpp", "common.hpp", "rope.hpp"]
 
 
@@ -81,10 +82,17 @@ def time_steps_median(fn, steps, warmup, blocks=3):
     return times[len(times) // 2]
 
 
-def settle(fn, seconds=0.02):
-    """Keep the GPU busy with the step for ~20 ms before an extras line is timed.  Coming out of an idle phase the
-    clocks take 10-15 ms to settle (the same kernel measured 159 us for its first ten launches, 171-187 for the next
-    sixty, 158.6 from then on); the headline value is not treated this way - it follows --warmup / --steps."""
+def settle(fn, seconds=0.05):
+    """Keep the GPU busy with the step for a while before it is timed (untimed, not counted among the warm-up steps).
+    Coming out of an idle phase the clocks take 10-15 ms to settle (the same kernel measured 159 us for its first ten
+    launches, 171-187 for the next sixty, 158.6 from then on), and a timed region of a few milliseconds that starts
+    five launches after the data was generated lies wholly inside that ramp.
+
+    A second effect this does NOT cover, which is why nothing in this file gives memory back to the driver
+    (no torch.cuda.empty_cache()): for 50-250 ms after gigabytes of device memory were freed, every kernel here runs
+    3-4 % slower (the ragged grouped-query line 96.5 us instead of 93.0, the headline 164 instead of 157, blocks of 100
+    launches agreeing to 0.2 us within either state) and then drops back for good; idling, random-number kernels or
+    1 GiB copies in between do not bring that state on, freeing and re-allocating the caches does."""
     import time
     import torch
     t0, i = time.perf_counter(), 0
@@ -193,7 +201,10 @@ def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=
         capi.decode_attn(qkv, bias, kc, vc, out, Hq, max_t, D, 10000.0, t_dev=t_dev, max_t=max_t, workspace=ws,
                          flags=capi.ATTN_ZEROED_WORKSPACE)
 
-    # (the headline is timed as EXACTLY `steps` launches in one block; the other shapes take the median of three)
+    # (the headline is timed as EXACTLY `steps` launches in one block, after the clock ramp and `warmup` further
+    # launches; the other shapes take the median of three such blocks)
+    if not median:
+        settle(step, HEADLINE_SETTLE_S)
     ms = time_steps_median(step, steps, warmup) if median else time_steps(step, steps, warmup)
     bench_attention.last_step = step
     return ms, (qkv, bias, sets[0], out)
@@ -421,7 +432,6 @@ def projections_section(capi, dev, steps):
         e["weight_sets"] = n
         out["linear_m16_%s_%dx%d" % (name, K, N)] = e
         del wts
-        torch.cuda.empty_cache()
     return out
 
 
@@ -478,7 +488,6 @@ def ceilings_section(dev, steps, warmup):
         best("row_pairs_in_place_8192x%dB" % row_bytes, 4 * per + 2 * row_bytes,
              lambda pol: (lambda i: ac.rows(views[(2 * i) % n], views[(2 * i + 1) % n], shared, pol)))
     del big, half, fan_src, fan_dst, views, tm, hm
-    torch.cuda.empty_cache()
     return out
 
 
@@ -508,7 +517,6 @@ def extras_section(capi, dev, args, with_cpu):
         cpu = cpu_attention(qkv, bias, kc, vc, H, c, D, 3.0)[0] if with_cpu else None
         ex["decode_attn_ctx%d" % c] = entry(ms, attn_bytes(B, H, H, D, [c] * B, 2), cpu)
         del qkv, bias, kc, vc
-        torch.cuda.empty_cache()
 
     # BASELINE configs[2]: batch 32, 32 query heads over 8 KV heads, lengths U[1024, 8192], S = 8192
     B3, Hq3, Hkv3, S3 = 32, 32, 8, 8192
@@ -525,15 +533,12 @@ def extras_section(capi, dev, args, with_cpu):
     ex["decode_attn_gqa_fused_b32_q32_kv8_len8192"] = entry(ms_u, attn_bytes(B3, Hq3, Hkv3, D, [S3] * B3, 2))
     ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, 16, 64, Hkv3, D, S3, S3, nsets=3)
     ex["decode_attn_gqa_fused_b16_q64_kv8_len8192"] = entry(ms_u, attn_bytes(16, 64, Hkv3, D, [S3] * 16, 2))
-    torch.cuda.empty_cache()
     # the same 64-over-8 head shape with fp32 caches (the reference's own element type), batch 8 (the same bytes)
     ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, 8, 64, Hkv3, D, S3, S3, nsets=3, fp32=True)
     ex["decode_attn_gqa_fused_fp32_b8_q64_kv8_len8192"] = entry(ms_u, attn_bytes(8, 64, Hkv3, D, [S3] * 8, 4))
-    torch.cuda.empty_cache()
     # config 2's shape with fp32 caches at batch 8 (the same bytes as the headline): the reference's own element type
     ms_u, _ = bench_attention(capi, dev, steps3, args.warmup, 8, 32, 32, D, 4096, 4096, nsets=3, fp32=True)
     ex["decode_attn_fp32_b8_h32_ctx4096"] = entry(ms_u, attn_bytes(8, 32, 32, D, [4096] * 8, 4))
-    torch.cuda.empty_cache()
     # the reference-style path on the same data: concat the new row, repeat KV to 32 heads, attend over 32 heads
     hist = (t_dev - 1).contiguous()
     ones = torch.ones(B3, dtype=torch.int32, device=dev)
@@ -560,15 +565,12 @@ def extras_section(capi, dev, args, with_cpu):
     e["note"] = "concat -> repeat -> attend on the same data; gbps/frac are against the FUSED path's algorithmic bytes"
     ex["decode_attn_gqa_repeat_path_total"] = e
     del rk, rv, kc, vc, qkv, bias, qkv_r, ws
-    torch.cuda.empty_cache()
 
     ex.update(projections_section(capi, dev, args.steps))
     ex.update(decoder_layer_section(capi, dev, args))
-    torch.cuda.empty_cache()
     # the same layer width with grouped-query heads at BASELINE configs[2]'s batch and cache (32 sequences, 32 q / 8 kv
     # heads, 8192 rows each: the layers take one step count for the whole batch): 32 rows through the projections
     ex.update(decoder_layer_section(capi, dev, args, B=32, H=32, Hkv=8, S=8192, key="decoder_layer_gqa_b32_q32_kv8_ctx8192"))
-    torch.cuda.empty_cache()
 
     for (N, Hd) in ((16, 4096), (512, 4096), (8192, 4096), (8192, 8192)):
         for fused in (False, True):
@@ -579,7 +581,6 @@ def extras_section(capi, dev, args, with_cpu):
                 e = with_graph(e, bench_norms.last_step)
             ex["%s_%dx%d" % ("fused_norm" if fused else "rmsnorm", N, Hd)] = e
             bench_norms.last_step = None
-        torch.cuda.empty_cache()
 
     # the callers either side of the path: prefill QKV bias + RoPE + transpose (4 x 2048 tokens, 32 heads x 128)
     # and the SwiGLU gate (8192 x 11008)
@@ -599,7 +600,6 @@ def extras_section(capi, dev, args, with_cpu):
         cpu = time_cpu(lambda: ref.qkv_bias_rope_transpose(hq, hk, hv, h_in, h_b, h_po, h_hl, D, 10000.0), 4.0)[0]
     ex["prefill_qkv_bias_rope_4x2048_tokens_32x128"] = entry(ms, 2 * Bp * Sp * 3 * Hp * D * 2 + 3 * Hp * D * 2, cpu)
     del qkvs, qb, kb, vb
-    torch.cuda.empty_cache()
     ins = [torch.randn(8192, 2, 11008, device=dev).half() for _ in range(3)]
     oa = torch.empty(8192, 11008, dtype=torch.float16, device=dev)
     ms = time_steps_median(lambda i: capi.silu_and_mul(ins[i % 3], oa), steps3, 5)
@@ -610,7 +610,6 @@ def extras_section(capi, dev, args, with_cpu):
         cpu = time_cpu(lambda: ref.silu_and_mul(h_in, h_out), 3.0)[0]
     ex["swiglu_8192x11008"] = entry(ms, 3 * 8192 * 11008 * 2, cpu)
     del ins, oa
-    torch.cuda.empty_cache()
 
     logits = torch.randn(32, 32000, device=dev).mul_(2.0)
     wsk = torch.empty(capi.beam_topk_workspace_bytes(8, 4, 4) // 4, dtype=torch.float32, device=dev)
@@ -626,7 +625,6 @@ def extras_section(capi, dev, args, with_cpu):
     e["launches_graph_replay"] = capi.beam_topk_last_launches()   # under capture: a second launch merges
     ex["beam_topk_b8_beam4_v32000_k4"] = e
     del logits, wsk
-    torch.cuda.empty_cache()
 
     ceil = ceilings_section(dev, args.steps, args.warmup)
     ex["ceilings"] = ceil
@@ -670,7 +668,6 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-        torch.cuda.empty_cache()
 
     B, H, D, S, t = 16, 32, 128, 4096, args.ctx
     ms, (qkv, bias, (kc, vc), out) = bench_attention(capi, dev, args.steps, args.warmup, B, H, H, D, S, t, nsets=4, median=False)
@@ -682,7 +679,7 @@ def main():
         "metric": "decode-attn us/step at Llama-2-7B shape, ctx %d (fused masked MHA: qkv bias + RoPE + KV-cache write + softmax + V sum)" % t,
         "value": round(ms * 1e3, 2), "unit": "us/step", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic", "settle_s_before_warmup": HEADLINE_SETTLE_S,
         "config": {"workload": "BASELINE configs[1]: batch 16, 32 heads x 128, MHA, fp16 KV cache [1,16,32,4096,128], ctx %d, "
                                "RoPE base 10000; 4 cache sets rotated per step" % t,
                    "storage": "fp16", "arithmetic": "fp32"},
@@ -711,7 +708,6 @@ def main():
                                               "sample": "sequence 0 of the batch only (%.1f ms, median of %d runs), "
                                                         "multiplied by the batch size %d" % (one_us / 1e3, runs1, B)}
     del qkv, bias, kc, vc, out
-    torch.cuda.empty_cache()
     if not args.no_extras:
         # the other shapes are measurements of their own, not the contract's "step": at least 100 timed launches
         # after at least 10 untimed ones each, whatever --steps / --warmup asked of the headline

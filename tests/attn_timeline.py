@@ -89,8 +89,10 @@ def main():
         L.onellm_attn_set_stamp_buffer(None)
         raw = stamps.cpu().numpy()
         d = raw[:8192 * 4].reshape(-1, 4)
-        used = d[:, 0] != 0
-        n = int(used.sum())
+        # a workgroup's record is (entry, end, XCD id, hardware id); the phase stamps that follow the records are clock
+        # values in every word, so the records are the leading rows whose third word is an XCD id
+        used = (d[:, 0] != 0) & (d[:, 2] < 16) & (d[:, 3] < 2 ** 32)
+        n = int(np.argmin(used)) if not used.all() else len(used)
         if phases:
             ev = raw[n * 4:n * 4 + n * EVENTS].reshape(n, EVENTS).astype(np.float64)
             t0 = d[:n, 0].min()
