@@ -35,7 +35,8 @@ struct AttnArgs {
     int item_rows;
     int unit_cost;        // what starting on another unit costs a workgroup, in items (set-up, finish, an emptied load queue)
     int turns;            // co-resident workgroups take turns at wave priority (take_turns below); 0: they do not
-    int gt;               // query heads per tile, for the merge kernel
+    int gt;               // query heads per tile
+    int on_mfma;          // the step runs on the matrix-core kernels (host-side choice)
     // fused finish (counters != NULL): one arrival counter per unit, zero between calls; the piece
     // that arrives last merges the unit's partial states itself and no merge kernel is launched
     int* counters;

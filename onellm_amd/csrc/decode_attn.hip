@@ -355,22 +355,30 @@ int launch_shape(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 constexpr bool mfma_head_size(int D) { return D == 64 || D == 128 || D == 256; }
 
 // shapes that run on the matrix cores: fp16 caches with three or more query heads per kv head at those head
-// sizes (with two the vector ALU keeps up with the stream and is as fast or faster: 16 q / 8 kv heads, 8192 rows,
-// D = 128, batch 32: 152.8 against 154.4 us; D = 64: 78.9 against 86.8; D = 256, 4096 rows: 152.7 against 157.4 -
-// with four heads it is 13 % slower); fp32 caches at D = 64 or 128 with more than four
-bool on_matrix_cores(bool fp16, int D, int G)
+// sizes, fp32 caches at D = 64 or 128 with more than four.  With two heads per kv head the vector ALU keeps up with
+// the stream, and which kernel is faster depends on how long a unit streams between its set-up and its finish:
+// at D = 128 the matrix-core kernel wins from about 2048 rows (16 q / 8 kv heads, batch 32: 8192 rows 158.2 -> 152.3
+// us, lengths 1024..8192 94.9 -> 92.2, 2048 rows 44.2 -> 43.8; 64 q / 32 kv heads, batch 16, 4096 rows 159.0 ->
+// 157.8) and loses below (512 rows 15.1 -> 15.6, lengths 256..2048 at batch 96 76.4 -> 78.8), so it takes steps whose
+// longest sequence has 4096 rows or more; at D = 64 (82.4 against 86.7) and D = 256 (lengths 512..4096: 96.5 against
+// 98.9) the vector-ALU kernel stays.  One head per kv head: equal from 4096 rows (157.7 both at the Llama-2-7B shape),
+// the vector ALU ahead below (512 rows 23.7 against 24.6), so it keeps all of them.
+// Tuning key attn_gqa_valu: 1 = never the matrix cores, 0 = always where a matrix-core kernel exists.
+bool on_matrix_cores(bool fp16, int D, int G, int max_t)
 {
     if (tune_get("attn_gqa_valu") == 1) return false;
-    return fp16 ? (G > 2 && mfma_head_size(D)) : (G > 4 && (D == 128 || D == 64));
+    if (tune_get("attn_gqa_valu") == 0 && fp16 && mfma_head_size(D)) return true;
+    if (!fp16) return G > 4 && (D == 128 || D == 64);
+    return mfma_head_size(D) && (G > 2 || (G == 2 && D == 128 && max_t >= 4096));
 }
 
 // query heads one workgroup serves (they share every K/V row it reads)
-int heads_per_tile(bool fp16, int D, int G)
+int heads_per_tile(bool fp16, int D, int G, int max_t)
 {
-    if (G == 1) return 1;       // one head: memory-bound on either kernel (measured equal), keep the lighter one
+    if (G == 1 && !on_matrix_cores(fp16, D, G, max_t)) return 1;       // one head: memory-bound on either kernel (measured equal), keep the lighter one
     // three or more query heads per kv head, fp16: both products on the matrix cores, where up to 16
     // heads cost the same as 4 (8 at D = 256: the per-wave states of 16 heads would not fit 64 KiB of LDS)
-    if (on_matrix_cores(fp16, D, G)) {
+    if (on_matrix_cores(fp16, D, G, max_t)) {
         const int cap = D == 256 ? 8 : 16;
         const int gt = G <= 4 ? 4 : (G <= 8 ? 8 : 16);
         return gt < cap ? gt : cap;
@@ -386,12 +394,12 @@ int launch_gt(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 {
     constexpr bool kHalf = std::is_same<T, __half>::value;
     constexpr int D = LPR * Elt<T>::kVec;
-    const int gt = heads_per_tile(kHalf, D, a.G);
+    const int gt = a.gt;
     if constexpr (!kHalf && (D == 128 || D == 64)) {
-        if (on_matrix_cores(false, D, a.G)) return gt == 8 ? launch_gqa_mfma_f32<D, 8>(a, fr, st) : launch_gqa_mfma_f32<D, 16>(a, fr, st);
+        if (a.on_mfma) return gt == 8 ? launch_gqa_mfma_f32<D, 8>(a, fr, st) : launch_gqa_mfma_f32<D, 16>(a, fr, st);
     }
     if constexpr (kHalf && mfma_head_size(D)) {
-        if (on_matrix_cores(true, D, a.G)) {
+        if (a.on_mfma) {
             switch (gt) {
                 case 4: return launch_gqa_mfma<D, 4>(a, fr, st);
                 case 8: return launch_gqa_mfma<D, 8>(a, fr, st);
@@ -430,9 +438,9 @@ int launch_lpr(int lpr, const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 
 
 // rows per work item of the balanced schedule: one workgroup iteration of the kernel that runs
-int item_rows_for(bool fp16, int D, int G)
+int item_rows_for(bool fp16, int D, int G, int max_t)
 {
-    if (on_matrix_cores(fp16, D, G)) return 64;
+    if (on_matrix_cores(fp16, D, G, max_t)) return 64;
     const int lpr = D * (fp16 ? 2 : 4) / 16;
     const int rpi = 1024 / lpr;               // 4 waves x (64 / lpr) rows x 4 per row group
     return rpi < 64 ? 64 : rpi;
@@ -561,12 +569,13 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // needs no merge pass.  Per-sequence lengths: finer chunks (about 16 workgroups per compute unit,
     // at least 256 rows each) so that the dispatcher can balance ragged work.
     const int G = a.G;
-    const int gt = padded ? (G == 1 ? 1 : 4) : heads_per_tile(dtype == ONELLM_FP16, D, G);
+    const int gt = padded ? (G == 1 ? 1 : 4) : heads_per_tile(dtype == ONELLM_FP16, D, G, max_t);
     const int ngt = (G + gt - 1) / gt;
     const long base_wgs = (long)B * Hkv * ngt;
     const int user_target = tune_get("attn_target_wgs");
     // (the matrix-core kernel at D = 64 has half the bytes in flight per workgroup: two per compute unit)
-    const bool mfma64 = D == 64 && on_matrix_cores(dtype == ONELLM_FP16, D, G) && dtype == ONELLM_FP16;
+    const bool mfma_kernel = !padded && on_matrix_cores(dtype == ONELLM_FP16, D, G, max_t);
+    const bool mfma64 = D == 64 && mfma_kernel && dtype == ONELLM_FP16;
     const int target = user_target > 0 ? user_target : (t_dev ? 4096 : (mfma64 ? 512 : 256));
     int nsplit = (int)((target + base_wgs - 1) / base_wgs);
     int cap = max_splits(max_t);
@@ -588,6 +597,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     a.chunk = chunk;
     a.nsplit = nsplit;
     a.gt = gt;
+    a.on_mfma = mfma_kernel;
 
     // Balanced schedule: a fixed number of workgroups (what the chip holds at once) share the rows
     // of the step equally, whatever the lengths and however the units divide among compute units.
@@ -602,7 +612,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     float* const partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + counter_bytes);
     const int bal = tune_get("attn_balanced");
     // (the step's size in work items if every sequence had the longest length: all the host knows)
-    const int item_rows = item_rows_for(dtype == ONELLM_FP16, D, G);
+    const int item_rows = item_rows_for(dtype == ONELLM_FP16, D, G, max_t);
     const long long items = (max_t - 1 + item_rows - 1) / item_rows;
     const long long wmax = (long long)B * nunits * (items < 1 ? 1 : items);
     // Equal lengths whose grid does not fill the chip evenly - between one and two workgroups per compute unit (one
@@ -610,7 +620,6 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // run two workgroups and the rest one.  One equal share per compute unit instead (measured: 40 heads x batch 8 =
     // 320 units 116 -> 101 us; 8 kv heads x batch 10, cut in four = 320 workgroups 75 -> 59 us; 8 kv heads x batch 48
     // = 384 units 144 -> 130 us; 384 single-head units 121.5 -> 124.6, hence the lower bound there).
-    const bool mfma_kernel = on_matrix_cores(dtype == ONELLM_FP16, D, G);
     const long grid_wgs = base_wgs * nsplit;
     // (the matrix-core kernels hold two workgroups per unit at most, so any grid that is not a whole number of such
     // rounds ends with part of the chip idle: 576 units 227 -> 190 us, 640 units 265 -> 212, 768 units 284 -> 249)

@@ -513,6 +513,30 @@ def test_long_sequences_of_a_small_batch(capi, ref, dev, B, Hq, Hkv, D, t):
         assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0
 
 
+@pytest.mark.parametrize("max_t", [4095, 4096])
+@pytest.mark.parametrize("ragged", [False, True])
+def test_two_heads_per_kv_head_either_side_of_the_kernel_switch(capi, ref, dev, max_t, ragged):
+    """16 query heads over 8 kv heads at head size 128: steps whose longest sequence has 4096 rows or more run on the
+    matrix-core kernel, shorter ones on the vector-ALU kernel (onellm_amd/csrc/decode_attn.hip: on_matrix_cores).
+    Both sides of that switch, equal and per-sequence lengths, merge launch and fused finish, against the oracle."""
+    announce("attn two heads per kv head", max_t, "ragged" if ragged else "equal")
+    B, Hq, Hkv, D = 3, 16, 8, 128
+    S = 4096
+    lens = np.array([max_t, 700, 2500]) if ragged else np.full(B, max_t)
+    qkv, bias, kc, vc = _case(np.float16, B, Hq, Hkv, D, S, 1, seed=max_t, std=0.5)
+    d_qkv, d_bias = torch.from_numpy(qkv).to(dev), torch.from_numpy(bias).to(dev)
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    t_dev = torch.from_numpy(lens.astype(np.int32)).to(dev) if ragged else None
+    r_kc, r_vc = kc.copy(), vc.copy()
+    want = ref.decode_attn(qkv, bias, r_kc, r_vc, Hq, lens if ragged else max_t, D, 10000.0)
+    for flags in (capi.ATTN_ZEROED_WORKSPACE, 0, capi.ATTN_ZEROED_WORKSPACE):
+        d_kc, d_vc = torch.from_numpy(kc).to(dev), torch.from_numpy(vc).to(dev)
+        out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+        capi.decode_attn(d_qkv, d_bias, d_kc, d_vc, out, Hq, max_t, D, 10000.0, t_dev=t_dev, max_t=max_t, workspace=ws, flags=flags)
+        _assert_parity((out.cpu().numpy(), want, d_kc.cpu().numpy(), d_vc.cpu().numpy(), r_kc, r_vc), np.float16)
+        assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0
+
+
 def test_default_dispatch_at_medium_sizes(capi, ref, dev):
     """Sixteen seeded shapes of a few hundred units and a few thousand rows, equal and per-sequence lengths, with and
     without a zeroed workspace, no tuning keys: whatever schedule the launcher picks by itself (grid with or without a
