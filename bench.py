@@ -204,6 +204,8 @@ def bench_attention(capi, dev, steps, warmup, B, Hq, Hkv, D, S, t, nsets, t_dev=
     # (the headline is timed as EXACTLY `steps` launches in one block, after the clock ramp and `warmup` further
     # launches; the other shapes take the median of three such blocks)
     if not median:
+        # (also reported: the same block timed straight after the data was generated, inside the clock ramp)
+        bench_attention.unsettled_ms = time_steps(step, steps, warmup)
         settle(step, HEADLINE_SETTLE_S)
     ms = time_steps_median(step, steps, warmup) if median else time_steps(step, steps, warmup)
     bench_attention.last_step = step
@@ -680,6 +682,7 @@ def main():
         "value": round(ms * 1e3, 2), "unit": "us/step", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic", "settle_s_before_warmup": HEADLINE_SETTLE_S,
+        "us_without_settle": round(bench_attention.unsettled_ms * 1e3, 2),
         "config": {"workload": "BASELINE configs[1]: batch 16, 32 heads x 128, MHA, fp16 KV cache [1,16,32,4096,128], ctx %d, "
                                "RoPE base 10000; 4 cache sets rotated per step" % t,
                    "storage": "fp16", "arithmetic": "fp32"},
