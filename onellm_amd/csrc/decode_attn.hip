@@ -589,6 +589,16 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     }
     if (nsplit > cap) nsplit = cap;
     if (nsplit < 1) nsplit = 1;
+    // Equal lengths, a little fewer units than compute units: whole units on that many compute units, no split.  The
+    // active units already draw what the memory system gives (vector-ALU kernel: 43 GB/s each, 7 TB/s from 160 units),
+    // and a split would put every unit in two pieces.  Measured against two pieces per unit on equal shares: 192 / 224
+    // single-head units of 4096 rows 65.8 -> 60.3 / 75.5 -> 70.4 us, of 1024 rows 21.6 -> 19.9 / 23.1 -> 22.0; 160 units:
+    // 20.6 -> 18.5 (1024 rows), 54.9 -> 55.9 (4096).  A matrix-core workgroup draws ~30 GB/s alone, so there it takes
+    // more units or shorter rows: 224 units 149.2 -> 142.9 (8192 rows), 46.6 -> 42.3 (2048); 192 units 42.1 -> 39.5
+    // (2048) but 127.8 -> 136.8 (8192); 160 units 106 -> 132.
+    if (user_target <= 0 && !t_dev && !mfma64 && nsplit == 2 && base_wgs < 256
+        && (mfma_kernel ? (base_wgs >= 208 || (base_wgs >= 176 && max_t <= 2048)) : (base_wgs >= 176 || (base_wgs >= 160 && max_t <= 2048))))
+        nsplit = 1;
     const int forced = tune_get("attn_nsplit");
     if (forced > 0) nsplit = forced > max_splits(max_t) ? max_splits(max_t) : forced;
     int chunk = (max_t + nsplit - 1) / nsplit;
@@ -647,8 +657,11 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
                                     && (long)B * nunits <= kBalancedWorkgroups / 2 && items >= 64;
         a.unit_cost = user_cost >= 0 ? user_cost : (few_long_units ? 6 : 3);
         const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
-        long long nwg = user_wgs > 0 ? user_wgs
-                        : ((uneven_grid && bal != 1 && grid_wgs < 512) || few_long_units ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
+        // (an uneven grid of SHORT units keeps two shares per compute unit: with a share of a few hundred rows the second
+        // workgroup covers the first one's set-up and finish - 288 single-head units of 600 rows 23.1 -> 21.2 us, 36
+        // sequences x 8 kv heads of 600 rows 28.4 -> 26.2; from about 1200 rows on one share per unit is as fast or faster)
+        const bool one_share_per_unit = (uneven_grid && bal != 1 && grid_wgs < 512 && max_t >= 1024) || few_long_units;
+        long long nwg = user_wgs > 0 ? user_wgs : (one_share_per_unit ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
         // (the matrix-core kernel for D = 256 keeps one workgroup per compute unit resident: a second 256 would only
         // queue behind the first - 16 sequences of 512..4096 rows x 4 kv heads: 65.7 -> 47.1 us)
         if (user_wgs <= 0 && mfma_kernel && dtype == ONELLM_FP16 && D == 256 && nwg > kBalancedWorkgroups / 2) nwg = kBalancedWorkgroups / 2;
