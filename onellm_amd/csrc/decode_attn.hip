@@ -639,8 +639,15 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // stays on the grid schedule)
     const int cost_bound = tune_get("attn_balanced_cost") > 6 ? tune_get("attn_balanced_cost") : 6;
     const bool walk_fits = (wmax + (long long)B * nunits * cost_bound) * (kBalancedWorkgroups * 2) < (long long)kBalancedMaxItemsTimesWorkgroups;
+    // Per-sequence lengths on the vector-ALU kernel, a step of middling size (256-byte rows, 2048 rows or more at the
+    // longest, 8192..50000 items): one equal share per compute unit.  Measured against the default it replaces (the grid
+    // schedule below 16384 items, 512 shares above), single-head units, lengths uniform in [S/8, S]: 8 sequences x 32
+    // heads, S 2048 / 4096: 31.3 -> 28.7 / 53.2 -> 51.3 us; 12 sequences: 37.5 -> 35.7 / 64.7 -> 63.1 / (S 8192) 122.6 ->
+    // 119.9; 16 sequences: 46.6 -> 44.3 / 84.6 -> 81.1; 24 sequences, S 4096: 124.0 -> 121.6.  Not for shorter rows (8 x 32
+    // units of 128..1024 rows: 17.1 -> 19.4) nor beyond (16 sequences of 1024..8192 rows: 159.4 -> 161.2).
+    const bool valu_mid_ragged = t_dev && !mfma_kernel && lpr == 16 && max_t >= 2048 && wmax >= 8192 && wmax <= 50000;
     if (forced <= 0 && !padded && walk_fits
-        && (bal == 1 || (bal != 0 && (uneven_grid || balanced_by_default(t_dev != nullptr, mfma_kernel, G, wmax))))) {
+        && (bal == 1 || (bal != 0 && (uneven_grid || valu_mid_ragged || balanced_by_default(t_dev != nullptr, mfma_kernel, G, wmax))))) {
         a.item_rows = item_rows;
         // (what a change of unit costs a workgroup, in items: measured on the matrix-core kernel, where workgroups whose
         // equal-row shares held one / two / three units finished at 82 / 90 / 94 us of a 101 us step)
@@ -655,12 +662,12 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
         // D = 64, with half the bytes in flight per workgroup: 66 against 85), so they keep two per compute unit.
         const bool few_long_units = t_dev && mfma_kernel && dtype == ONELLM_FP16 && D == 128
                                     && (long)B * nunits <= kBalancedWorkgroups / 2 && items >= 64;
-        a.unit_cost = user_cost >= 0 ? user_cost : (few_long_units ? 6 : 3);
+        a.unit_cost = user_cost >= 0 ? user_cost : (few_long_units ? 6 : (valu_mid_ragged && bal != 1 ? 5 : 3));
         const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
         // (an uneven grid of SHORT units keeps two shares per compute unit: with a share of a few hundred rows the second
         // workgroup covers the first one's set-up and finish - 288 single-head units of 600 rows 23.1 -> 21.2 us, 36
         // sequences x 8 kv heads of 600 rows 28.4 -> 26.2; from about 1200 rows on one share per unit is as fast or faster)
-        const bool one_share_per_unit = (uneven_grid && bal != 1 && grid_wgs < 512 && max_t >= 1024) || few_long_units;
+        const bool one_share_per_unit = (uneven_grid && bal != 1 && grid_wgs < 512 && max_t >= 1024) || few_long_units || (valu_mid_ragged && bal != 1);
         long long nwg = user_wgs > 0 ? user_wgs : (one_share_per_unit ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
         // (the matrix-core kernel for D = 256 keeps one workgroup per compute unit resident: a second 256 would only
         // queue behind the first - 16 sequences of 512..4096 rows x 4 kv heads: 65.7 -> 47.1 us)

@@ -537,6 +537,34 @@ def test_two_heads_per_kv_head_either_side_of_the_kernel_switch(capi, ref, dev, 
         assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,tmax,ragged", [(8, 32, 32, 2048, True), (12, 32, 32, 2100, True), (6, 32, 32, 1024, False),
+                                                   (24, 32, 8, 2048, False), (28, 32, 8, 2500, False)])
+@pytest.mark.parametrize("zeroed", [False, True])
+def test_default_dispatch_choices_found_by_interleaved_timing(capi, ref, dev, B, Hq, Hkv, tmax, ragged, zeroed):
+    """Shapes at which the launcher's own choice changed after timings on buffers that are never freed: per-sequence
+    lengths on the vector-ALU kernel with 2048 rows or more and 8192..50000 items (one equal share per compute unit, a
+    unit change charged five items), and equal lengths with 160..255 units (whole units, no split; the matrix-core kernel
+    from 176 units at 2048 rows and from 208 beyond).  No tuning keys; against the oracle, twice on one workspace."""
+    announce("attn dispatch choices", B, Hq, Hkv, tmax, "ragged" if ragged else "equal", "zeroed" if zeroed else "merge launch")
+    D, S = 128, tmax
+    rng = np.random.default_rng(B * 1000 + tmax)
+    lens = rng.integers(tmax // 8, tmax + 1, size=B) if ragged else np.full(B, tmax)
+    lens[0] = tmax
+    qkv, bias, kc, vc = _case(np.float16, B, Hq, Hkv, D, S, 1, seed=B + tmax, std=0.5)
+    d_qkv, d_bias = torch.from_numpy(qkv).to(dev), torch.from_numpy(bias).to(dev)
+    d_kc, d_vc = torch.from_numpy(kc).to(dev), torch.from_numpy(vc).to(dev)
+    out = torch.zeros(B, Hq * D, dtype=torch.float16, device=dev)
+    ws = torch.zeros(capi.decode_attn_workspace_bytes(B, Hq, Hkv, D, S), dtype=torch.uint8, device=dev)
+    t_dev = torch.from_numpy(lens.astype(np.int32)).to(dev) if ragged else None
+    for _ in range(2):
+        capi.decode_attn(d_qkv, d_bias, d_kc, d_vc, out, Hq, tmax, D, 10000.0, t_dev=t_dev, max_t=tmax,
+                         flags=capi.ATTN_ZEROED_WORKSPACE if zeroed else 0, workspace=ws)
+    r_kc, r_vc = kc.copy(), vc.copy()
+    want = ref.decode_attn(qkv, bias, r_kc, r_vc, Hq, lens if ragged else tmax, D, 10000.0)
+    _assert_parity((out.cpu().numpy(), want, d_kc.cpu().numpy(), d_vc.cpu().numpy(), r_kc, r_vc), np.float16)
+    assert int(ws[:65536].view(torch.int32).abs().max().item()) == 0
+
+
 def test_default_dispatch_at_medium_sizes(capi, ref, dev):
     """Sixteen seeded shapes of a few hundred units and a few thousand rows, equal and per-sequence lengths, with and
     without a zeroed workspace, no tuning keys: whatever schedule the launcher picks by itself (grid with or without a
