@@ -32,7 +32,7 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
-template <int D, int GT, int NW, bool DOUBLE_BUFFER>
+template <int D, int GT, int NW>
 __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds, int& ev)
 {
     stamp_event(a, ev);
@@ -69,17 +69,46 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
     const T* kp = kc + (size_t)(wave * 16 + slot) * D + grp * VEC;
     const T* vp = vc + (size_t)(wave * 16 + 4 * grp) * D + vslot * VEC;
 
-    auto issue = [&](Vec16<T> (&kv)[NKJ], Vec16<T> (&vv)[CG * 4], int rbase) {
+    // One register buffer, K and V requested separately: the K registers are free once the batch's scores are computed
+    // and the V registers once its output products are, so the next batch's K rows are on their way during this batch's
+    // softmax and output products and its V rows during the next batch's scores.  The partial last batch takes the
+    // same road, its row indices held at the piece's last row and its scores masked.  Measured at D = 256 against
+    // requesting both after the whole batch was consumed: 32 q / 8 kv heads, batch 16 / 32, 4096 rows 90.5 -> 86.2 /
+    // 159.5 -> 155.8 us; lengths 512..4096, batch 32: 102.5 -> 98.0; 12 q / 4 kv heads, batch 16: 52.1 -> 47.7; batch 4,
+    // 8192 rows 54.1 -> 49.2; batch 64, 1024 rows 97.7 -> 90.1.
+    auto issue_k = [&](Vec16<T> (&kv)[NKJ], int rbase) {
 #pragma unroll
         for (int j = 0; j < NKJ; ++j) kv[j] = load16_stream(kp + (size_t)rbase * D + j * 32);
+    };
+    auto issue_v = [&](Vec16<T> (&vv)[CG * 4], int rbase) {
 #pragma unroll
         for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
             for (int e = 0; e < 4; ++e) vv[cg * 4 + e] = load16_stream(vp + (size_t)(rbase + e) * D + cg * 128);
     };
+    auto issue_k_clamped = [&](Vec16<T> (&kv)[NKJ], int rbase) {
+        const int krow = min(rbase + wave * 16 + slot, r1 - 1);
+#pragma unroll
+        for (int j = 0; j < NKJ; ++j) kv[j] = load16_stream(kc + (size_t)krow * D + grp * VEC + j * 32);
+    };
+    auto issue_v_clamped = [&](Vec16<T> (&vv)[CG * 4], int rbase) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int vrow = min(rbase + wave * 16 + 4 * grp + e, r1 - 1);
+#pragma unroll
+            for (int cg = 0; cg < CG; ++cg) vv[cg * 4 + e] = load16_stream(vc + (size_t)vrow * D + vslot * VEC + cg * 128);
+        }
+    };
     const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
-    Vec16<T> ka[NKJ], va[CG * 4], kb[DOUBLE_BUFFER ? NKJ : 1], vb[DOUBLE_BUFFER ? CG * 4 : 1];
-    if (nfull > 0) issue(ka, va, r0);
+    const bool partial = r1 > r0 && r0 + nfull * RPI < r1;
+    Vec16<T> ka[NKJ], va[CG * 4];
+    if (nfull > 0) {
+        issue_k(ka, r0);
+        issue_v(va, r0);
+    } else if (partial) {
+        issue_k_clamped(ka, r0);
+        issue_v_clamped(va, r0);
+    }
 
     stage_q_and_new_row<T, D, GT, NTHR>(a, fr, u, kc, vc, sq, sk, sv, snew);
 
@@ -108,7 +137,8 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
 #pragma unroll
     for (int c = 0; c < CG * VEC; ++c) o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto consume = [&](const Vec16<T> (&kv)[NKJ], const Vec16<T> (&vv)[CG * 4], int rbase, auto masked_tag) {
+    // scores of the batch at rbase (row 4*grp + r of the batch, head lane % GT); after it the K registers are free
+    auto scores = [&](const Vec16<T> (&kv)[NKJ], int rbase, float (&s)[4], auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -120,14 +150,15 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
             s0 = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qhi[jp * 2 + 1], s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qlo[jp * 2 + 1], s1, 0, 0, 0);
         }
-        float s[4];
-        float bm = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            s[r] = s0[r] + s1[r];               // score of row 4*grp + r of the batch, head lane % GT
+            s[r] = s0[r] + s1[r];
             if constexpr (MASKED) s[r] = (rbase + wave * 16 + 4 * grp + r < r1) ? s[r] : -INFINITY;
-            bm = fmaxf(bm, s[r]);
         }
+    };
+    // softmax update and output products of the batch; after it the V registers are free
+    auto accumulate = [&](const float (&s)[4], const Vec16<T> (&vv)[CG * 4]) {
+        float bm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
         if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
             bm = fmaxf(bm, __shfl_xor(bm, 16, kWave));
             bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
@@ -177,42 +208,33 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
     if (nfull == 0) look = first_look(a, u);
     if (r1 > r0) {
         int rbase = r0;
-        if constexpr (DOUBLE_BUFFER) {
-            for (int it = 0; it < nfull; it += 2) {
-                take_turns(a);
-                if (it + 2 >= nfull) look = first_look(a, u);
-                if (it + 1 < nfull) issue(kb, vb, rbase + RPI);
-                consume(ka, va, rbase, std::false_type{});
-                if (it + 1 < nfull) {
-                    if (it + 2 < nfull) issue(ka, va, rbase + 2 * RPI);
-                    consume(kb, vb, rbase + RPI, std::false_type{});
-                }
-                rbase += 2 * RPI;
-            }
-        } else {
-            // one register buffer: the other waves of the compute unit cover the load latency
-            for (int it = 0; it < nfull; ++it) {
-                take_turns(a);
-                if (it + 1 >= nfull) look = first_look(a, u);
-                consume(ka, va, rbase, std::false_type{});
-                rbase += RPI;
-                if (it + 1 < nfull) issue(ka, va, rbase);
-            }
+        float s[4];
+        int it = 0;
+        // while two more full batches lie ahead the loop holds nothing conditional (a load requested under a condition -
+        // the look below is one - makes the compiler wait for every load in flight, each time round)
+        for (; it + 2 < nfull; ++it) {
+            take_turns(a);
+            scores(ka, rbase, s, std::false_type{});
+            issue_k(ka, rbase + RPI);
+            accumulate(s, va);
+            issue_v(va, rbase + RPI);
+            rbase += RPI;
         }
-        rbase = r0 + nfull * RPI;
-        if (rbase < r1) {
-            // partial batch: rows past the end are read from the last valid row and masked
-            const int krow = min(rbase + wave * 16 + slot, r1 - 1);
-#pragma unroll
-            for (int j = 0; j < NKJ; ++j) ka[j] = load16_stream(kc + (size_t)krow * D + grp * VEC + j * 32);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int vrow = min(rbase + wave * 16 + 4 * grp + e, r1 - 1);
-#pragma unroll
-                for (int cg = 0; cg < CG; ++cg) va[cg * 4 + e] = load16_stream(vc + (size_t)vrow * D + vslot * VEC + cg * 128);
-            }
-            // a wave whose rows are all past the end must not touch its state (its scores are all -inf)
-            if (rbase + wave * 16 < r1) consume(ka, va, rbase, std::true_type{});
+        for (; it < nfull; ++it) {              // the last two full batches; the partial one is requested behind them
+            take_turns(a);
+            if (it + 2 == nfull || nfull == 1) look = first_look(a, u);
+            scores(ka, rbase, s, std::false_type{});
+            if (it + 1 < nfull) issue_k(ka, rbase + RPI);
+            else if (partial) issue_k_clamped(ka, rbase + RPI);
+            accumulate(s, va);
+            if (it + 1 < nfull) issue_v(va, rbase + RPI);
+            else if (partial) issue_v_clamped(va, rbase + RPI);
+            rbase += RPI;
+        }
+        // a wave whose rows of the partial batch are all past the end must not touch its state (its scores are all -inf)
+        if (partial && rbase + wave * 16 < r1) {
+            scores(ka, rbase, s, std::true_type{});
+            accumulate(s, va);
         }
     }
 
@@ -238,9 +260,9 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
     stamp_event(a, ev);
 }
 
-// ---- the unit of the grid schedule with two register buffers (D = 64, 128): one unit per workgroup.
+// ---- the unit with two register buffers (D = 64, 128), both schedules.
 //
-// Differences from gqa_mfma_unit above, each measured on MI355X:
+// Differences from gqa_mfma_unit above (one buffer: D = 256), each measured on MI355X:
 //   * a unit's last, partial batch of rows (read from the last valid row where it reaches past the end, and masked)
 //     goes through the same two buffers as the full ones instead of being asked for after the last full batch was
 //     consumed - a memory round trip with nothing else in flight at the end of every unit;
@@ -249,14 +271,13 @@ __device__ __forceinline__ void gqa_mfma_unit(const AttnArgs& a, const RopeFreqs
 //     the loads a product needs (with a conditional request in the loop it waits for all loads: both buffers).
 // 4 sequences x 8 kv heads of 8192 rows in eight pieces each 28.1 -> 26.8 us; 8 sequences of 256..2048 rows 16.4 ->
 // 15.4; 64 q / 8 kv heads x 16 sequences x 8192 rows 85.4 -> 83.7; 32 sequences x 8 kv heads x 8192 rows 153.6 -> 152.0.
-// The balanced schedule keeps gqa_mfma_unit: the same loop inside its walk over several units measured 0.5-2.5 us
-// slower there (config 3 ragged 93.3 -> 93.9, 96 sequences of 256..2048 rows 80.9 -> 83.3) - the schedule state of two
-// units no longer fits the scalar registers.  Also built and measured there, and not kept: asking for the next piece's
-// rows before the current piece is finished, at the end of its streaming loop or right behind the counter add of a
-// piece that is handed over.  A piece's finish waits for its stores to be acknowledged with `s_waitcnt vmcnt(0)`,
-// which also waits for every load in flight (64 KiB per workgroup: the finish went from 2.5 to 4.7-5.8 us and ate what
-// the set-up saved), and the registers that stay live across the finish cost the second wave per SIMD (96 sequences
-// of 256..2048 rows: 80 -> 105 us).
+// Also built and measured, and not kept: a look-ahead at the next unit inside the balanced walk (the schedule state
+// of two units no longer fits the scalar registers: config 3 ragged 93.3 -> 93.9, 96 sequences of 256..2048 rows
+// 80.9 -> 83.3), and asking for the next piece's rows before the current piece is finished, at the end of its
+// streaming loop or right behind the counter add of a piece that is handed over.  A piece's finish waits for its
+// stores to be acknowledged with `s_waitcnt vmcnt(0)`, which also waits for every load in flight (64 KiB per
+// workgroup: the finish went from 2.5 to 4.7-5.8 us and ate what the set-up saved), and the registers that stay live
+// across the finish cost the second wave per SIMD (96 sequences of 256..2048 rows: 80 -> 105 us).
 template <int D>
 struct KvBatch {
     static constexpr int NKJ = D / 32;
@@ -529,7 +550,7 @@ void decode_attn_gqa_mfma_kernel(const AttnArgs a, const RopeFreqs fr)
     if constexpr (DOUBLE_BUFFER) {
         for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_grid_unit<D, GT, NW>(a, fr, u, lds, ev); });
     } else {
-        for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_unit<D, GT, NW, DOUBLE_BUFFER>(a, fr, u, lds, ev); });
+        for_each_unit<GT, BALANCED>(a, [&](const Unit& u) { gqa_mfma_unit<D, GT, NW>(a, fr, u, lds, ev); });
     }
     stamp_end(a);
 }
@@ -560,7 +581,11 @@ int launch_gqa_mfma(const AttnArgs& a, const RopeFreqs& fr, hipStream_t st)
 // 4*grp + {0..3} of head slot % GT, and score register r is the A operand of output product r
 // (k = grp <-> row 4*grp + r), against V loaded as rows 4*grp + {0..3}, four columns per lane.
 // 64 products of 32 cycles per 16 rows (16 KiB of K and V): about a third of what the memory stream
-// leaves per SIMD.  One register buffer (two would leave one wave per SIMD).
+// leaves per SIMD.  One register buffer (two would leave one wave per SIMD), K and V requested separately as in
+// gqa_mfma_unit.  Measured against requesting both after the whole batch was consumed: 64 q / 8 kv heads, batch 8,
+// 8192 rows 87.3 -> 85.0 us; D = 64, batch 16: 97.5 -> 81.9; batch 4: 51.1 -> 48.7; 32 sequences of 256..2048 rows
+// 64.3 -> 62.6; 128 q / 8 kv heads, batch 8, 4096 rows 56.1 -> 56.8.  (A first version with the look inside the
+// steady-state loop was 8-12 % slower than before: the conditional load made every wait a wait for all loads.)
 template <int D, int GT, int NW>
 __device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeFreqs& fr, const Unit& u, float* lds)
 {
@@ -594,17 +619,44 @@ __device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeF
     const T* kp = kc + (size_t)(wave * 16 + slot) * D + grp * VEC;
     const T* vp = vc + (size_t)(wave * 16 + 4 * grp) * D + slot * VEC;
 
-    auto issue = [&](Vec16<T> (&kv)[NKJ], Vec16<T> (&vv)[CG * 4], int rbase) {
+    // K and V of a batch are requested separately: the K registers are free once the batch's scores are computed and
+    // the V registers once its output products are, so the next batch's K rows are on their way during this batch's
+    // softmax and output products and its V rows during the next batch's scores - a pipeline in the one register
+    // buffer (two would leave one wave per SIMD).  The partial last batch takes the same road, with its row indices
+    // held at the piece's last row and its scores masked.
+    auto issue_k = [&](Vec16<T> (&kv)[NKJ], int rbase) {
 #pragma unroll
         for (int j = 0; j < NKJ; ++j) kv[j] = load16_stream(kp + (size_t)rbase * D + j * 16);
+    };
+    auto issue_v = [&](Vec16<T> (&vv)[CG * 4], int rbase) {
 #pragma unroll
         for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
             for (int e = 0; e < 4; ++e) vv[cg * 4 + e] = load16_stream(vp + (size_t)(rbase + e) * D + cg * 64);
     };
+    auto issue_k_clamped = [&](Vec16<T> (&kv)[NKJ], int rbase) {
+        const int krow = min(rbase + wave * 16 + slot, r1 - 1);
+#pragma unroll
+        for (int j = 0; j < NKJ; ++j) kv[j] = load16_stream(kc + (size_t)krow * D + grp * VEC + j * 16);
+    };
+    auto issue_v_clamped = [&](Vec16<T> (&vv)[CG * 4], int rbase) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int vrow = min(rbase + wave * 16 + 4 * grp + e, r1 - 1);
+#pragma unroll
+            for (int cg = 0; cg < CG; ++cg) vv[cg * 4 + e] = load16_stream(vc + (size_t)vrow * D + slot * VEC + cg * 64);
+        }
+    };
     const int nfull = r1 > r0 ? (r1 - r0) / RPI : 0;
+    const bool partial = r1 > r0 && r0 + nfull * RPI < r1;
     Vec16<T> ka[NKJ], va[CG * 4];
-    if (nfull > 0) issue(ka, va, r0);
+    if (nfull > 0) {
+        issue_k(ka, r0);
+        issue_v(va, r0);
+    } else if (partial) {
+        issue_k_clamped(ka, r0);
+        issue_v_clamped(va, r0);
+    }
 
     stage_q_and_new_row<T, D, GT, NTHR>(a, fr, u, kc, vc, sq, sk, sv, snew);
 
@@ -624,21 +676,23 @@ __device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeF
 #pragma unroll
     for (int c = 0; c < CG * VEC; ++c) o[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto consume = [&](const Vec16<T> (&kv)[NKJ], const Vec16<T> (&vv)[CG * 4], int rbase, auto masked_tag) {
+    // scores of the batch at rbase (row 4*grp + r of the batch, head lane % GT); after it the K registers are free
+    auto scores = [&](const Vec16<T> (&kv)[NKJ], int rbase, float (&s)[4], auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         f32x4 sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < NKJ; ++j)
 #pragma unroll
             for (int e = 0; e < VEC; ++e) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[j].raw[e], qb[j][e], sc, 0, 0, 0);
-        float s[4];
-        float bm = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            s[r] = sc[r];                       // score of row 4*grp + r of the batch, head lane % GT
+            s[r] = sc[r];
             if constexpr (MASKED) s[r] = (rbase + wave * 16 + 4 * grp + r < r1) ? s[r] : -INFINITY;
-            bm = fmaxf(bm, s[r]);
         }
+    };
+    // softmax update and output products of the batch; after it the V registers are free
+    auto accumulate = [&](const float (&s)[4], const Vec16<T> (&vv)[CG * 4]) {
+        float bm = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
         if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
             bm = fmaxf(bm, __shfl_xor(bm, 16, kWave));
             bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
@@ -673,27 +727,32 @@ __device__ __forceinline__ void gqa_mfma_f32_unit(const AttnArgs& a, const RopeF
     if (nfull == 0) look = first_look(a, u);
     if (r1 > r0) {
         int rbase = r0;
-        // one register buffer: the other waves of the compute unit cover the load latency
-        for (int it = 0; it < nfull; ++it) {
+        float s[4];
+        int it = 0;
+        // while two more full batches lie ahead the loop holds nothing conditional (a load requested under a condition -
+        // the look below is one - makes the compiler wait for every load in flight, each time round)
+        for (; it + 2 < nfull; ++it) {
             take_turns(a);
-            if (it + 1 >= nfull) look = first_look(a, u);
-            consume(ka, va, rbase, std::false_type{});
+            scores(ka, rbase, s, std::false_type{});
+            issue_k(ka, rbase + RPI);
+            accumulate(s, va);
+            issue_v(va, rbase + RPI);
             rbase += RPI;
-            if (it + 1 < nfull) issue(ka, va, rbase);
         }
-        rbase = r0 + nfull * RPI;
-        if (rbase < r1) {
-            // partial batch: rows past the end are read from the last valid row and masked
-            const int krow = min(rbase + wave * 16 + slot, r1 - 1);
-#pragma unroll
-            for (int j = 0; j < NKJ; ++j) ka[j] = load16_stream(kc + (size_t)krow * D + grp * VEC + j * 16);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int vrow = min(rbase + wave * 16 + 4 * grp + e, r1 - 1);
-#pragma unroll
-                for (int cg = 0; cg < CG; ++cg) va[cg * 4 + e] = load16_stream(vc + (size_t)vrow * D + slot * VEC + cg * 64);
-            }
-            if (rbase + wave * 16 < r1) consume(ka, va, rbase, std::true_type{});
+        for (; it < nfull; ++it) {              // the last two full batches; the partial one is requested behind them
+            take_turns(a);
+            if (it + 2 == nfull || nfull == 1) look = first_look(a, u);
+            scores(ka, rbase, s, std::false_type{});
+            if (it + 1 < nfull) issue_k(ka, rbase + RPI);
+            else if (partial) issue_k_clamped(ka, rbase + RPI);
+            accumulate(s, va);
+            if (it + 1 < nfull) issue_v(va, rbase + RPI);
+            else if (partial) issue_v_clamped(va, rbase + RPI);
+            rbase += RPI;
+        }
+        if (partial && rbase + wave * 16 < r1) {
+            scores(ka, rbase, s, std::true_type{});
+            accumulate(s, va);
         }
     }
 
