@@ -595,9 +595,12 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // single-head units of 4096 rows 65.8 -> 60.3 / 75.5 -> 70.4 us, of 1024 rows 21.6 -> 19.9 / 23.1 -> 22.0; 160 units:
     // 20.6 -> 18.5 (1024 rows), 54.9 -> 55.9 (4096).  A matrix-core workgroup draws ~30 GB/s alone, so there it takes
     // more units or shorter rows: 224 units 149.2 -> 142.9 (8192 rows), 46.6 -> 42.3 (2048); 192 units 42.1 -> 39.5
-    // (2048) but 127.8 -> 136.8 (8192); 160 units 106 -> 132.
+    // (2048) but 127.8 -> 136.8 (8192); 160 units 106 -> 132.  The vector-ALU kernel with several heads per tile is
+    // as heavy per row (fp32 caches, 32 q / 8 kv heads, 192 units of 4096 rows: 127.8 -> 142.4; 224 units 148.0 -> 146.0)
+    // and takes the matrix-core kernel's bounds.
+    const bool light_rows = !mfma_kernel && gt == 1;
     if (user_target <= 0 && !t_dev && !mfma64 && nsplit == 2 && base_wgs < 256
-        && (mfma_kernel ? (base_wgs >= 208 || (base_wgs >= 176 && max_t <= 2048)) : (base_wgs >= 176 || (base_wgs >= 160 && max_t <= 2048))))
+        && (light_rows ? (base_wgs >= 176 || (base_wgs >= 160 && max_t <= 2048)) : (base_wgs >= 208 || (base_wgs >= 176 && max_t <= 2048))))
         nsplit = 1;
     const int forced = tune_get("attn_nsplit");
     if (forced > 0) nsplit = forced > max_splits(max_t) ? max_splits(max_t) : forced;
