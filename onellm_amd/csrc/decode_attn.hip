@@ -465,7 +465,10 @@ bool balanced_by_default(bool ragged, bool mfma, int G, long long max_items)
     // where the dispatcher keeps four workgroups per compute unit busy with the grid schedule's chunks: a tie up to
     // ~16000 items, then 3-6 % - 16 sequences x 32 heads of 512..4096 rows 105 -> 100 us, 64 of 128..2048: 184 -> 174)
     if (!ragged) return false;
-    if (mfma || G == 2) return max_items >= kBalancedMinItems;
+    if (mfma) return max_items >= kBalancedMinItems;
+    // (two heads per tile on the vector-ALU kernel: 16 sequences x 8 kv heads of 256..2048 / 375..3000 rows, 4096 / 6016
+    // items, 21.3 / 25.4 us on equal shares against 17.9 / 22.1 on the grid; from 8192 items the shares are ahead)
+    if (G == 2) return max_items >= 8192;
     return max_items >= 16384;
 }
 
