@@ -459,13 +459,17 @@ int item_rows_for(bool fp16, int D, int G, int max_t)
 // the grid schedule with the fused finish is faster (8 sequences of 256..2048 rows: 24.9 against 17.6 us; 4 of
 // 512..4096: 25.2 / 19.6; even at 3500..4100 items; the balanced schedule is ahead from ~7000: 16 sequences of
 // 1024..8192 rows 56.7 / 67.6).
-bool balanced_by_default(bool ragged, bool mfma, int G, long long max_items)
+bool balanced_by_default(bool ragged, bool mfma, int G, long long max_items, long units, int max_t)
 {
     // (two heads per kv head on the vector-ALU kernel: 32 sequences of 1024..8192 rows 105.4 -> 98.1 us.  One head,
     // where the dispatcher keeps four workgroups per compute unit busy with the grid schedule's chunks: a tie up to
     // ~16000 items, then 3-6 % - 16 sequences x 32 heads of 512..4096 rows 105 -> 100 us, 64 of 128..2048: 184 -> 174)
     if (!ragged) return false;
-    if (mfma) return max_items >= kBalancedMinItems;
+    // (matrix-core kernels: fewer than 128 units of fewer than 4000 rows are cut into few chunks by the grid schedule
+    // and finish faster there - 12 sequences x 8 kv heads of 256..2048 / 375..3000 rows 18.9 / 21.9 us on equal shares,
+    // 16.7 / 19.3 on the grid - while 16 sequences of 256..2048 rows, 21.5 / 24.9, and 12 of 500..4000, 24.9 / 30.8, go
+    // the other way)
+    if (mfma) return max_items >= kBalancedMinItems && (units >= 128 || max_t >= 4000);
     // (two heads per tile on the vector-ALU kernel: 16 sequences x 8 kv heads of 256..2048 / 375..3000 rows, 4096 / 6016
     // items, 21.3 / 25.4 us on equal shares against 17.9 / 22.1 on the grid; from 8192 items the shares are ahead)
     if (G == 2) return max_items >= 8192;
@@ -653,7 +657,7 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // units of 128..1024 rows: 17.1 -> 19.4) nor beyond (16 sequences of 1024..8192 rows: 159.4 -> 161.2).
     const bool valu_mid_ragged = t_dev && !mfma_kernel && lpr == 16 && max_t >= 2048 && wmax >= 8192 && wmax <= 50000;
     if (forced <= 0 && !padded && walk_fits
-        && (bal == 1 || (bal != 0 && (uneven_grid || valu_mid_ragged || balanced_by_default(t_dev != nullptr, mfma_kernel, G, wmax))))) {
+        && (bal == 1 || (bal != 0 && (uneven_grid || valu_mid_ragged || balanced_by_default(t_dev != nullptr, mfma_kernel, G, wmax, (long)B * nunits, max_t))))) {
         a.item_rows = item_rows;
         // (what a change of unit costs a workgroup, in items: measured on the matrix-core kernel, where workgroups whose
         // equal-row shares held one / two / three units finished at 82 / 90 / 94 us of a 101 us step)
@@ -666,8 +670,11 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
         // workgroup per compute unit (config 3: 96.9 -> 94.3 us; 64 q / 8 kv heads, batch 16: 66.5 -> 64.3; lengths
         // 7000..8192: 159 -> 155).  Many short units go the other way (96 sequences of 256..2048 rows: 79 against 86 us;
         // D = 64, with half the bytes in flight per workgroup: 66 against 85), so they keep two per compute unit.
+        // (with half as many units as compute units or fewer it holds for shorter rows too: 16 sequences x 8 kv heads of
+        // 256..2048 / 500..4000 rows 23.9 -> 21.5 / 32.0 -> 29.6 us, 12 sequences of 500..4000 rows 27.2 -> 24.9)
         const bool few_long_units = t_dev && mfma_kernel && dtype == ONELLM_FP16 && D == 128
-                                    && (long)B * nunits <= kBalancedWorkgroups / 2 && items >= 64;
+                                    && ((long)B * nunits <= kBalancedWorkgroups / 4
+                                        || ((long)B * nunits <= kBalancedWorkgroups / 2 && items >= 64));
         a.unit_cost = user_cost >= 0 ? user_cost : (few_long_units ? 6 : (valu_mid_ragged && bal != 1 ? 5 : 3));
         const long long wmax_cost = wmax + (long long)B * nunits * a.unit_cost;
         // (an uneven grid of SHORT units keeps two shares per compute unit: with a share of a few hundred rows the second
