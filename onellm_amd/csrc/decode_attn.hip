@@ -643,8 +643,16 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     const long grid_wgs = base_wgs * nsplit;
     // (the matrix-core kernels hold two workgroups per unit at most, so any grid that is not a whole number of such
     // rounds ends with part of the chip idle: 576 units 227 -> 190 us, 640 units 265 -> 212, 768 units 284 -> 249)
+    // (the vector-ALU kernel keeps four workgroups per unit resident, so a grid a little above a whole number of
+    // workgroups per compute unit runs them all at once and ends with the few units that hold one more, alone, at a
+    // fraction of the bandwidth: 544 / 576 / 800 / 832 single-head units of 4096 rows 192.9 / 195.2 / 269.6 / 271.4 us
+    // against 178.4 / 182.8 / 250.0 / 260.0 on 512 equal shares; of 1024 rows 51.9 / 52.7 / 71.1 / 71.8 against 49.6 /
+    // 52.3 / 70.4 / 70.1; with 96 units or more over the multiple the grid is as fast - 608, 640 units - or faster)
+    const bool zeroed_ws = (flags & ONELLM_ATTN_ZEROED_WORKSPACE) && tune_get("attn_fused_finish") != 0;
+    const bool valu_tail = grid_wgs > 512 && grid_wgs < 2048 && grid_wgs % 256 != 0 && grid_wgs % 256 <= 80
+                           && (max_t >= 2048 || (zeroed_ws && max_t >= 1024));
     const bool uneven_grid = !t_dev && wmax >= 2048 && grid_wgs > 256
-                             && (mfma_kernel ? (grid_wgs % 512 != 0 && grid_wgs < 4096) : grid_wgs < 384);
+                             && (mfma_kernel ? (grid_wgs % 512 != 0 && grid_wgs < 4096) : (grid_wgs < 384 || valu_tail));
     // (the walk counts items in 32 bits: a step of more items than that allows - hundreds of millions of rows -
     // stays on the grid schedule)
     const int cost_bound = tune_get("attn_balanced_cost") > 6 ? tune_get("attn_balanced_cost") : 6;

@@ -538,13 +538,18 @@ def test_two_heads_per_kv_head_either_side_of_the_kernel_switch(capi, ref, dev, 
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,tmax,ragged", [(8, 32, 32, 2048, True), (12, 32, 32, 2100, True), (6, 32, 32, 1024, False),
-                                                   (24, 32, 8, 2048, False), (28, 32, 8, 2500, False)])
+                                                   (24, 32, 8, 2048, False), (28, 32, 8, 2500, False), (17, 32, 32, 1100, False),
+                                                   (18, 32, 32, 2050, False), (16, 32, 8, 2048, True), (12, 32, 8, 3000, True),
+                                                   (16, 16, 8, 2048, True)])
 @pytest.mark.parametrize("zeroed", [False, True])
 def test_default_dispatch_choices_found_by_interleaved_timing(capi, ref, dev, B, Hq, Hkv, tmax, ragged, zeroed):
     """Shapes at which the launcher's own choice changed after timings on buffers that are never freed: per-sequence
     lengths on the vector-ALU kernel with 2048 rows or more and 8192..50000 items (one equal share per compute unit, a
     unit change charged five items), and equal lengths with 160..255 units (whole units, no split; the matrix-core kernel
-    from 176 units at 2048 rows and from 208 beyond).  No tuning keys; against the oracle, twice on one workspace."""
+    from 176 units at 2048 rows and from 208 beyond); 544 and 576 single-head units (a few more than two per compute unit:
+    512 equal shares); per-sequence lengths on the matrix-core kernel with 128 and with 96 units (one share per compute
+    unit / the grid schedule) and two-head vector-ALU tiles below 8192 items (the grid schedule).  No tuning keys; against
+    the oracle, twice on one workspace."""
     announce("attn dispatch choices", B, Hq, Hkv, tmax, "ragged" if ragged else "equal", "zeroed" if zeroed else "merge launch")
     D, S = 128, tmax
     rng = np.random.default_rng(B * 1000 + tmax)
