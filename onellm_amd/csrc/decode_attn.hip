@@ -657,13 +657,19 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
     // stays on the grid schedule)
     const int cost_bound = tune_get("attn_balanced_cost") > 6 ? tune_get("attn_balanced_cost") : 6;
     const bool walk_fits = (wmax + (long long)B * nunits * cost_bound) * (kBalancedWorkgroups * 2) < (long long)kBalancedMaxItemsTimesWorkgroups;
-    // Per-sequence lengths on the vector-ALU kernel, a step of middling size (256-byte rows, 2048 rows or more at the
-    // longest, 8192..50000 items): one equal share per compute unit.  Measured against the default it replaces (the grid
+    // Per-sequence lengths on the vector-ALU kernel, a step of middling size (2048 rows or more at the longest, 128..800
+    // MiB of K rows): one equal share per compute unit.  Measured against the default it replaces (the grid
     // schedule below 16384 items, 512 shares above), single-head units, lengths uniform in [S/8, S]: 8 sequences x 32
     // heads, S 2048 / 4096: 31.3 -> 28.7 / 53.2 -> 51.3 us; 12 sequences: 37.5 -> 35.7 / 64.7 -> 63.1 / (S 8192) 122.6 ->
     // 119.9; 16 sequences: 46.6 -> 44.3 / 84.6 -> 81.1; 24 sequences, S 4096: 124.0 -> 121.6.  Not for shorter rows (8 x 32
     // units of 128..1024 rows: 17.1 -> 19.4) nor beyond (16 sequences of 1024..8192 rows: 159.4 -> 161.2).
-    const bool valu_mid_ragged = t_dev && !mfma_kernel && lpr == 16 && max_t >= 2048 && wmax >= 8192 && wmax <= 50000;
+    // The bounds are in bytes of K rows if every sequence had the longest length (8192..50000 items of 64 rows of 256 bytes),
+    // which carries over to the other row sizes: fp32 caches, head size 128 (512-byte rows), 4 / 8 / 16 sequences x 32 heads
+    // of 512..4096 / 256..2048 rows 41.4 -> 38.5 / 51.6 -> 49.8 / 84.4 -> 81.4 us, 32 q / 8 kv heads x 16 / 32 sequences of
+    // 512..4096 rows 53.2 -> 48.7 / 100.4 -> 94.3; fp16, head size 64, 8 sequences x 32 heads of 512..4096 rows 33.7 -> 28.7;
+    // head size 256, 16 sequences x 16 heads of 256..2048 rows 48.1 -> 43.3.
+    const long long wbytes = wmax * item_rows * row_bytes;
+    const bool valu_mid_ragged = t_dev && !mfma_kernel && max_t >= 2048 && wbytes >= (128ll << 20) && wbytes <= (800ll << 20);
     if (forced <= 0 && !padded && walk_fits
         && (bal == 1 || (bal != 0 && (uneven_grid || valu_mid_ragged || balanced_by_default(t_dev != nullptr, mfma_kernel, G, wmax, (long)B * nunits, max_t))))) {
         a.item_rows = item_rows;
