@@ -694,7 +694,13 @@ extern "C" int onellm_decode_attn(int dtype, const void* qkv, const void* qkv_bi
         // (an uneven grid of SHORT units keeps two shares per compute unit: with a share of a few hundred rows the second
         // workgroup covers the first one's set-up and finish - 288 single-head units of 600 rows 23.1 -> 21.2 us, 36
         // sequences x 8 kv heads of 600 rows 28.4 -> 26.2; from about 1200 rows on one share per unit is as fast or faster)
-        const bool one_share_per_unit = (uneven_grid && bal != 1 && grid_wgs < 512 && max_t >= 1024) || few_long_units || (valu_mid_ragged && bal != 1);
+        // (fp32 caches on the matrix-core kernel, head size 128: its one register buffer is a pipeline of its own since K
+        // and V rows are requested separately, and one share per compute unit is ahead - 64 q / 8 kv heads, 8 / 16 / 32
+        // sequences of 1024..8192 / 512..4096 rows: 57.7 -> 56.3 / 92.0 -> 88.6 / 104.2 -> 98.9 us; not for rows shorter than
+        // 2048: 96 sequences of 128..1024 rows 93.1 -> 96.6)
+        const bool fp32_mfma_shares = t_dev && mfma_kernel && dtype == ONELLM_FP32 && D == 128 && max_t >= 2048 && bal != 1;
+        const bool one_share_per_unit = (uneven_grid && bal != 1 && grid_wgs < 512 && max_t >= 1024) || few_long_units
+                                        || (valu_mid_ragged && bal != 1) || fp32_mfma_shares;
         long long nwg = user_wgs > 0 ? user_wgs : (one_share_per_unit ? kBalancedWorkgroups / 2 : kBalancedWorkgroups);
         // (the matrix-core kernel for D = 256 keeps one workgroup per compute unit resident: a second 256 would only
         // queue behind the first - 16 sequences of 512..4096 rows x 4 kv heads: 65.7 -> 47.1 us)
