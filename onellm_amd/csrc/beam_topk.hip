@@ -572,13 +572,13 @@ int launch_topk(const float* logits, int B, int beam, int V, int K, int nblk, fl
         }
         two = cs != hipStreamCaptureStatusNone;
     }
-    // Eight waves per workgroup for long rows (four chunks or more per wave) while the launch leaves room for them (up
-    // to two workgroups per compute unit): measured on MI355X, graph replay, batch 8 x beam 4, K = 4: V = 128256
-    // 14.1 -> 13.5 us; V = 32000 7.6 -> 8.2 us (a wave's fixed work - floor, marks, ranking - does not shrink with its
-    // share of the row, and the workgroup merges eight lists instead of four), so short rows keep four.  Tuning key
-    // topk_waves = 4 / 8 forces either.
+    // Eight waves per workgroup (512 threads: two dependent chains per SIMD, half the values per wave) pay only where a
+    // wave's per-value work is heavy - the per-lane lists of K > 4 - and its row slice long: graph replay, batch 8 x beam
+    // 4, V = 128256: K = 8 26.1 -> 24.5 us (K = 5: 25.0 -> 23.4; V = 65536: 19.6 -> 20.3; batch 16: 29.5 -> 30.0), but K = 4
+    // 14.06 -> 14.01, V = 65536 9.68 -> 10.07 (batch 16: 10.66 -> 11.77), V = 32000 7.73 -> 8.00 - a wave's fixed work (floor, marks, ranking) does not shrink with its share of the row, and
+    // the workgroup merges eight lists instead of four.  Tuning key topk_waves = 4 / 8 forces either.
     const int want_waves = tune_get("topk_waves");
-    const bool eight = want_waves == 8 || (want_waves != 4 && (long)B * beam * nblk <= 512 && V >= nblk * 8 * 256 * 4);
+    const bool eight = want_waves == 8 || (want_waves != 4 && KP > 4 && (long)B * beam * nblk <= 256 && V >= nblk * 8 * 256 * 6);
     int set = -1;
     g_last_path = ONELLM_TOPK_PATH_TWO_LAUNCHES;
     if (B <= kArrivalEntries && !two) {
